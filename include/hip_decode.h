@@ -1,0 +1,156 @@
+/*
+ * hip_decode.h -- C ABI of the MI355X (gfx950) decode backend for rustane.
+ *
+ * This is the boundary a `hip-decode` FFI crate binds: one entry point per public item of the
+ * reference's `metal_decode::Model` (crates/metal-decode/src/lib.rs), plus the few additions a
+ * backend without an Apple Neural Engine needs (prompt prefill, full logits, multi-token runs).
+ * Plain pointers and sizes only; every call returns a status code and never aborts the process
+ * (the reference panics where this returns HIPDEC_ERR_*).
+ *
+ * Threading: one model owns one HIP stream.  Calls on one model are synchronous and not
+ * re-entrant; distinct models may be used from distinct threads.
+ */
+#ifndef HIP_DECODE_H
+#define HIP_DECODE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Constants that are part of the interface (crates/metal-decode/src/lib.rs:14-15, :156, :201). */
+#define HIPDEC_MAX_GPU_TOPK 32u   /* MAX_GPU_TOPK, lib.rs:15 */
+#define HIPDEC_HEAD_BLOCK 256u    /* vocab rows per head block, lib.rs:156 (argmax_threads) */
+#define HIPDEC_RMS_EPS 1e-5f      /* RMS_EPS, lib.rs:14 */
+
+typedef enum {
+    HIPDEC_OK = 0,
+    HIPDEC_ERR_ARG = 1,      /* bad argument: null pointer, short buffer, token >= vocab, k out of range */
+    HIPDEC_ERR_FULL = 2,     /* len >= cfg.seq: the KV window is full (lib.rs:242-245 panics here) */
+    HIPDEC_ERR_HIP = 3,      /* a HIP runtime call failed; see hipdec_last_error */
+    HIPDEC_ERR_UNSUPPORTED = 4 /* shape or option this build has no kernel for */
+} hipdec_status;
+
+typedef enum {
+    HIPDEC_W_F32 = 0,        /* weights streamed as fp32 (the reference's precision) */
+    HIPDEC_W_BF16 = 1,       /* round-to-nearest-even bf16 */
+    HIPDEC_W_FP8_E4M3 = 2,   /* OCP e4m3fn, per-output-channel fp32 scale amax/448; embed stays bf16 */
+    HIPDEC_W_INT4_G128 = 3   /* symmetric 4-bit, groups of 128 along the reduction axis, bf16 scale
+                                amax/7; embed stays bf16 */
+} hipdec_weight_dtype;
+
+typedef enum {
+    HIPDEC_KV_F32 = 0,
+    HIPDEC_KV_BF16 = 1
+} hipdec_kv_dtype;
+
+/* metal_decode::Config, lib.rs:22-35 (same fields, same meaning). */
+typedef struct {
+    uint32_t dim, hidden, heads, kv_heads, hd, seq, nlayers, vocab, q_dim, kv_dim, gqa_ratio;
+} hipdec_config;
+
+/* metal_decode::LayerInit, lib.rs:37-47.  Row-major fp32, borrowed for the call only:
+ * wq[dim*q_dim], wk/wv[dim*kv_dim], wo[q_dim*dim], w1/w3[dim*hidden] with row = input channel;
+ * w2[dim*hidden] with row = output channel; gamma1/gamma2[dim]. */
+typedef struct {
+    const float *wq, *wk, *wv, *wo, *w1, *w3, *w2, *gamma1, *gamma2;
+} hipdec_layer_f32;
+
+/* metal_decode::FinalHeadInit, lib.rs:49-52: gamma_final[dim], embed[vocab*dim] (tied LM head). */
+typedef struct {
+    const float *gamma_final, *embed;
+} hipdec_head_f32;
+
+typedef struct {
+    uint32_t weight_dtype;   /* hipdec_weight_dtype */
+    uint32_t kv_dtype;       /* hipdec_kv_dtype */
+    int32_t device;          /* HIP device ordinal */
+    uint32_t ffn_activation; /* 0 = SwiGLU, 1 = leaky_relu(x, 0.5)^2  (engine/src/model.rs:3-7) */
+    uint32_t flags;          /* HIPDEC_FLAG_* */
+    uint32_t max_rows;       /* rows of the batched decode entry points (0 or 1 = single row) */
+} hipdec_options;
+
+#define HIPDEC_FLAG_NO_GRAPH 1u   /* launch kernels eagerly instead of replaying a captured hipGraph */
+
+typedef struct hipdec_model hipdec_model;
+
+/* Model::new, lib.rs:147-207.  Copies (and converts) the weights to device memory; the caller
+ * keeps ownership of every pointer.  n_layers must equal cfg->nlayers (lib.rs:186-188). */
+int hipdec_create(const hipdec_config *cfg, const hipdec_layer_f32 *layers, size_t n_layers,
+                  const hipdec_head_f32 *head, const hipdec_options *opts, hipdec_model **out);
+void hipdec_destroy(hipdec_model *m);
+
+/* Text of the last error on this model (or of the last failed hipdec_create when m is NULL). */
+const char *hipdec_last_error(const hipdec_model *m);
+
+/* Model::len / Model::set_len, lib.rs:209-215 (set_len clamps to cfg.seq). */
+size_t hipdec_len(const hipdec_model *m);
+int hipdec_set_len(hipdec_model *m, size_t len);
+
+/* Model::seed_layer_cache_from_channel_first, lib.rs:217-237:
+ * cache[pos*kv_dim + d] = k_rope_cf[d*seq + pos] for pos < live_len, the rest zero. */
+int hipdec_seed_layer_cache_from_channel_first(hipdec_model *m, size_t layer_idx, size_t live_len,
+                                               const float *k_rope_cf, const float *v_cf);
+
+/* Model::decode_token, lib.rs:239-269: x_in[dim] -> layers -> x_out[dim]; len += 1. */
+int hipdec_decode_token(hipdec_model *m, const float *x_in, float *x_out);
+/* Model::decode_token_from_id, lib.rs:271-304. */
+int hipdec_decode_token_from_id(hipdec_model *m, uint32_t token, float *x_out);
+/* Model::decode_token_argmax, lib.rs:306-338. */
+int hipdec_decode_token_argmax(hipdec_model *m, const float *x_in, uint32_t *out_token);
+/* Model::decode_token_argmax_from_id, lib.rs:340-375: final norm, tied LM head, argmax with ties
+ * to the lower index (lib.rs:1553, :1749); no softcap (monotone). */
+int hipdec_decode_token_argmax_from_id(hipdec_model *m, uint32_t token, uint32_t *out_token);
+/* Model::decode_token_topk_from_id, lib.rs:377-434: per 256-row block, the top_k largest raw
+ * logits (value desc, index asc), padded with (-inf, 0xffffffff).  Writes blocks*top_k pairs;
+ * cap = capacity of both output arrays in elements; *out_count = blocks*top_k. */
+int hipdec_decode_token_topk_from_id(hipdec_model *m, uint32_t token, uint32_t top_k,
+                                     float *out_vals, uint32_t *out_idxs, size_t cap,
+                                     size_t *out_count);
+/* Model::decode_token_block_stats_from_id, lib.rs:436-487: z = softcap(logit) * inv_temperature;
+ * per block max z and sum exp(z - max).  *out_count = blocks. */
+int hipdec_decode_token_block_stats_from_id(hipdec_model *m, uint32_t token, float inv_temperature,
+                                            float softcap, float *out_maxes, float *out_sums,
+                                            size_t cap, size_t *out_count);
+/* Model::materialize_current_logits_block, lib.rs:489-511: softcapped (not temperature-scaled)
+ * logits of one block of the step that ran last; does not advance len.
+ * *out_valid = min(256, vocab - 256*block_idx). */
+int hipdec_materialize_current_logits_block(hipdec_model *m, size_t block_idx, float softcap,
+                                            float *out_logits, size_t cap, size_t *out_valid);
+
+/* ---- additions with no counterpart in metal_decode::Model ---- */
+
+/* The work of DecodeContext::decode_next_logits (engine/src/decode.rs:91-127) done on the GPU:
+ * layers, final RMSNorm, tied LM head, optional softcap; out_logits[vocab]. */
+int hipdec_decode_logits_from_id(hipdec_model *m, uint32_t token, float softcap, float *out_logits);
+
+/* Prompt prefill (the reference prefills on the ANE, engine/src/inference.rs:136-144): runs
+ * positions len .. len+n-1 with causal attention, fills the KV cache, len += n.  last_logits
+ * (nullable, [vocab]) receives the softcapped logits of the last position. */
+int hipdec_prefill(hipdec_model *m, const uint32_t *ids, size_t n, float softcap, float *last_logits);
+
+/* Greedy run without a host round trip per token (the loop of engine/src/inference.rs:576-585):
+ * starting from `token`, performs n_steps argmax steps, each feeding its result to the next;
+ * out_tokens[n_steps].  Equivalent to n_steps calls of hipdec_decode_token_argmax_from_id. */
+int hipdec_decode_greedy_run(hipdec_model *m, uint32_t token, size_t n_steps, uint32_t *out_tokens);
+
+/* Per-step device time of the last hipdec_decode_greedy_run / hipdec_prefill, measured with HIP
+ * events on the model's stream: total milliseconds over that call. */
+int hipdec_last_device_ms(const hipdec_model *m, float *out_ms);
+
+/* Bytes of device memory the model streams per decoded token at the given live KV length
+ * (weights + scales + norms + one embedding row + KV read/write): the algorithmic traffic the
+ * bandwidth roofline is computed from. */
+int hipdec_bytes_per_token(const hipdec_model *m, size_t kv_len, uint64_t *out_bytes);
+
+/* Debug/verification: copy one stored weight matrix back as fp32 after de-quantisation, in
+ * out-major [rows][k] order.  which: 0 wqkv (rows q_dim+2*kv_dim, k dim), 1 wo (dim, q_dim),
+ * 2 w13 (2*hidden interleaved gate/up rows, dim), 3 w2 (dim, hidden), 4 embed (vocab, dim). */
+int hipdec_export_weight(hipdec_model *m, size_t layer_idx, uint32_t which, float *out, size_t cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIP_DECODE_H */

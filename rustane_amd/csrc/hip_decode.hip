@@ -1,0 +1,694 @@
+// C ABI of the gfx950 decode backend (see include/hip_decode.h): model construction, weight
+// conversion, hipGraph-captured decode steps and the head variants.
+#include "../../include/hip_decode.h"
+#include "hipdec_kernels.h"
+
+#include <math.h>
+#include <stdio.h>
+#include <string.h>
+#include <string>
+#include <vector>
+
+namespace {
+
+enum Variant { V_X = 0, V_ARGMAX, V_TOPK, V_STATS, V_LOGITS, V_COUNT };
+
+struct DevLayer {
+    void *wqkv = nullptr, *wo = nullptr, *w13 = nullptr, *w2 = nullptr;
+    void *s_qkv = nullptr, *s_wo = nullptr, *s_w13 = nullptr, *s_w2 = nullptr;
+    float *g1 = nullptr, *g2 = nullptr;
+    void *kc = nullptr, *vc = nullptr;
+};
+
+std::string g_create_error;
+
+}  // namespace
+
+struct hipdec_model {
+    hipdec_config cfg{};
+    hipdec_options opt{};
+    int wt = WT_F32, embed_wt = WT_F32, kvbf16 = 0;
+    int num_cu = 256;
+    hipStream_t stream = nullptr;
+    std::vector<DevLayer> layers;
+    void *embed = nullptr;
+    float *gfinal = nullptr;
+    float *x_a = nullptr, *x_b = nullptr, *q = nullptr, *att = nullptr, *gate = nullptr, *logits = nullptr,
+          *x_in = nullptr, *part = nullptr;
+    unsigned *counters = nullptr;
+    float *rope_cos = nullptr, *rope_sin = nullptr;
+    StepParams *d_sp = nullptr, *h_sp = nullptr;      // h_sp: pinned array [seq + 1]
+    float *d_topk_vals = nullptr, *d_bmax = nullptr, *d_bsum = nullptr, *d_out = nullptr;
+    uint32_t *d_topk_idxs = nullptr, *d_ring = nullptr;
+    float *h_out = nullptr;                           // pinned staging, max(vocab, 2*blocks*32) floats
+    size_t h_out_elems = 0;
+    size_t len = 0;
+    int NS = 1, blocks = 0;
+    float alpha = 1.0f;
+    hipGraphExec_t graphs[V_COUNT] = {};
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    float last_ms = 0.0f;
+    std::vector<void *> allocs;
+    std::string err;
+};
+
+namespace {
+
+#define HCHK(expr)                                                                           \
+    do {                                                                                     \
+        hipError_t e_ = (expr);                                                              \
+        if (e_ != hipSuccess) {                                                              \
+            char b_[512];                                                                    \
+            snprintf(b_, sizeof b_, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_),   \
+                     __FILE__, __LINE__);                                                    \
+            m->err = b_;                                                                     \
+            return HIPDEC_ERR_HIP;                                                           \
+        }                                                                                    \
+    } while (0)
+
+int fail(hipdec_model *m, int code, const char *msg) {
+    if (m) m->err = msg; else g_create_error = msg;
+    return code;
+}
+
+template <typename T> int dalloc(hipdec_model *m, T **p, size_t bytes) {
+    void *v = nullptr;
+    HCHK(hipMalloc(&v, bytes ? bytes : 16));
+    m->allocs.push_back(v);
+    *p = (T *)v;
+    return HIPDEC_OK;
+}
+
+size_t wt_row_bytes(int wt, size_t K) {
+    switch (wt) {
+        case WT_F32: return K * 4;
+        case WT_BF16: return K * 2;
+        case WT_FP8: return K;
+        default: return K / 2;
+    }
+}
+size_t wt_scale_bytes(int wt, size_t rows, size_t K) {
+    if (wt == WT_FP8) return rows * 4;
+    if (wt == WT_INT4) return rows * (K / 128) * 2;
+    return 0;
+}
+
+template <int WT> void launch_convert(hipStream_t s, const float *src, void *dst, void *scales, int rows, int K,
+                                      int mul, int off) {
+    hipLaunchKernelGGL(k_convert_rows<WT>, dim3(rows), dim3(256), 0, s, src, dst, scales, K, mul, off);
+}
+void convert_rows(int wt, hipStream_t s, const float *src, void *dst, void *scales, int rows, int K, int mul, int off) {
+    switch (wt) {
+        case WT_F32: launch_convert<WT_F32>(s, src, dst, scales, rows, K, mul, off); break;
+        case WT_BF16: launch_convert<WT_BF16>(s, src, dst, scales, rows, K, mul, off); break;
+        case WT_FP8: launch_convert<WT_FP8>(s, src, dst, scales, rows, K, mul, off); break;
+        default: launch_convert<WT_INT4>(s, src, dst, scales, rows, K, mul, off); break;
+    }
+}
+
+// host fp32 matrix -> device storage.  transpose: the host matrix is [K][O] (row = input
+// channel) and is turned into out-major [O][K] first.
+int load_matrix(hipdec_model *m, int wt, const float *host, int O, int K, bool transpose, float *stage_a,
+                float *stage_b, void *dst, void *scales, int mul, int off) {
+    HCHK(hipMemcpy(stage_a, host, (size_t)O * K * sizeof(float), hipMemcpyHostToDevice));
+    const float *src = stage_a;
+    if (transpose) {
+        dim3 grid((O + 31) / 32, (K + 31) / 32), block(32, 8);
+        hipLaunchKernelGGL(k_transpose_f32, grid, block, 0, m->stream, stage_a, stage_b, K, O);
+        src = stage_b;
+    }
+    convert_rows(wt, m->stream, src, dst, scales, O, K, mul, off);
+    HCHK(hipGetLastError());
+    HCHK(hipStreamSynchronize(m->stream));
+    return HIPDEC_OK;
+}
+
+// ---- one decode step, enqueued on the model's stream
+template <int WT, int EPI, int KVB> void launch_gemv_t(hipdec_model *m, const GemvArgs &a) {
+    int n_groups = (a.rows + 1) / 2;
+    size_t lds = (size_t)a.K * sizeof(float);
+    int per_cu = (int)(150 * 1024 / (lds + 64));
+    if (per_cu > 8) per_cu = 8;
+    if (per_cu < 1) per_cu = 1;
+    int grid = (n_groups + 3) / 4;
+    int cap = m->num_cu * per_cu;
+    if (grid > cap) grid = cap;
+    hipLaunchKernelGGL((k_gemv<WT, EPI, KVB>), dim3(grid), dim3(256), lds, m->stream, a);
+}
+template <int EPI> void launch_gemv(hipdec_model *m, int wt, const GemvArgs &a) {
+    const int kvb = (EPI == EPI_QKV) ? m->kvbf16 : 0;
+#define GEMV_CASE(W)                                                    \
+    if (kvb) launch_gemv_t<W, EPI, 1>(m, a); else launch_gemv_t<W, EPI, 0>(m, a);
+    switch (wt) {
+        case WT_F32: GEMV_CASE(WT_F32) break;
+        case WT_BF16: GEMV_CASE(WT_BF16) break;
+        case WT_FP8: GEMV_CASE(WT_FP8) break;
+        default: GEMV_CASE(WT_INT4) break;
+    }
+#undef GEMV_CASE
+}
+
+void launch_attn(hipdec_model *m, const DevLayer &L) {
+    const hipdec_config &c = m->cfg;
+    dim3 grid(c.heads, m->NS), block(256);
+    float scale = 1.0f / sqrtf((float)c.hd);
+    int gqa = c.gqa_ratio ? c.gqa_ratio : 1;
+#define ATT(KVB, HD)                                                                                          \
+    hipLaunchKernelGGL((k_attn_decode<KVB, HD>), grid, block, 0, m->stream, m->q, L.kc, L.vc, m->d_sp, m->part, \
+                       m->counters, m->att, (int)c.kv_dim, gqa, m->NS, scale)
+    if (m->kvbf16) { if (c.hd == 64) ATT(1, 64); else ATT(1, 128); }
+    else { if (c.hd == 64) ATT(0, 64); else ATT(0, 128); }
+#undef ATT
+}
+
+void enqueue_step(hipdec_model *m, int variant) {
+    const hipdec_config &c = m->cfg;
+    const int D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden, V = c.vocab;
+    if (m->embed_wt == WT_F32)
+        hipLaunchKernelGGL(k_embed<WT_F32>, dim3((D + 255) / 256), dim3(256), 0, m->stream, m->embed, m->x_in,
+                           m->d_sp, m->x_a, D);
+    else
+        hipLaunchKernelGGL(k_embed<WT_BF16>, dim3((D + 255) / 256), dim3(256), 0, m->stream, m->embed, m->x_in,
+                           m->d_sp, m->x_a, D);
+    for (uint32_t l = 0; l < c.nlayers; ++l) {
+        const DevLayer &L = m->layers[l];
+        GemvArgs a{};
+        a.sp = m->d_sp; a.alpha = m->alpha; a.q_dim = Q; a.kv_dim = KV; a.hd = c.hd; a.act = m->opt.ffn_activation;
+        a.rope_cos = m->rope_cos; a.rope_sin = m->rope_sin;
+        // q/k/v projections + RoPE + cache append
+        a.W = L.wqkv; a.scales = L.s_qkv; a.in = m->x_a; a.gamma = L.g1; a.out = m->q; a.kc = L.kc; a.vc = L.vc;
+        a.rows = Q + 2 * KV; a.K = D;
+        launch_gemv<EPI_QKV>(m, m->wt, a);
+        launch_attn(m, L);
+        // output projection + residual: x_b = x_a + alpha * (att . wo)
+        a.W = L.wo; a.scales = L.s_wo; a.in = m->att; a.gamma = nullptr; a.resid = m->x_a; a.out = m->x_b;
+        a.rows = D; a.K = Q;
+        launch_gemv<EPI_WO>(m, m->wt, a);
+        // gate/up + activation
+        a.W = L.w13; a.scales = L.s_w13; a.in = m->x_b; a.gamma = L.g2; a.resid = nullptr; a.out = m->gate;
+        a.rows = 2 * H; a.K = D;
+        launch_gemv<EPI_W13>(m, m->wt, a);
+        // down projection + residual: x_a = x_b + alpha * (gate . w2)
+        a.W = L.w2; a.scales = L.s_w2; a.in = m->gate; a.gamma = nullptr; a.resid = m->x_b; a.out = m->x_a;
+        a.rows = D; a.K = H;
+        launch_gemv<EPI_W2>(m, m->wt, a);
+    }
+    if (variant == V_X) {
+        hipLaunchKernelGGL(k_advance, dim3(1), dim3(1), 0, m->stream, m->d_sp);
+        return;
+    }
+    GemvArgs a{};
+    a.sp = m->d_sp; a.W = m->embed; a.in = m->x_a; a.gamma = m->gfinal; a.out = m->logits; a.rows = V; a.K = D;
+    launch_gemv<EPI_HEAD>(m, m->embed_wt, a);
+    switch (variant) {
+        case V_ARGMAX:
+            hipLaunchKernelGGL(k_head_argmax, dim3(1), dim3(1024), 0, m->stream, m->logits, V, m->d_sp, m->d_ring,
+                               (int)c.seq);
+            break;
+        case V_TOPK:
+            hipLaunchKernelGGL(k_head_topk, dim3(m->blocks), dim3(256), 0, m->stream, m->logits, V, m->d_sp,
+                               m->d_topk_vals, m->d_topk_idxs);
+            hipLaunchKernelGGL(k_advance, dim3(1), dim3(1), 0, m->stream, m->d_sp);
+            break;
+        case V_STATS:
+            hipLaunchKernelGGL(k_head_block_stats, dim3(m->blocks), dim3(256), 0, m->stream, m->logits, V, m->d_sp,
+                               m->d_bmax, m->d_bsum);
+            hipLaunchKernelGGL(k_advance, dim3(1), dim3(1), 0, m->stream, m->d_sp);
+            break;
+        default:
+            hipLaunchKernelGGL(k_advance, dim3(1), dim3(1), 0, m->stream, m->d_sp);
+            break;
+    }
+}
+
+int run_step(hipdec_model *m, int variant) {
+    if (m->opt.flags & HIPDEC_FLAG_NO_GRAPH) {
+        enqueue_step(m, variant);
+        HCHK(hipGetLastError());
+        return HIPDEC_OK;
+    }
+    if (!m->graphs[variant]) {
+        hipGraph_t g = nullptr;
+        HCHK(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
+        enqueue_step(m, variant);
+        hipError_t e = hipStreamEndCapture(m->stream, &g);
+        if (e != hipSuccess || !g) { m->err = std::string("graph capture failed: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+        HCHK(hipGraphInstantiate(&m->graphs[variant], g, nullptr, nullptr, 0));
+        HCHK(hipGraphDestroy(g));
+    }
+    HCHK(hipGraphLaunch(m->graphs[variant], m->stream));
+    return HIPDEC_OK;
+}
+
+// upload the step parameters from pinned slot `slot`, then run one step
+int step_with(hipdec_model *m, int variant, size_t slot, const StepParams &p) {
+    m->h_sp[slot] = p;
+    HCHK(hipMemcpyAsync(m->d_sp, &m->h_sp[slot], sizeof(StepParams), hipMemcpyHostToDevice, m->stream));
+    return run_step(m, variant);
+}
+
+int check_step(hipdec_model *m, uint32_t token, bool from_id) {
+    if (!m) return HIPDEC_ERR_ARG;
+    if (m->len >= m->cfg.seq) return fail(m, HIPDEC_ERR_FULL, "decode only supports lengths within cfg.seq");
+    if (from_id && token >= m->cfg.vocab) return fail(m, HIPDEC_ERR_ARG, "token id must fit vocab");
+    return HIPDEC_OK;
+}
+
+StepParams base_params(hipdec_model *m, uint32_t token) {
+    StepParams p{};
+    p.tok = (int)token; p.pos = (int)m->len; p.step = 0; p.top_k = 1; p.inv_t = 1.0f; p.softcap = 0.0f;
+    p.use_x_in = 0; p.block_idx = 0;
+    return p;
+}
+
+int softcap_out(hipdec_model *m, int start, int n, float cap, float *host_out) {
+    hipLaunchKernelGGL(k_softcap_copy, dim3((n + 255) / 256), dim3(256), 0, m->stream, m->logits, m->d_out, start, n, cap);
+    HCHK(hipGetLastError());
+    HCHK(hipMemcpyAsync(m->h_out, m->d_out, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, m->stream));
+    HCHK(hipStreamSynchronize(m->stream));
+    memcpy(host_out, m->h_out, (size_t)n * sizeof(float));
+    return HIPDEC_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *hipdec_last_error(const hipdec_model *m) { return m ? m->err.c_str() : g_create_error.c_str(); }
+
+void hipdec_destroy(hipdec_model *m) {
+    if (!m) return;
+    if (m->stream) (void)hipStreamSynchronize(m->stream);
+    for (auto &g : m->graphs) if (g) (void)hipGraphExecDestroy(g);
+    for (void *p : m->allocs) (void)hipFree(p);
+    if (m->h_sp) (void)hipHostFree(m->h_sp);
+    if (m->h_out) (void)hipHostFree(m->h_out);
+    if (m->ev0) (void)hipEventDestroy(m->ev0);
+    if (m->ev1) (void)hipEventDestroy(m->ev1);
+    if (m->stream) (void)hipStreamDestroy(m->stream);
+    delete m;
+}
+
+static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hipdec_head_f32 *head) {
+    const hipdec_config &c = m->cfg;
+    const size_t D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden, V = c.vocab, S = c.seq;
+    HCHK(hipSetDevice(m->opt.device));
+    hipDeviceProp_t prop;
+    HCHK(hipGetDeviceProperties(&prop, m->opt.device));
+    m->num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    HCHK(hipStreamCreate(&m->stream));
+    HCHK(hipEventCreate(&m->ev0));
+    HCHK(hipEventCreate(&m->ev1));
+
+    size_t max_elems = V * D;
+    if (D * H > max_elems) max_elems = D * H;
+    if (D * Q > max_elems) max_elems = D * Q;
+    float *stage_a = nullptr, *stage_b = nullptr;
+    HCHK(hipMalloc((void **)&stage_a, max_elems * sizeof(float)));
+    HCHK(hipMalloc((void **)&stage_b, max_elems * sizeof(float)));
+    int rc = HIPDEC_OK;
+    auto done = [&](int code) { (void)hipFree(stage_a); (void)hipFree(stage_b); return code; };
+
+    const int wt = m->wt;
+    const size_t kvsz = m->kvbf16 ? 2 : 4;
+    m->layers.resize(c.nlayers);
+    for (uint32_t l = 0; l < c.nlayers && rc == HIPDEC_OK; ++l) {
+        DevLayer &L = m->layers[l];
+        const hipdec_layer_f32 &src = layers[l];
+        if (!src.wq || !src.wk || !src.wv || !src.wo || !src.w1 || !src.w3 || !src.w2 || !src.gamma1 || !src.gamma2)
+            return done(fail(m, HIPDEC_ERR_ARG, "null layer weight pointer"));
+#define TRY(x) do { rc = (x); if (rc != HIPDEC_OK) return done(rc); } while (0)
+        TRY(dalloc(m, &L.wqkv, wt_row_bytes(wt, D) * (Q + 2 * KV)));
+        TRY(dalloc(m, &L.wo, wt_row_bytes(wt, Q) * D));
+        TRY(dalloc(m, &L.w13, wt_row_bytes(wt, D) * 2 * H));
+        TRY(dalloc(m, &L.w2, wt_row_bytes(wt, H) * D));
+        TRY(dalloc(m, &L.s_qkv, wt_scale_bytes(wt, Q + 2 * KV, D)));
+        TRY(dalloc(m, &L.s_wo, wt_scale_bytes(wt, D, Q)));
+        TRY(dalloc(m, &L.s_w13, wt_scale_bytes(wt, 2 * H, D)));
+        TRY(dalloc(m, &L.s_w2, wt_scale_bytes(wt, D, H)));
+        TRY(dalloc(m, &L.g1, D * 4));
+        TRY(dalloc(m, &L.g2, D * 4));
+        TRY(dalloc(m, &L.kc, S * KV * kvsz));
+        TRY(dalloc(m, &L.vc, S * KV * kvsz));
+        HCHK(hipMemsetAsync(L.kc, 0, S * KV * kvsz, m->stream));
+        HCHK(hipMemsetAsync(L.vc, 0, S * KV * kvsz, m->stream));
+        TRY(load_matrix(m, wt, src.wq, Q, D, true, stage_a, stage_b, L.wqkv, L.s_qkv, 1, 0));
+        TRY(load_matrix(m, wt, src.wk, KV, D, true, stage_a, stage_b, L.wqkv, L.s_qkv, 1, (int)Q));
+        TRY(load_matrix(m, wt, src.wv, KV, D, true, stage_a, stage_b, L.wqkv, L.s_qkv, 1, (int)(Q + KV)));
+        TRY(load_matrix(m, wt, src.wo, D, Q, true, stage_a, stage_b, L.wo, L.s_wo, 1, 0));
+        TRY(load_matrix(m, wt, src.w1, H, D, true, stage_a, stage_b, L.w13, L.s_w13, 2, 0));
+        TRY(load_matrix(m, wt, src.w3, H, D, true, stage_a, stage_b, L.w13, L.s_w13, 2, 1));
+        TRY(load_matrix(m, wt, src.w2, D, H, false, stage_a, stage_b, L.w2, L.s_w2, 1, 0));
+        HCHK(hipMemcpy(L.g1, src.gamma1, D * 4, hipMemcpyHostToDevice));
+        HCHK(hipMemcpy(L.g2, src.gamma2, D * 4, hipMemcpyHostToDevice));
+    }
+    TRY(dalloc(m, &m->embed, wt_row_bytes(m->embed_wt, D) * V));
+    TRY(load_matrix(m, m->embed_wt, head->embed, V, D, false, stage_a, stage_b, m->embed, nullptr, 1, 0));
+    TRY(dalloc(m, &m->gfinal, D * 4));
+    HCHK(hipMemcpy(m->gfinal, head->gamma_final, D * 4, hipMemcpyHostToDevice));
+
+    m->blocks = (int)((V + HIPDEC_HEAD_BLOCK - 1) / HIPDEC_HEAD_BLOCK);
+    int ns = (int)(256 / c.heads);
+    if (ns < 1) ns = 1;
+    if (ns > 32) ns = 32;
+    m->NS = ns;
+    TRY(dalloc(m, &m->x_a, D * 4));
+    TRY(dalloc(m, &m->x_b, D * 4));
+    TRY(dalloc(m, &m->x_in, D * 4));
+    TRY(dalloc(m, &m->q, Q * 4));
+    TRY(dalloc(m, &m->att, Q * 4));
+    TRY(dalloc(m, &m->gate, H * 4));
+    TRY(dalloc(m, &m->logits, V * 4));
+    TRY(dalloc(m, &m->d_out, (V > 256 ? V : 256) * 4));
+    TRY(dalloc(m, &m->part, (size_t)c.heads * ns * (c.hd + 2) * 4));
+    TRY(dalloc(m, &m->counters, (size_t)c.heads * 4));
+    HCHK(hipMemset(m->counters, 0, (size_t)c.heads * 4));
+    TRY(dalloc(m, &m->d_sp, sizeof(StepParams)));
+    HCHK(hipMemset(m->d_sp, 0, sizeof(StepParams)));
+    TRY(dalloc(m, &m->d_topk_vals, (size_t)m->blocks * HIPDEC_MAX_GPU_TOPK * 4));
+    TRY(dalloc(m, &m->d_topk_idxs, (size_t)m->blocks * HIPDEC_MAX_GPU_TOPK * 4));
+    TRY(dalloc(m, &m->d_bmax, (size_t)m->blocks * 4));
+    TRY(dalloc(m, &m->d_bsum, (size_t)m->blocks * 4));
+    TRY(dalloc(m, &m->d_ring, S * 4));
+#undef TRY
+    // RoPE table, theta = pos / 10000^(2i/hd) (engine/src/kernels/sdpa_fwd.rs:18-33, lib.rs:1401)
+    {
+        const size_t hp = c.hd / 2;
+        std::vector<float> ct(S * hp), st(S * hp);
+        for (size_t p = 0; p < S; ++p)
+            for (size_t i = 0; i < hp; ++i) {
+                float theta = (float)p / powf(10000.0f, 2.0f * (float)i / (float)c.hd);
+                ct[p * hp + i] = cosf(theta);
+                st[p * hp + i] = sinf(theta);
+            }
+        rc = dalloc(m, &m->rope_cos, S * hp * 4); if (rc) return done(rc);
+        rc = dalloc(m, &m->rope_sin, S * hp * 4); if (rc) return done(rc);
+        HCHK(hipMemcpy(m->rope_cos, ct.data(), S * hp * 4, hipMemcpyHostToDevice));
+        HCHK(hipMemcpy(m->rope_sin, st.data(), S * hp * 4, hipMemcpyHostToDevice));
+    }
+    HCHK(hipHostMalloc((void **)&m->h_sp, sizeof(StepParams) * (S + 1), hipHostMallocDefault));
+    m->h_out_elems = V > 2 * (size_t)m->blocks * HIPDEC_MAX_GPU_TOPK ? V : 2 * (size_t)m->blocks * HIPDEC_MAX_GPU_TOPK;
+    if (m->h_out_elems < S) m->h_out_elems = S;
+    if (m->h_out_elems < D) m->h_out_elems = D;
+    HCHK(hipHostMalloc((void **)&m->h_out, m->h_out_elems * 4, hipHostMallocDefault));
+    HCHK(hipStreamSynchronize(m->stream));
+    return done(HIPDEC_OK);
+}
+
+int hipdec_create(const hipdec_config *cfg, const hipdec_layer_f32 *layers, size_t n_layers,
+                  const hipdec_head_f32 *head, const hipdec_options *opts, hipdec_model **out) {
+    if (out) *out = nullptr;
+    if (!cfg || !layers || !head || !out) return fail(nullptr, HIPDEC_ERR_ARG, "null argument");
+    if (!head->embed || !head->gamma_final) return fail(nullptr, HIPDEC_ERR_ARG, "null head weight pointer");
+    if (n_layers != cfg->nlayers) return fail(nullptr, HIPDEC_ERR_ARG, "layer count does not match cfg.nlayers");
+    const hipdec_config &c = *cfg;
+    if (!c.dim || !c.hidden || !c.heads || !c.kv_heads || !c.hd || !c.seq || !c.nlayers || !c.vocab)
+        return fail(nullptr, HIPDEC_ERR_ARG, "zero-sized config field");
+    if (c.q_dim != c.heads * c.hd || c.kv_dim != c.kv_heads * c.hd || c.heads % c.kv_heads != 0 ||
+        (c.gqa_ratio ? c.gqa_ratio : 1) != c.heads / c.kv_heads)
+        return fail(nullptr, HIPDEC_ERR_ARG, "inconsistent head geometry");
+    hipdec_options o{};
+    if (opts) o = *opts;
+    if (o.weight_dtype > HIPDEC_W_INT4_G128 || o.kv_dtype > HIPDEC_KV_BF16 || o.ffn_activation > 1)
+        return fail(nullptr, HIPDEC_ERR_ARG, "unknown option value");
+    if (c.hd != 64 && c.hd != 128) return fail(nullptr, HIPDEC_ERR_UNSUPPORTED, "head dim must be 64 or 128");
+    uint32_t kmul = o.weight_dtype == HIPDEC_W_INT4_G128 ? 128 : (o.weight_dtype == HIPDEC_W_FP8_E4M3 ? 16 : 8);
+    if (c.dim % kmul || c.hidden % kmul || c.q_dim % kmul || c.kv_dim % 8)
+        return fail(nullptr, HIPDEC_ERR_UNSUPPORTED, "dim / hidden / q_dim must be multiples of the weight load width");
+    if ((size_t)(c.hidden > c.dim ? c.hidden : c.dim) * 4 > 150 * 1024)
+        return fail(nullptr, HIPDEC_ERR_UNSUPPORTED, "reduction axis does not fit LDS");
+    hipdec_model *m = new hipdec_model();
+    m->cfg = c;
+    m->opt = o;
+    m->wt = (int)o.weight_dtype;
+    m->embed_wt = o.weight_dtype == HIPDEC_W_F32 ? WT_F32 : WT_BF16;
+    m->kvbf16 = o.kv_dtype == HIPDEC_KV_BF16;
+    m->alpha = 1.0f / sqrtf(2.0f * (float)c.nlayers);   // lib.rs:201
+    int rc = create_impl(m, layers, head);
+    if (rc != HIPDEC_OK) {
+        g_create_error = m->err;
+        hipdec_destroy(m);
+        return rc;
+    }
+    *out = m;
+    return HIPDEC_OK;
+}
+
+size_t hipdec_len(const hipdec_model *m) { return m ? m->len : 0; }
+
+int hipdec_set_len(hipdec_model *m, size_t len) {
+    if (!m) return HIPDEC_ERR_ARG;
+    m->len = len < m->cfg.seq ? len : m->cfg.seq;
+    return HIPDEC_OK;
+}
+
+int hipdec_seed_layer_cache_from_channel_first(hipdec_model *m, size_t layer_idx, size_t live_len,
+                                               const float *k_rope_cf, const float *v_cf) {
+    if (!m || !k_rope_cf || !v_cf) return HIPDEC_ERR_ARG;
+    if (layer_idx >= m->cfg.nlayers) return fail(m, HIPDEC_ERR_ARG, "layer_idx out of range");
+    const int KV = m->cfg.kv_dim, S = m->cfg.seq;
+    if (live_len > (size_t)S) live_len = S;
+    float *stage = nullptr;
+    HCHK(hipMalloc((void **)&stage, (size_t)KV * S * 4));
+    dim3 grid((S + 31) / 32, (KV + 31) / 32), block(32, 8);
+    for (int which = 0; which < 2; ++which) {
+        hipError_t e = hipMemcpy(stage, which ? v_cf : k_rope_cf, (size_t)KV * S * 4, hipMemcpyHostToDevice);
+        if (e != hipSuccess) { (void)hipFree(stage); m->err = hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+        void *dst = which ? m->layers[layer_idx].vc : m->layers[layer_idx].kc;
+        if (m->kvbf16) hipLaunchKernelGGL(k_seed_cache<1>, grid, block, 0, m->stream, stage, dst, KV, S, (int)live_len);
+        else hipLaunchKernelGGL(k_seed_cache<0>, grid, block, 0, m->stream, stage, dst, KV, S, (int)live_len);
+        e = hipStreamSynchronize(m->stream);
+        if (e != hipSuccess) { (void)hipFree(stage); m->err = hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+    }
+    HCHK(hipFree(stage));
+    return HIPDEC_OK;
+}
+
+static int read_x(hipdec_model *m, float *x_out) {
+    HCHK(hipMemcpyAsync(m->h_out, m->x_a, (size_t)m->cfg.dim * 4, hipMemcpyDeviceToHost, m->stream));
+    HCHK(hipStreamSynchronize(m->stream));
+    memcpy(x_out, m->h_out, (size_t)m->cfg.dim * 4);
+    return HIPDEC_OK;
+}
+
+static int upload_x(hipdec_model *m, const float *x_in) {
+    memcpy(m->h_out, x_in, (size_t)m->cfg.dim * 4);
+    HCHK(hipMemcpyAsync(m->x_in, m->h_out, (size_t)m->cfg.dim * 4, hipMemcpyHostToDevice, m->stream));
+    return HIPDEC_OK;
+}
+
+int hipdec_decode_token(hipdec_model *m, const float *x_in, float *x_out) {
+    int rc = check_step(m, 0, false);
+    if (rc) return rc;
+    if (!x_in || !x_out) return fail(m, HIPDEC_ERR_ARG, "null buffer");
+    if ((rc = upload_x(m, x_in))) return rc;
+    StepParams p = base_params(m, 0);
+    p.use_x_in = 1;
+    if ((rc = step_with(m, V_X, 0, p))) return rc;
+    if ((rc = read_x(m, x_out))) return rc;
+    m->len += 1;
+    return HIPDEC_OK;
+}
+
+int hipdec_decode_token_from_id(hipdec_model *m, uint32_t token, float *x_out) {
+    int rc = check_step(m, token, true);
+    if (rc) return rc;
+    if (!x_out) return fail(m, HIPDEC_ERR_ARG, "null buffer");
+    if ((rc = step_with(m, V_X, 0, base_params(m, token)))) return rc;
+    if ((rc = read_x(m, x_out))) return rc;
+    m->len += 1;
+    return HIPDEC_OK;
+}
+
+static int finish_argmax(hipdec_model *m, uint32_t *out_token) {
+    HCHK(hipMemcpyAsync(m->h_out, m->d_ring, 4, hipMemcpyDeviceToHost, m->stream));
+    HCHK(hipStreamSynchronize(m->stream));
+    memcpy(out_token, m->h_out, 4);
+    m->len += 1;
+    return HIPDEC_OK;
+}
+
+int hipdec_decode_token_argmax(hipdec_model *m, const float *x_in, uint32_t *out_token) {
+    int rc = check_step(m, 0, false);
+    if (rc) return rc;
+    if (!x_in || !out_token) return fail(m, HIPDEC_ERR_ARG, "null buffer");
+    if ((rc = upload_x(m, x_in))) return rc;
+    StepParams p = base_params(m, 0);
+    p.use_x_in = 1;
+    if ((rc = step_with(m, V_ARGMAX, 0, p))) return rc;
+    return finish_argmax(m, out_token);
+}
+
+int hipdec_decode_token_argmax_from_id(hipdec_model *m, uint32_t token, uint32_t *out_token) {
+    int rc = check_step(m, token, true);
+    if (rc) return rc;
+    if (!out_token) return fail(m, HIPDEC_ERR_ARG, "null buffer");
+    if ((rc = step_with(m, V_ARGMAX, 0, base_params(m, token)))) return rc;
+    return finish_argmax(m, out_token);
+}
+
+int hipdec_decode_token_topk_from_id(hipdec_model *m, uint32_t token, uint32_t top_k, float *out_vals,
+                                     uint32_t *out_idxs, size_t cap, size_t *out_count) {
+    int rc = check_step(m, token, true);
+    if (rc) return rc;
+    if (top_k == 0) return fail(m, HIPDEC_ERR_ARG, "top_k must be positive");
+    if (top_k > HIPDEC_MAX_GPU_TOPK) return fail(m, HIPDEC_ERR_ARG, "top_k exceeds decode top-k capacity");
+    const size_t count = (size_t)m->blocks * top_k;
+    if (!out_vals || !out_idxs || cap < count) return fail(m, HIPDEC_ERR_ARG, "output buffers too small for top-k candidates");
+    StepParams p = base_params(m, token);
+    p.top_k = (int)top_k;
+    if ((rc = step_with(m, V_TOPK, 0, p))) return rc;
+    HCHK(hipMemcpyAsync(m->h_out, m->d_topk_vals, count * 4, hipMemcpyDeviceToHost, m->stream));
+    HCHK(hipMemcpyAsync(m->h_out + count, m->d_topk_idxs, count * 4, hipMemcpyDeviceToHost, m->stream));
+    HCHK(hipStreamSynchronize(m->stream));
+    memcpy(out_vals, m->h_out, count * 4);
+    memcpy(out_idxs, m->h_out + count, count * 4);
+    if (out_count) *out_count = count;
+    m->len += 1;
+    return HIPDEC_OK;
+}
+
+int hipdec_decode_token_block_stats_from_id(hipdec_model *m, uint32_t token, float inv_temperature, float softcap,
+                                            float *out_maxes, float *out_sums, size_t cap, size_t *out_count) {
+    int rc = check_step(m, token, true);
+    if (rc) return rc;
+    const size_t B = (size_t)m->blocks;
+    if (!out_maxes || !out_sums || cap < B) return fail(m, HIPDEC_ERR_ARG, "block stats buffers too small");
+    StepParams p = base_params(m, token);
+    p.inv_t = inv_temperature;
+    p.softcap = softcap;
+    if ((rc = step_with(m, V_STATS, 0, p))) return rc;
+    HCHK(hipMemcpyAsync(m->h_out, m->d_bmax, B * 4, hipMemcpyDeviceToHost, m->stream));
+    HCHK(hipMemcpyAsync(m->h_out + B, m->d_bsum, B * 4, hipMemcpyDeviceToHost, m->stream));
+    HCHK(hipStreamSynchronize(m->stream));
+    memcpy(out_maxes, m->h_out, B * 4);
+    memcpy(out_sums, m->h_out + B, B * 4);
+    if (out_count) *out_count = B;
+    m->len += 1;
+    return HIPDEC_OK;
+}
+
+int hipdec_materialize_current_logits_block(hipdec_model *m, size_t block_idx, float softcap, float *out_logits,
+                                            size_t cap, size_t *out_valid) {
+    if (!m) return HIPDEC_ERR_ARG;
+    if (block_idx >= (size_t)m->blocks) return fail(m, HIPDEC_ERR_ARG, "block_idx out of range");
+    size_t start = block_idx * HIPDEC_HEAD_BLOCK;
+    size_t valid = m->cfg.vocab - start;
+    if (valid > HIPDEC_HEAD_BLOCK) valid = HIPDEC_HEAD_BLOCK;
+    if (!out_logits || cap < valid) return fail(m, HIPDEC_ERR_ARG, "out_logits too small");
+    int rc = softcap_out(m, (int)start, (int)valid, softcap, out_logits);
+    if (rc) return rc;
+    if (out_valid) *out_valid = valid;
+    return HIPDEC_OK;
+}
+
+int hipdec_decode_logits_from_id(hipdec_model *m, uint32_t token, float softcap, float *out_logits) {
+    int rc = check_step(m, token, true);
+    if (rc) return rc;
+    if (!out_logits) return fail(m, HIPDEC_ERR_ARG, "null buffer");
+    if ((rc = step_with(m, V_LOGITS, 0, base_params(m, token)))) return rc;
+    if ((rc = softcap_out(m, 0, (int)m->cfg.vocab, softcap, out_logits))) return rc;
+    m->len += 1;
+    return HIPDEC_OK;
+}
+
+int hipdec_prefill(hipdec_model *m, const uint32_t *ids, size_t n, float softcap, float *last_logits) {
+    if (!m || (!ids && n)) return HIPDEC_ERR_ARG;
+    if (n == 0) return HIPDEC_OK;
+    if (m->len + n > m->cfg.seq) return fail(m, HIPDEC_ERR_FULL, "prefill exceeds cfg.seq");
+    for (size_t i = 0; i < n; ++i)
+        if (ids[i] >= m->cfg.vocab) return fail(m, HIPDEC_ERR_ARG, "token id must fit vocab");
+    HCHK(hipEventRecord(m->ev0, m->stream));
+    for (size_t i = 0; i < n; ++i) {
+        StepParams p = base_params(m, ids[i]);
+        p.pos = (int)(m->len + i);
+        int variant = (i + 1 == n && last_logits) ? V_LOGITS : V_X;
+        int rc = step_with(m, variant, i, p);
+        if (rc) return rc;
+    }
+    HCHK(hipEventRecord(m->ev1, m->stream));
+    if (last_logits) {
+        int rc = softcap_out(m, 0, (int)m->cfg.vocab, softcap, last_logits);
+        if (rc) return rc;
+    } else {
+        HCHK(hipStreamSynchronize(m->stream));
+    }
+    HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+    m->len += n;
+    return HIPDEC_OK;
+}
+
+int hipdec_decode_greedy_run(hipdec_model *m, uint32_t token, size_t n_steps, uint32_t *out_tokens) {
+    int rc = check_step(m, token, true);
+    if (rc) return rc;
+    if (n_steps == 0) return HIPDEC_OK;
+    if (!out_tokens) return fail(m, HIPDEC_ERR_ARG, "null buffer");
+    if (m->len + n_steps > m->cfg.seq) return fail(m, HIPDEC_ERR_FULL, "greedy run exceeds cfg.seq");
+    m->h_sp[0] = base_params(m, token);
+    HCHK(hipMemcpyAsync(m->d_sp, &m->h_sp[0], sizeof(StepParams), hipMemcpyHostToDevice, m->stream));
+    HCHK(hipEventRecord(m->ev0, m->stream));
+    for (size_t i = 0; i < n_steps; ++i)
+        if ((rc = run_step(m, V_ARGMAX))) return rc;
+    HCHK(hipEventRecord(m->ev1, m->stream));
+    HCHK(hipMemcpyAsync(m->h_out, m->d_ring, n_steps * 4, hipMemcpyDeviceToHost, m->stream));
+    HCHK(hipStreamSynchronize(m->stream));
+    HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+    memcpy(out_tokens, m->h_out, n_steps * 4);
+    m->len += n_steps;
+    return HIPDEC_OK;
+}
+
+int hipdec_last_device_ms(const hipdec_model *m, float *out_ms) {
+    if (!m || !out_ms) return HIPDEC_ERR_ARG;
+    *out_ms = m->last_ms;
+    return HIPDEC_OK;
+}
+
+int hipdec_bytes_per_token(const hipdec_model *m, size_t kv_len, uint64_t *out_bytes) {
+    if (!m || !out_bytes) return HIPDEC_ERR_ARG;
+    const hipdec_config &c = m->cfg;
+    const uint64_t D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden, V = c.vocab, L = c.nlayers;
+    auto mat = [&](int wt, uint64_t rows, uint64_t K) { return (uint64_t)wt_row_bytes(wt, K) * rows + wt_scale_bytes(wt, rows, K); };
+    uint64_t per_layer = mat(m->wt, Q + 2 * KV, D) + mat(m->wt, D, Q) + mat(m->wt, 2 * H, D) + mat(m->wt, D, H);
+    uint64_t kvsz = m->kvbf16 ? 2 : 4;
+    uint64_t b = L * per_layer + mat(m->embed_wt, V, D) + wt_row_bytes(m->embed_wt, D) + (2 * L + 1) * D * 4 +
+                 L * 2 * (uint64_t)kv_len * KV * kvsz + L * 2 * KV * kvsz;
+    *out_bytes = b;
+    return HIPDEC_OK;
+}
+
+int hipdec_export_weight(hipdec_model *m, size_t layer_idx, uint32_t which, float *out, size_t cap) {
+    if (!m || !out) return HIPDEC_ERR_ARG;
+    const hipdec_config &c = m->cfg;
+    const void *src = nullptr, *sc = nullptr;
+    size_t rows = 0, K = 0;
+    int wt = m->wt;
+    if (which == 4) { src = m->embed; rows = c.vocab; K = c.dim; wt = m->embed_wt; }
+    else {
+        if (layer_idx >= c.nlayers) return fail(m, HIPDEC_ERR_ARG, "layer_idx out of range");
+        const DevLayer &L = m->layers[layer_idx];
+        switch (which) {
+            case 0: src = L.wqkv; sc = L.s_qkv; rows = c.q_dim + 2 * c.kv_dim; K = c.dim; break;
+            case 1: src = L.wo; sc = L.s_wo; rows = c.dim; K = c.q_dim; break;
+            case 2: src = L.w13; sc = L.s_w13; rows = 2 * c.hidden; K = c.dim; break;
+            case 3: src = L.w2; sc = L.s_w2; rows = c.dim; K = c.hidden; break;
+            default: return fail(m, HIPDEC_ERR_ARG, "unknown weight selector");
+        }
+    }
+    if (cap < rows * K) return fail(m, HIPDEC_ERR_ARG, "export buffer too small");
+    float *tmp = nullptr;
+    HCHK(hipMalloc((void **)&tmp, rows * K * 4));
+    switch (wt) {
+        case WT_F32: hipLaunchKernelGGL(k_export_rows<WT_F32>, dim3(rows), dim3(256), 0, m->stream, src, sc, tmp, (int)K); break;
+        case WT_BF16: hipLaunchKernelGGL(k_export_rows<WT_BF16>, dim3(rows), dim3(256), 0, m->stream, src, sc, tmp, (int)K); break;
+        case WT_FP8: hipLaunchKernelGGL(k_export_rows<WT_FP8>, dim3(rows), dim3(256), 0, m->stream, src, sc, tmp, (int)K); break;
+        default: hipLaunchKernelGGL(k_export_rows<WT_INT4>, dim3(rows), dim3(256), 0, m->stream, src, sc, tmp, (int)K); break;
+    }
+    hipError_t e = hipStreamSynchronize(m->stream);
+    if (e == hipSuccess) e = hipMemcpy(out, tmp, rows * K * 4, hipMemcpyDeviceToHost);
+    (void)hipFree(tmp);
+    if (e != hipSuccess) { m->err = hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+    return HIPDEC_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,131 @@
+// Shared device helpers for the gfx950 decode kernels: weight-stream decoders, wave reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define WAVE 64
+
+// ---------------------------------------------------------------- step parameters
+// One small block of device memory carries everything that changes between two replays of a
+// captured step: kernels read it instead of taking launch arguments, so one hipGraph serves
+// every token.  The reference passes slot / attn_len / token as per-dispatch constants
+// (crates/metal-decode/src/lib.rs:249-250, :647, :709, :743, :781).
+struct StepParams {
+    int tok;        // input token id
+    int pos;        // slot = len before the step; attends over pos + 1 rows
+    int step;       // index into the output token ring of a multi-step greedy run
+    int top_k;      // head variant parameter
+    float inv_t;    // block-stats 1/temperature
+    float softcap;  // <= 0 disables
+    int use_x_in;   // 1: the residual stream starts from x_in instead of an embedding row
+    int block_idx;  // materialise: which 256-row block
+};
+
+enum { WT_F32 = 0, WT_BF16 = 1, WT_FP8 = 2, WT_INT4 = 3 };
+
+__device__ __forceinline__ float bf16_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// round-to-nearest-even fp32 -> bf16 bits (finite inputs)
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7f800000u) == 0x7f800000u) return (uint16_t)(u >> 16);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+
+// (value desc, index asc) ordering used by every head kernel of the reference
+// (crates/metal-decode/src/lib.rs:1553, :1612-1613, :1749)
+__device__ __forceinline__ bool better(float v, uint32_t i, float bv, uint32_t bi) {
+    return v > bv || (v == bv && i < bi);
+}
+__device__ __forceinline__ void wave_argbest(float &v, uint32_t &i) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        float ov = __shfl_xor(v, o, WAVE);
+        uint32_t oi = (uint32_t)__shfl_xor((int)i, o, WAVE);
+        if (better(ov, oi, v, i)) { v = ov; i = oi; }
+    }
+}
+
+// ---------------------------------------------------------------- weight stream decoders
+// Every weight matrix is stored out-major: row = output channel, reduction axis contiguous, so
+// one 128-bit load gives a lane EPL consecutive reduction elements of one output row.
+template <int WT> struct WS;
+
+template <> struct WS<WT_F32> {
+    static constexpr int EPL = 4;                       // elements per 16-byte load
+    static __device__ __forceinline__ size_t row_bytes(int K) { return (size_t)K * 4; }
+    static __device__ __forceinline__ void decode(const uint4 &w, float *f) {
+        f[0] = __uint_as_float(w.x); f[1] = __uint_as_float(w.y);
+        f[2] = __uint_as_float(w.z); f[3] = __uint_as_float(w.w);
+    }
+};
+template <> struct WS<WT_BF16> {
+    static constexpr int EPL = 8;
+    static __device__ __forceinline__ size_t row_bytes(int K) { return (size_t)K * 2; }
+    static __device__ __forceinline__ void decode(const uint4 &w, float *f) {
+        f[0] = __uint_as_float(w.x << 16); f[1] = __uint_as_float(w.x & 0xffff0000u);
+        f[2] = __uint_as_float(w.y << 16); f[3] = __uint_as_float(w.y & 0xffff0000u);
+        f[4] = __uint_as_float(w.z << 16); f[5] = __uint_as_float(w.z & 0xffff0000u);
+        f[6] = __uint_as_float(w.w << 16); f[7] = __uint_as_float(w.w & 0xffff0000u);
+    }
+};
+template <> struct WS<WT_FP8> {
+    static constexpr int EPL = 16;
+    static __device__ __forceinline__ size_t row_bytes(int K) { return (size_t)K; }
+    static __device__ __forceinline__ void decode(const uint4 &w, float *f) {
+        const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(u[i], false);   // bytes 0,1 (OCP e4m3 on gfx950)
+            auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(u[i], true);    // bytes 2,3
+            f[4 * i + 0] = lo[0]; f[4 * i + 1] = lo[1];
+            f[4 * i + 2] = hi[0]; f[4 * i + 3] = hi[1];
+        }
+    }
+};
+template <> struct WS<WT_INT4> {
+    static constexpr int EPL = 32;
+    static __device__ __forceinline__ size_t row_bytes(int K) { return (size_t)K / 2; }
+    // nibbles are offset-binary (q + 8); element 2j is the low nibble of byte j
+    static __device__ __forceinline__ void decode(const uint4 &w, float *f) {
+        const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) f[8 * i + j] = (float)(int)((u[i] >> (4 * j)) & 0xfu) - 8.0f;
+    }
+};
+
+// software OCP e4m3fn encoder, round to nearest even, saturating (used once, at weight load)
+__device__ __forceinline__ uint8_t f32_to_e4m3(float f) {
+    uint32_t u = __float_as_uint(f);
+    uint8_t sign = (uint8_t)((u >> 24) & 0x80);
+    float a = fabsf(f);
+    if (a != a) return sign | 0x7f;
+    if (a >= 464.0f) return sign | 0x7e;
+    if (a < 0.0009765625f) return sign;
+    int e;
+    float mant = frexpf(a, &e);
+    int ex = e - 1;
+    if (ex < -6) {
+        int qi = (int)rintf(a * 512.0f);
+        if (qi >= 8) return sign | 0x08;
+        return sign | (uint8_t)qi;
+    }
+    int mi = (int)rintf((2.0f * mant - 1.0f) * 8.0f);
+    if (mi == 8) { mi = 0; ex += 1; }
+    if (ex > 8 || (ex == 8 && mi > 6)) return sign | 0x7e;
+    return sign | (uint8_t)(((ex + 7) << 3) | mi);
+}

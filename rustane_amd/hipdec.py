@@ -1,0 +1,275 @@
+"""ctypes view of the C ABI in include/hip_decode.h.
+
+Method names follow the reference's `metal_decode::Model` (crates/metal-decode/src/lib.rs:146-511)
+so a test written against that type reads the same here.  Errors the reference raises as panics
+come back as `HipDecodeError` carrying the status code.  There is no CPU fallback: if the library
+is missing, importing a model fails.
+"""
+import ctypes as C
+import enum
+import os
+
+import numpy as np
+
+_LIB = None
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libhipdecode.so")
+
+MAX_GPU_TOPK = 32
+HEAD_BLOCK = 256
+
+OK, ERR_ARG, ERR_FULL, ERR_HIP, ERR_UNSUPPORTED = 0, 1, 2, 3, 4
+
+EXPORTS = [
+    "hipdec_create", "hipdec_destroy", "hipdec_last_error", "hipdec_len", "hipdec_set_len",
+    "hipdec_seed_layer_cache_from_channel_first", "hipdec_decode_token", "hipdec_decode_token_from_id",
+    "hipdec_decode_token_argmax", "hipdec_decode_token_argmax_from_id", "hipdec_decode_token_topk_from_id",
+    "hipdec_decode_token_block_stats_from_id", "hipdec_materialize_current_logits_block",
+    "hipdec_decode_logits_from_id", "hipdec_prefill", "hipdec_decode_greedy_run", "hipdec_last_device_ms",
+    "hipdec_bytes_per_token", "hipdec_export_weight",
+]
+
+
+class WeightDtype(enum.IntEnum):
+    F32 = 0
+    BF16 = 1
+    FP8_E4M3 = 2
+    INT4_G128 = 3
+
+
+class KvDtype(enum.IntEnum):
+    F32 = 0
+    BF16 = 1
+
+
+class HipDecodeError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__("hipdec status %d: %s" % (status, message))
+        self.status = status
+
+
+class Config(C.Structure):
+    """metal_decode::Config, crates/metal-decode/src/lib.rs:22-35."""
+    _fields_ = [(n, C.c_uint32) for n in
+                ("dim", "hidden", "heads", "kv_heads", "hd", "seq", "nlayers", "vocab", "q_dim", "kv_dim", "gqa_ratio")]
+
+    @classmethod
+    def make(cls, dim, hidden, heads, hd, seq, nlayers, vocab, kv_heads=None):
+        kv_heads = heads if kv_heads is None else kv_heads
+        return cls(dim, hidden, heads, kv_heads, hd, seq, nlayers, vocab, heads * hd, kv_heads * hd, heads // kv_heads)
+
+    def param_count(self):
+        """ModelConfig::param_count, crates/engine/src/model.rs:182-187."""
+        per_layer = 4 * self.dim * self.dim + 3 * self.dim * self.hidden
+        return self.nlayers * per_layer + self.vocab * self.dim + self.dim * (2 * self.nlayers + 1)
+
+
+class _Layer(C.Structure):
+    _fields_ = [(n, C.POINTER(C.c_float)) for n in ("wq", "wk", "wv", "wo", "w1", "w3", "w2", "gamma1", "gamma2")]
+
+
+class _Head(C.Structure):
+    _fields_ = [("gamma_final", C.POINTER(C.c_float)), ("embed", C.POINTER(C.c_float))]
+
+
+class _Options(C.Structure):
+    _fields_ = [("weight_dtype", C.c_uint32), ("kv_dtype", C.c_uint32), ("device", C.c_int32),
+                ("ffn_activation", C.c_uint32), ("flags", C.c_uint32), ("max_rows", C.c_uint32)]
+
+
+FLAG_NO_GRAPH = 1
+
+
+def load_library(path=None):
+    """Loads libhipdecode.so (built in-tree by `__graft_entry__.build()`); raises if absent."""
+    global _LIB
+    if _LIB is not None and path is None:
+        return _LIB
+    p = path or _LIB_PATH
+    if not os.path.exists(p):
+        raise HipDecodeError(ERR_HIP, "%s not found: build it with __graft_entry__.build()" % p)
+    lib = C.CDLL(p)
+    lib.hipdec_last_error.restype = C.c_char_p
+    lib.hipdec_last_error.argtypes = [C.c_void_p]
+    lib.hipdec_len.restype = C.c_size_t
+    lib.hipdec_len.argtypes = [C.c_void_p]
+    lib.hipdec_destroy.restype = None
+    lib.hipdec_destroy.argtypes = [C.c_void_p]
+    fp, u32p = C.POINTER(C.c_float), C.POINTER(C.c_uint32)
+    lib.hipdec_create.argtypes = [C.POINTER(Config), C.POINTER(_Layer), C.c_size_t, C.POINTER(_Head),
+                                  C.POINTER(_Options), C.POINTER(C.c_void_p)]
+    lib.hipdec_set_len.argtypes = [C.c_void_p, C.c_size_t]
+    lib.hipdec_seed_layer_cache_from_channel_first.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, fp, fp]
+    lib.hipdec_decode_token.argtypes = [C.c_void_p, fp, fp]
+    lib.hipdec_decode_token_from_id.argtypes = [C.c_void_p, C.c_uint32, fp]
+    lib.hipdec_decode_token_argmax.argtypes = [C.c_void_p, fp, u32p]
+    lib.hipdec_decode_token_argmax_from_id.argtypes = [C.c_void_p, C.c_uint32, u32p]
+    lib.hipdec_decode_token_topk_from_id.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, fp, u32p, C.c_size_t,
+                                                     C.POINTER(C.c_size_t)]
+    lib.hipdec_decode_token_block_stats_from_id.argtypes = [C.c_void_p, C.c_uint32, C.c_float, C.c_float, fp, fp,
+                                                            C.c_size_t, C.POINTER(C.c_size_t)]
+    lib.hipdec_materialize_current_logits_block.argtypes = [C.c_void_p, C.c_size_t, C.c_float, fp, C.c_size_t,
+                                                            C.POINTER(C.c_size_t)]
+    lib.hipdec_decode_logits_from_id.argtypes = [C.c_void_p, C.c_uint32, C.c_float, fp]
+    lib.hipdec_prefill.argtypes = [C.c_void_p, u32p, C.c_size_t, C.c_float, fp]
+    lib.hipdec_decode_greedy_run.argtypes = [C.c_void_p, C.c_uint32, C.c_size_t, u32p]
+    lib.hipdec_last_device_ms.argtypes = [C.c_void_p, fp]
+    lib.hipdec_bytes_per_token.argtypes = [C.c_void_p, C.c_size_t, C.POINTER(C.c_uint64)]
+    lib.hipdec_export_weight.argtypes = [C.c_void_p, C.c_size_t, C.c_uint32, fp, C.c_size_t]
+    if path is None:
+        _LIB = lib
+    return lib
+
+
+def _fptr(a):
+    return a.ctypes.data_as(C.POINTER(C.c_float))
+
+
+def _f32(a, n=None, name="array"):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    if n is not None and a.size != n:
+        raise ValueError("%s has %d elements, expected %d" % (name, a.size, n))
+    return a
+
+
+class HipDecodeModel:
+    """`metal_decode::Model` over the HIP backend.
+
+    weights: dict with "embed" [vocab*dim], "gamma_final" [dim] and "layers": list of dicts with
+    wq wk wv wo w1 w3 w2 gamma1 gamma2 in the reference's layouts (crates/engine/src/layer.rs:19-36).
+    """
+
+    def __init__(self, cfg, weights, weight_dtype=WeightDtype.F32, kv_dtype=KvDtype.F32, device=0,
+                 ffn_activation=0, flags=0):
+        self._lib = load_library()
+        self._h = C.c_void_p()
+        self.cfg = cfg
+        D, Q, KV, H, V = cfg.dim, cfg.q_dim, cfg.kv_dim, cfg.hidden, cfg.vocab
+        sizes = dict(wq=D * Q, wk=D * KV, wv=D * KV, wo=Q * D, w1=D * H, w3=D * H, w2=D * H, gamma1=D, gamma2=D)
+        keep = []
+        layers = (_Layer * len(weights["layers"]))()
+        for i, lw in enumerate(weights["layers"]):
+            for name, n in sizes.items():
+                a = _f32(lw[name], n, name)
+                keep.append(a)
+                setattr(layers[i], name, _fptr(a))
+        embed = _f32(weights["embed"], V * D, "embed")
+        gf = _f32(weights["gamma_final"], D, "gamma_final")
+        head = _Head(_fptr(gf), _fptr(embed))
+        opts = _Options(int(weight_dtype), int(kv_dtype), device, ffn_activation, flags, 0)
+        rc = self._lib.hipdec_create(C.byref(cfg), layers, len(weights["layers"]), C.byref(head), C.byref(opts),
+                                     C.byref(self._h))
+        if rc != OK:
+            raise HipDecodeError(rc, (self._lib.hipdec_last_error(None) or b"").decode())
+        self.blocks = (V + HEAD_BLOCK - 1) // HEAD_BLOCK
+
+    def close(self):
+        if getattr(self, "_h", None) and self._h.value:
+            self._lib.hipdec_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _chk(self, rc):
+        if rc != OK:
+            raise HipDecodeError(rc, (self._lib.hipdec_last_error(self._h) or b"").decode())
+
+    # ---- metal_decode::Model surface
+    def len(self):
+        return int(self._lib.hipdec_len(self._h))
+
+    def set_len(self, n):
+        self._chk(self._lib.hipdec_set_len(self._h, n))
+
+    def seed_layer_cache_from_channel_first(self, layer_idx, live_len, k_rope_cf, v_cf):
+        n = self.cfg.kv_dim * self.cfg.seq
+        k, v = _f32(k_rope_cf, n, "k_rope_cf"), _f32(v_cf, n, "v_cf")
+        self._chk(self._lib.hipdec_seed_layer_cache_from_channel_first(self._h, layer_idx, live_len, _fptr(k), _fptr(v)))
+
+    def decode_token(self, x_in):
+        x = _f32(x_in, self.cfg.dim, "x_in")
+        out = np.empty(self.cfg.dim, np.float32)
+        self._chk(self._lib.hipdec_decode_token(self._h, _fptr(x), _fptr(out)))
+        return out
+
+    def decode_token_from_id(self, token):
+        out = np.empty(self.cfg.dim, np.float32)
+        self._chk(self._lib.hipdec_decode_token_from_id(self._h, token, _fptr(out)))
+        return out
+
+    def decode_token_argmax(self, x_in):
+        x = _f32(x_in, self.cfg.dim, "x_in")
+        t = C.c_uint32()
+        self._chk(self._lib.hipdec_decode_token_argmax(self._h, _fptr(x), C.byref(t)))
+        return t.value
+
+    def decode_token_argmax_from_id(self, token):
+        t = C.c_uint32()
+        self._chk(self._lib.hipdec_decode_token_argmax_from_id(self._h, token, C.byref(t)))
+        return t.value
+
+    def decode_token_topk_from_id(self, token, top_k, cap=None):
+        cap = self.blocks * max(int(top_k), 1) if cap is None else cap
+        vals = np.empty(max(cap, 1), np.float32)
+        idxs = np.empty(max(cap, 1), np.uint32)
+        cnt = C.c_size_t()
+        self._chk(self._lib.hipdec_decode_token_topk_from_id(
+            self._h, token, top_k, _fptr(vals), idxs.ctypes.data_as(C.POINTER(C.c_uint32)), cap, C.byref(cnt)))
+        return vals[:cnt.value], idxs[:cnt.value]
+
+    def decode_token_block_stats_from_id(self, token, inv_temperature, softcap, cap=None):
+        cap = self.blocks if cap is None else cap
+        mx = np.empty(max(cap, 1), np.float32)
+        sm = np.empty(max(cap, 1), np.float32)
+        cnt = C.c_size_t()
+        self._chk(self._lib.hipdec_decode_token_block_stats_from_id(
+            self._h, token, inv_temperature, softcap, _fptr(mx), _fptr(sm), cap, C.byref(cnt)))
+        return mx[:cnt.value], sm[:cnt.value]
+
+    def materialize_current_logits_block(self, block_idx, softcap, cap=HEAD_BLOCK):
+        out = np.empty(max(cap, 1), np.float32)
+        valid = C.c_size_t()
+        self._chk(self._lib.hipdec_materialize_current_logits_block(self._h, block_idx, softcap, _fptr(out), cap,
+                                                                    C.byref(valid)))
+        return out[:valid.value]
+
+    # ---- additions
+    def decode_logits_from_id(self, token, softcap=0.0):
+        out = np.empty(self.cfg.vocab, np.float32)
+        self._chk(self._lib.hipdec_decode_logits_from_id(self._h, token, softcap, _fptr(out)))
+        return out
+
+    def prefill(self, ids, softcap=0.0, want_logits=True):
+        ids = np.ascontiguousarray(ids, dtype=np.uint32)
+        out = np.empty(self.cfg.vocab, np.float32) if want_logits else None
+        self._chk(self._lib.hipdec_prefill(self._h, ids.ctypes.data_as(C.POINTER(C.c_uint32)), ids.size, softcap,
+                                           _fptr(out) if want_logits else None))
+        return out
+
+    def decode_greedy_run(self, token, n_steps):
+        out = np.empty(max(n_steps, 1), np.uint32)
+        self._chk(self._lib.hipdec_decode_greedy_run(self._h, token, n_steps,
+                                                     out.ctypes.data_as(C.POINTER(C.c_uint32))))
+        return out[:n_steps]
+
+    def last_device_ms(self):
+        ms = C.c_float()
+        self._chk(self._lib.hipdec_last_device_ms(self._h, C.byref(ms)))
+        return ms.value
+
+    def bytes_per_token(self, kv_len):
+        b = C.c_uint64()
+        self._chk(self._lib.hipdec_bytes_per_token(self._h, kv_len, C.byref(b)))
+        return b.value
+
+    def export_weight(self, layer_idx, which):
+        c = self.cfg
+        shapes = {0: (c.q_dim + 2 * c.kv_dim, c.dim), 1: (c.dim, c.q_dim), 2: (2 * c.hidden, c.dim),
+                  3: (c.dim, c.hidden), 4: (c.vocab, c.dim)}
+        rows, k = shapes[which]
+        out = np.empty(rows * k, np.float32)
+        self._chk(self._lib.hipdec_export_weight(self._h, layer_idx, which, _fptr(out), out.size))
+        return out.reshape(rows, k)

@@ -1,0 +1,290 @@
+"""GPU parity: the HIP decode backend, called through the C ABI, against the CPU oracle on the
+same seeded weights and prompts.  Shapes and tolerances follow the reference's own decode parity
+tests (crates/engine/tests/auto_kv_decode.rs:7-28, :67-215): exact greedy ids, exact top-k ids,
+1e-4 on logits, 1e-3 on block sums."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from rustane_amd import synth
+from rustane_amd.hipdec import (Config, HipDecodeModel, HipDecodeError, KvDtype, WeightDtype, ERR_ARG, ERR_FULL)
+
+pytestmark = pytest.mark.gpu
+
+
+def tiny_cfg(vocab=64):
+    # auto_kv_decode.rs:7-21 (vocab 64) and :23-28 (vocab 320 = two head blocks)
+    return Config.make(dim=256, hidden=640, heads=2, hd=128, seq=64, nlayers=2, vocab=vocab)
+
+
+def rel_err(a, b):
+    return float(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64)).max() / max(np.abs(b).max(), 1e-30))
+
+
+def pair(cfg, seed=11, std=0.02, wdt=WeightDtype.F32, kvdt=KvDtype.F32, flags=0, act=0):
+    w = synth.make_weights(cfg, seed=seed, std=std, round_bf16=(wdt != WeightDtype.F32))
+    orc = O.Oracle(cfg, w, kv_round_bf16=(kvdt == KvDtype.BF16), ffn_activation=act)
+    dev = HipDecodeModel(cfg, w, weight_dtype=wdt, kv_dtype=kvdt, flags=flags, ffn_activation=act)
+    return w, orc, dev
+
+
+@pytest.mark.parametrize("std", [0.02, 0.08])
+@pytest.mark.parametrize("flags", [0, 1])
+def test_prefill_then_logits_match_oracle_fp32(std, flags):
+    cfg = tiny_cfg(320)
+    w, orc, dev = pair(cfg, std=std, flags=flags)
+    ids = np.array([1, 2, 3, 4, 5], np.uint32)
+    lg_o, _, _ = orc.forward_window(ids)
+    lg_d = dev.prefill(ids)
+    assert dev.len() == 5 and orc.len() == 5
+    assert rel_err(lg_d, lg_o[0]) < 1e-4
+    tok = int(O.argmax_lower(lg_o[0]))
+    for _ in range(6):
+        a = orc.decode_logits_from_id(tok)
+        b = dev.decode_logits_from_id(tok)
+        assert rel_err(b, a) < 1e-4
+        assert O.argmax_lower(b) == O.argmax_lower(a)
+        tok = int(O.argmax_lower(a))
+    assert dev.len() == 11
+
+
+def test_seeded_cache_greedy_tokens_match_window_forward():
+    # auto_kv_decode.rs:67-134: prompt through the full-window forward, caches handed over
+    # channel-first, then three cached steps against re-running the window.
+    cfg = tiny_cfg(64)
+    w, orc, dev = pair(cfg, std=0.08)
+    generated = [1, 2, 3]
+    lg, k_cf, v_cf = orc.forward_window(np.array(generated, np.uint32), want_caches=True)
+    dev.set_len(len(generated))
+    for l in range(cfg.nlayers):
+        dev.seed_layer_cache_from_channel_first(l, len(generated), k_cf[l], v_cf[l])
+    nxt = int(O.argmax_last(lg[0]))
+    generated.append(nxt)
+    for _ in range(3):
+        cached_next = dev.decode_token_argmax_from_id(nxt)
+        lg, _, _ = O.Oracle(cfg, w).forward_window(np.array(generated, np.uint32))
+        assert cached_next == int(O.argmax_lower(lg[0]))
+        nxt = cached_next
+        generated.append(nxt)
+
+
+def test_decode_token_variants_match_oracle():
+    cfg = tiny_cfg(64)
+    w, orc, dev = pair(cfg, std=0.08)
+    for tok in (3, 9):
+        a = orc.decode_token_from_id(tok)
+        b = dev.decode_token_from_id(tok)
+        assert rel_err(b, a) < 1e-5
+    x_in = synth.synth_normal(99, 7, cfg.dim, std=0.3)
+    a = orc.decode_token(x_in)
+    b = dev.decode_token(x_in)
+    assert rel_err(b, a) < 1e-5
+    # argmax from a caller-supplied residual stream
+    orc_x = orc.decode_token(x_in)
+    xf = orc_x / np.sqrt((orc_x.astype(np.float64) ** 2).mean() + 1e-5)
+    want = int(np.argmax(w["embed"].reshape(cfg.vocab, cfg.dim).astype(np.float64) @ xf))
+    got = dev.decode_token_argmax(x_in)
+    assert got == want
+    assert dev.len() == 4
+
+
+def test_topk_candidates_match_oracle():
+    # auto_kv_decode.rs:136-173 (vocab 320: the second block is ragged)
+    cfg = tiny_cfg(320)
+    w, orc, dev = pair(cfg, std=0.08)
+    ids = np.array([1, 2, 3], np.uint32)
+    orc.forward_window(ids)
+    dev.prefill(ids, want_logits=False)
+    for k in (1, 4, 32):
+        raw = orc.decode_logits_from_id(7)
+        vals, idxs = dev.decode_token_topk_from_id(7, k)
+        ov, oi = O.block_topk(raw, k)
+        assert vals.size == dev.blocks * k
+        np.testing.assert_array_equal(idxs, oi)
+        finite = np.isfinite(ov)
+        assert rel_err(vals[finite], ov[finite]) < 1e-4
+        assert np.all(np.isneginf(vals[~finite]))
+        mv, mi = O.merge_topk(vals, idxs, k)
+        order = np.lexsort((np.arange(raw.size), -raw))[:k]
+        np.testing.assert_array_equal(mi, order.astype(np.uint32))
+
+
+def test_block_stats_and_materialize_match_oracle():
+    # auto_kv_decode.rs:175-215
+    cfg = tiny_cfg(320)
+    w, orc, dev = pair(cfg, std=0.08)
+    ids = np.array([1, 2, 3, 4], np.uint32)
+    orc.forward_window(ids)
+    dev.prefill(ids, want_logits=False)
+    for temperature, softcap in ((0.8, 0.0), (1.0, 5.0)):
+        raw = orc.decode_logits_from_id(5)
+        mx, sm = dev.decode_token_block_stats_from_id(5, 1.0 / temperature, softcap)
+        omx, osm = O.block_stats(raw, 1.0 / temperature, softcap)
+        assert np.abs(mx - omx).max() < 1e-4
+        assert np.abs(sm - osm).max() < 1e-3
+        blk = dev.materialize_current_logits_block(1, softcap)
+        want = O.materialize_block(raw, 1, softcap)
+        assert blk.size == 64
+        assert np.abs(blk - want).max() < 1e-4
+    assert dev.len() == 6          # materialise does not advance
+
+
+def test_greedy_run_equals_single_steps_and_oracle():
+    cfg = tiny_cfg(320)
+    w, orc, dev = pair(cfg, std=0.08)
+    _, _, dev2 = pair(cfg, std=0.08)
+    ids = np.array([5, 6, 7], np.uint32)
+    lg, _, _ = orc.forward_window(ids)
+    dev.prefill(ids, want_logits=False)
+    dev2.prefill(ids, want_logits=False)
+    first = int(O.argmax_last(lg[0]))
+    run = dev.decode_greedy_run(first, 20)
+    cur, singles = first, []
+    for _ in range(20):
+        cur = dev2.decode_token_argmax_from_id(cur)
+        singles.append(cur)
+    np.testing.assert_array_equal(run, np.array(singles, np.uint32))
+    sampled, _ = orc.run_cached_sample(ids, lg[0], 21)
+    np.testing.assert_array_equal(run, sampled[1:])
+    assert dev.len() == 23 and dev2.len() == 23
+
+
+def test_c1_tiny_greedy_32_steps_identical_and_logits_1e4():
+    # configuration 1: dim 512, 8 layers, 8 heads x 64, hidden 1536, vocab 8192, seq 512, fp32
+    cfg = synth.config_c1()
+    w, orc, dev = pair(cfg, seed=1234)
+    prompt = synth.make_prompt(7, cfg.vocab, 4)
+    lg_o, _, _ = orc.forward_window(prompt)
+    lg_d = dev.prefill(prompt)
+    assert rel_err(lg_d, lg_o[0]) < 1e-4
+    sampled, _ = orc.run_cached_sample(prompt, lg_o[0], 32)
+    got = dev.decode_greedy_run(int(sampled[0]), 31)
+    np.testing.assert_array_equal(got, sampled[1:])
+    a = orc.decode_logits_from_id(int(sampled[-1]))
+    b = dev.decode_logits_from_id(int(sampled[-1]))
+    assert rel_err(b, a) < 1e-4
+
+
+def test_c1_shape_nondegenerate_stream():
+    # same shape with wider weights so that the greedy stream is not a fixed point
+    cfg = synth.config_c1()
+    w, orc, dev = pair(cfg, seed=77, std=0.07)
+    prompt = synth.make_prompt(9, cfg.vocab, 6)
+    lg_o, _, _ = orc.forward_window(prompt)
+    lg_d = dev.prefill(prompt)
+    assert rel_err(lg_d, lg_o[0]) < 1e-4
+    sampled, _ = orc.run_cached_sample(prompt, lg_o[0], 48)
+    assert len(set(sampled.tolist())) > 8
+    got = dev.decode_greedy_run(int(sampled[0]), 47)
+    np.testing.assert_array_equal(got, sampled[1:])
+
+
+@pytest.mark.parametrize("kvdt", [KvDtype.F32, KvDtype.BF16])
+def test_bf16_weights_match_oracle(kvdt):
+    cfg = Config.make(dim=512, hidden=1024, heads=4, hd=128, seq=128, nlayers=3, vocab=1000)
+    w, orc, dev = pair(cfg, seed=3, std=0.06, wdt=WeightDtype.BF16, kvdt=kvdt)
+    ids = synth.make_prompt(3, cfg.vocab, 9)
+    lg_o, _, _ = orc.forward_window(ids)
+    lg_d = dev.prefill(ids)
+    assert rel_err(lg_d, lg_o[0]) < 2e-2       # north-star bf16 bound
+    # fp32 accumulation over bf16-exact weights agrees to round-off; with a bf16 cache a 1-ulp
+    # difference upstream can flip the rounding of a cached value, which is a 2^-8 step
+    assert rel_err(lg_d, lg_o[0]) < (1e-4 if kvdt == KvDtype.F32 else 2e-3)
+    sampled, _ = orc.run_cached_sample(ids, lg_o[0], 40)
+    got = dev.decode_greedy_run(int(sampled[0]), 39)
+    np.testing.assert_array_equal(got, sampled[1:])
+    k = orc.kcache(1)[: dev.len()]
+    assert np.isfinite(k).all()
+
+
+def test_leaky_relu_sq_activation():
+    cfg = tiny_cfg(320)
+    w, orc, dev = pair(cfg, std=0.08, act=1)
+    ids = np.array([1, 2, 3], np.uint32)
+    lg_o, _, _ = orc.forward_window(ids)
+    lg_d = dev.prefill(ids)
+    assert rel_err(lg_d, lg_o[0]) < 1e-4
+
+
+@pytest.mark.parametrize("wdt,which_tol", [(WeightDtype.FP8_E4M3, 5e-2), (WeightDtype.INT4_G128, 5e-2)])
+def test_quantised_weights_bit_exact_and_logits(wdt, which_tol):
+    cfg = Config.make(dim=512, hidden=1024, heads=4, hd=128, seq=64, nlayers=2, vocab=512)
+    w = synth.make_weights(cfg, seed=21, std=0.05, round_bf16=True)
+    dev = HipDecodeModel(cfg, w, weight_dtype=wdt, kv_dtype=KvDtype.BF16)
+    L = O.lib()
+    D, Q, KV, H = cfg.dim, cfg.q_dim, cfg.kv_dim, cfg.hidden
+
+    def out_major(a, rows_in, cols_in, transpose):
+        a = O.f32(a).reshape(rows_in, cols_in)
+        return np.ascontiguousarray(a.T) if transpose else a
+
+    def dq(m):
+        m = np.ascontiguousarray(m, np.float32)
+        out = np.empty_like(m)
+        if wdt == WeightDtype.FP8_E4M3:
+            L.orc_quant_fp8_rows(O.P(m), m.shape[0], m.shape[1], None, None, O.P(out))
+        else:
+            L.orc_quant_int4_g128(O.P(m), m.shape[0], m.shape[1], None, None, O.P(out))
+        return out
+
+    wq_dq = {"embed": w["embed"], "gamma_final": w["gamma_final"], "layers": []}
+    for l, lw in enumerate(w["layers"]):
+        mats = {n: dq(out_major(lw[n], *shape)) for n, shape in
+                dict(wq=(D, Q, True), wk=(D, KV, True), wv=(D, KV, True), wo=(Q, D, True), w1=(D, H, True),
+                     w3=(D, H, True), w2=(D, H, False)).items()}
+        # stored weights, de-quantised on the device, must equal the oracle's bit for bit
+        qkv = dev.export_weight(l, 0)
+        np.testing.assert_array_equal(qkv, np.concatenate([mats["wq"], mats["wk"], mats["wv"]], 0))
+        np.testing.assert_array_equal(dev.export_weight(l, 1), mats["wo"])
+        w13 = dev.export_weight(l, 2)
+        np.testing.assert_array_equal(w13[0::2], mats["w1"])
+        np.testing.assert_array_equal(w13[1::2], mats["w3"])
+        np.testing.assert_array_equal(dev.export_weight(l, 3), mats["w2"])
+        lay = {n: np.ascontiguousarray(mats[n].T).ravel() for n in ("wq", "wk", "wv", "wo", "w1", "w3")}
+        lay["w2"] = mats["w2"].ravel()
+        lay["gamma1"], lay["gamma2"] = lw["gamma1"], lw["gamma2"]
+        wq_dq["layers"].append(lay)
+    np.testing.assert_array_equal(dev.export_weight(0, 4).ravel(), w["embed"])
+    orc = O.Oracle(cfg, wq_dq, kv_round_bf16=True)
+    ids = synth.make_prompt(5, cfg.vocab, 6)
+    lg_o, _, _ = orc.forward_window(ids)
+    lg_d = dev.prefill(ids)
+    assert rel_err(lg_d, lg_o[0]) < which_tol
+    assert rel_err(lg_d, lg_o[0]) < 1e-4
+    sampled, _ = orc.run_cached_sample(ids, lg_o[0], 24)
+    got = dev.decode_greedy_run(int(sampled[0]), 23)
+    np.testing.assert_array_equal(got, sampled[1:])
+
+
+def test_error_codes_replace_panics():
+    # crates/metal-decode/src/lib.rs:242-245, :277-280, :392-405, :452-453, :495, :501
+    cfg = tiny_cfg(320)
+    w, orc, dev = pair(cfg)
+    with pytest.raises(HipDecodeError) as e:
+        dev.decode_token_argmax_from_id(cfg.vocab)
+    assert e.value.status == ERR_ARG
+    for k in (0, 33):
+        with pytest.raises(HipDecodeError) as e:
+            dev.decode_token_topk_from_id(1, k)
+        assert e.value.status == ERR_ARG
+    with pytest.raises(HipDecodeError) as e:
+        dev.decode_token_topk_from_id(1, 4, cap=7)
+    assert e.value.status == ERR_ARG
+    with pytest.raises(HipDecodeError) as e:
+        dev.decode_token_block_stats_from_id(1, 1.0, 0.0, cap=1)
+    assert e.value.status == ERR_ARG
+    with pytest.raises(HipDecodeError) as e:
+        dev.materialize_current_logits_block(2, 0.0)
+    assert e.value.status == ERR_ARG
+    with pytest.raises(HipDecodeError) as e:
+        dev.materialize_current_logits_block(1, 0.0, cap=10)
+    assert e.value.status == ERR_ARG
+    assert dev.len() == 0
+    dev.set_len(10_000)
+    assert dev.len() == cfg.seq            # set_len clamps, lib.rs:213-215
+    with pytest.raises(HipDecodeError) as e:
+        dev.decode_token_argmax_from_id(1)
+    assert e.value.status == ERR_FULL
+    dev.set_len(cfg.seq - 1)
+    dev.decode_token_argmax_from_id(1)     # the last slot is usable
+    assert dev.len() == cfg.seq
