@@ -1,0 +1,139 @@
+#!/usr/bin/env python3
+"""Decode benchmark: tokens/s of the batch-1 KV-cache greedy token loop on one MI355X.
+
+A "step" is one decoded token (one pass of the whole token loop: embedding row, every layer,
+final norm, tied LM head, argmax).  The default workload is the configuration the headline metric
+is quoted on: the 600M-class bf16 model (dim 1536, 24 layers, 12 heads x 128, hidden 4096, vocab
+32768, seq 2048), a 128-token random prompt, greedy decode at batch 1.  Weights are synthetic
+N(0, 0.02) from a fixed seed and already resident in HBM when the timed region starts.
+
+Prints ONE JSON line (see the keys below).  `roofline.achieved` is the algorithmic bytes one token
+step streams (weights + scales + norms + one embedding row + the KV rows it reads and writes) divided
+by the per-step device time measured with HIP events on the model's own stream.
+`cpu_baseline` times the CPU oracle's cached token loop on a bounded number of steps of the same
+model on this box's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0
+
+WORKLOADS = {
+    # name: (config factory name, weight dtype, kv dtype, prompt tokens, generated steps)
+    "c1_tiny_fp32": ("config_c1", "F32", "F32", 4, 32),
+    "c2_600m_bf16_bs1": ("config_600m", "BF16", "BF16", 128, 256),
+    "c4_5b_bf16_bs1": ("config_5b", "BF16", "BF16", 1024, 128),
+    "c5_5b_fp8_bs1": ("config_5b", "FP8_E4M3", "BF16", 512, 256),
+    "c5_5b_int4_bs1": ("config_5b", "INT4_G128", "BF16", 512, 256),
+}
+
+
+def cpu_baseline(cfg, weights, kv_bf16, budget_s=20.0, max_steps=64):
+    """Times the oracle's KV-cached token loop (the CPU restatement of the reference's arithmetic)
+    from an empty cache; the weight stream dominates its cost, so the rate barely depends on the
+    position.  Returns the cpu_baseline object."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib as O
+    orc = O.Oracle(cfg, weights, kv_round_bf16=kv_bf16)
+    tok, n, t0 = 1, 0, time.perf_counter()
+    while n < max_steps and n < cfg.seq:
+        lg = orc.decode_logits_from_id(tok)
+        tok = int(O.argmax_lower(lg))
+        n += 1
+        if time.perf_counter() - t0 > budget_s:
+            break
+    dt = time.perf_counter() - t0
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {"value": n / dt, "unit": "tok/s", "cores": cores, "kind": "port",
+            "sample": "%d KV-cached greedy steps of the same model from an empty cache, fp32 CPU oracle" % n}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=255)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--workload", default="c2_600m_bf16_bs1", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=1234)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this decode path runs on one GPU (no sharding); --gpus %d is not supported" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    from rustane_amd import synth
+    from rustane_amd.hipdec import HipDecodeModel, KvDtype, WeightDtype
+
+    cfg_name, wdt, kvdt, n_prompt, gen_steps = WORKLOADS[args.workload]
+    cfg = getattr(synth, cfg_name)()
+    wdt, kvdt = WeightDtype[wdt], KvDtype[kvdt]
+    weights = synth.make_weights(cfg, seed=args.seed, std=0.02, round_bf16=(wdt != WeightDtype.F32))
+    dev = HipDecodeModel(cfg, weights, weight_dtype=wdt, kv_dtype=kvdt)
+    prompt = synth.make_prompt(7, cfg.vocab, n_prompt)
+
+    # prefill (reported, not part of the timed decode region)
+    t0 = time.perf_counter()
+    logits = dev.prefill(prompt)
+    prefill_wall_ms = (time.perf_counter() - t0) * 1e3
+    prefill_dev_ms = dev.last_device_ms()
+    first = int(np.argmax(logits))
+
+    room = cfg.seq - n_prompt
+    K, W = args.steps, args.warmup
+    if W > 0:
+        dev.decode_greedy_run(first, min(W, room))
+    # timed region: exactly K greedy steps, in runs that restart at the end of the prompt so every
+    # run sees the same KV lengths the workload defines; each run call returns after a stream sync
+    run_len = min(gen_steps - 1, room)
+    done, wall, dev_ms, kv_sum = 0, 0.0, 0.0, 0
+    while done < K:
+        n = min(run_len, K - done)
+        dev.set_len(n_prompt)
+        t0 = time.perf_counter()
+        dev.decode_greedy_run(first, n)
+        wall += time.perf_counter() - t0
+        dev_ms += dev.last_device_ms()
+        kv_sum += sum(range(n_prompt + 1, n_prompt + n + 1))
+        done += n
+    mean_kv = kv_sum // max(done, 1)
+    bytes_per_step = dev.bytes_per_token(mean_kv)
+    achieved = bytes_per_step * K / (dev_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "decode tok/s @600M bf16 bs1; % of HBM peak GB/s; prefill ms",
+        "value": K / wall,
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": wall * 1e3 / K,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {"F32": "f32", "BF16": "bf16", "FP8_E4M3": "fp8_e4m3", "INT4_G128": "int4"}[wdt.name],
+        "data": "synthetic",
+        "config": {"workload": args.workload, "prompt_tokens": n_prompt, "batch": 1, "kv_dtype": kvdt.name.lower(),
+                   "params": cfg.param_count(), "mean_kv_len": mean_kv},
+        "prefill_ms": prefill_dev_ms,
+        "prefill_wall_ms": prefill_wall_ms,
+        "device_ms_per_step": dev_ms / K,
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "bytes_per_step": bytes_per_step},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, weights, kvdt == KvDtype.BF16)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -191,8 +191,8 @@ static float softcap_f(float x, float cap) { return cap > 0.0f ? cap * tanhf(x /
 /* One query row of causal attention for every head over cache rows [0, n)  (lib.rs:1426-1489;
  * sdpa_fwd.rs:325-354 masks t2 > t with -65504 before the softmax, which in fp32 is the same as
  * leaving those positions out). */
-static void attend_row(const orc_config *c, const float *q, const float *kc, const float *vc,
-                       int n, float *out, float *scores) {
+void orc_attend_row(const orc_config *c, const float *q, const float *kc, const float *vc,
+                    int n, float *out, float *scores) {
     int hd = c->hd, KV = c->kv_dim;
     float scale = 1.0f / sqrtf((float)hd);
     for (int h = 0; h < c->heads; ++h) {
@@ -333,7 +333,7 @@ int orc_forward_window(orc_model *m, const uint32_t *input, int n_rows, float so
             float *scores = (float *)malloc(sizeof(float) * S);
             #pragma omp for schedule(dynamic, 4)
             for (int t = 0; t < T; ++t)
-                attend_row(c, q + (size_t)t * Q, m->kc[l], m->vc[l], t + 1, att + (size_t)t * Q, scores);
+                orc_attend_row(c, q + (size_t)t * Q, m->kc[l], m->vc[l], t + 1, att + (size_t)t * Q, scores);
             free(scores);
         }
         orc_gemm_in_major(att, T, Q, w->wo, D, o);
@@ -394,7 +394,7 @@ static int cached_layers(orc_model *m, float *x) {
             m->kc[l][(size_t)slot * KV + d] = m->kv_round_bf16 ? bf16_round(k[d]) : k[d];
             m->vc[l][(size_t)slot * KV + d] = m->kv_round_bf16 ? bf16_round(v[d]) : v[d];
         }
-        attend_row(c, q, m->kc[l], m->vc[l], attn_len, att, scores);
+        orc_attend_row(c, q, m->kc[l], m->vc[l], attn_len, att, scores);
         orc_gemm_in_major(att, 1, Q, w->wo, D, o);
         for (int d = 0; d < D; ++d) x[d] = x[d] + m->alpha * o[d];
         orc_rmsnorm(x, w->gamma2, xn, D);

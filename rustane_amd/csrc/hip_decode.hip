@@ -5,6 +5,7 @@
 
 #include <math.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 #include <string>
 #include <vector>
@@ -419,6 +420,9 @@ int hipdec_create(const hipdec_config *cfg, const hipdec_layer_f32 *layers, size
         return fail(nullptr, HIPDEC_ERR_UNSUPPORTED, "reduction axis does not fit LDS");
     hipdec_model *m = new hipdec_model();
     m->cfg = c;
+    // HIPDEC_NO_GRAPH=1 in the environment forces eager launches (profilers that cannot follow
+    // graph replays still see every kernel)
+    if (const char *e = getenv("HIPDEC_NO_GRAPH")) if (e[0] == '1') o.flags |= HIPDEC_FLAG_NO_GRAPH;
     m->opt = o;
     m->wt = (int)o.weight_dtype;
     m->embed_wt = o.weight_dtype == HIPDEC_W_F32 ? WT_F32 : WT_BF16;

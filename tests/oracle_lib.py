@@ -58,6 +58,7 @@ def lib():
         L.orc_rope_table.argtypes = [C.c_int, C.c_int, fp, fp]
         L.orc_gemm_in_major.argtypes = [fp, C.c_int, C.c_int, fp, C.c_int, fp]
         L.orc_gemm_out_major.argtypes = [fp, C.c_int, C.c_int, fp, C.c_int, fp]
+        L.orc_attend_row.argtypes = [C.POINTER(OrcConfig), fp, fp, fp, C.c_int, fp, fp]
         L.orc_argmax_lower.restype = C.c_uint32
         L.orc_argmax_lower.argtypes = [fp, C.c_int]
         L.orc_argmax_last.restype = C.c_uint32
