@@ -73,6 +73,7 @@ typedef struct {
 } hipdec_options;
 
 #define HIPDEC_FLAG_NO_GRAPH 1u   /* launch kernels eagerly instead of replaying a captured hipGraph */
+#define HIPDEC_FLAG_NO_MEGA 2u    /* one kernel per matrix product instead of the persistent per-token kernel */
 
 typedef struct hipdec_model hipdec_model;
 
@@ -149,6 +150,10 @@ int hipdec_bytes_per_token(const hipdec_model *m, size_t kv_len, uint64_t *out_b
  * out-major [rows][k] order.  which: 0 wqkv (rows q_dim+2*kv_dim, k dim), 1 wo (dim, q_dim),
  * 2 w13 (2*hidden interleaved gate/up rows, dim), 3 w2 (dim, hidden), 4 embed (vocab, dim). */
 int hipdec_export_weight(hipdec_model *m, size_t layer_idx, uint32_t which, float *out, size_t cap);
+
+/* Diagnostic: runs one greedy step with the persistent step kernel and returns the wall-clock stamps
+ * (100 MHz ticks) workgroup 0 took at its phase boundaries: (nlayers + 1) * 32 slots, unused ones 0. */
+int hipdec_debug_step_profile(hipdec_model *m, uint32_t token, uint64_t *out, size_t cap, size_t *out_count);
 
 #ifdef __cplusplus
 }

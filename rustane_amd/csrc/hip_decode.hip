@@ -1,7 +1,7 @@
 // C ABI of the gfx950 decode backend (see include/hip_decode.h): model construction, weight
 // conversion, hipGraph-captured decode steps and the head variants.
 #include "../../include/hip_decode.h"
-#include "hipdec_kernels.h"
+#include "hipdec_mega.h"
 
 #include <math.h>
 #include <stdio.h>
@@ -9,6 +9,7 @@
 #include <string.h>
 #include <string>
 #include <vector>
+#include <algorithm>
 
 namespace {
 
@@ -49,6 +50,12 @@ struct hipdec_model {
     hipGraphExec_t graphs[V_COUNT] = {};
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     float last_ms = 0.0f;
+    // persistent one-launch-per-token step (hipdec_mega.h)
+    bool mega_ok = false;
+    MegaArgs mega{};
+    int mega_grid = 0;
+    size_t mega_lds = 0;
+    unsigned *d_epochs = nullptr;
     std::vector<void *> allocs;
     std::string err;
 };
@@ -162,9 +169,65 @@ void launch_attn(hipdec_model *m, const DevLayer &L) {
 #undef ATT
 }
 
+template <int WT> void launch_mega_t(hipdec_model *m, const MegaArgs &a) {
+    dim3 grid(m->mega_grid), block(MEGA_THREADS);
+#define MEGA(KVB, HD) hipLaunchKernelGGL((k_mega<WT, KVB, HD>), grid, block, m->mega_lds, m->stream, a)
+    if (m->kvbf16) { if (m->cfg.hd == 64) MEGA(1, 64); else MEGA(1, 128); }
+    else { if (m->cfg.hd == 64) MEGA(0, 64); else MEGA(0, 128); }
+#undef MEGA
+}
+void launch_mega(hipdec_model *m, int do_head, int advance) {
+    MegaArgs a = m->mega;
+    a.do_head = do_head;
+    a.advance = advance;
+    switch (m->wt) {
+        case WT_F32: launch_mega_t<WT_F32>(m, a); break;
+        case WT_BF16: launch_mega_t<WT_BF16>(m, a); break;
+        case WT_FP8: launch_mega_t<WT_FP8>(m, a); break;
+        default: launch_mega_t<WT_INT4>(m, a); break;
+    }
+}
+
+template <int WT> hipError_t mega_set_lds_t(hipdec_model *m) {
+    hipError_t e = hipSuccess;
+#define MEGA_ATTR(KVB, HD)                                                                                       \
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mega<WT, KVB, HD>),                                 \
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)m->mega_lds)
+    if (m->kvbf16) { if (m->cfg.hd == 64) MEGA_ATTR(1, 64); else MEGA_ATTR(1, 128); }
+    else { if (m->cfg.hd == 64) MEGA_ATTR(0, 64); else MEGA_ATTR(0, 128); }
+#undef MEGA_ATTR
+    return e;
+}
+
 void enqueue_step(hipdec_model *m, int variant) {
     const hipdec_config &c = m->cfg;
     const int D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden, V = c.vocab;
+    if (m->mega_ok) {
+        // the whole step in one persistent launch; with 8-bit/4-bit weights the (bf16) LM head
+        // stays a separate GEMV
+        const bool head_inside = (m->wt == m->embed_wt);
+        if (variant == V_X) { launch_mega(m, 0, 1); return; }
+        if (head_inside) {
+            launch_mega(m, 1, 1);
+        } else {
+            launch_mega(m, 0, 0);
+            GemvArgs a{};
+            a.sp = m->d_sp; a.W = m->embed; a.in = m->x_a; a.gamma = m->gfinal; a.out = m->logits; a.rows = V; a.K = D;
+            launch_gemv<EPI_HEAD>(m, m->embed_wt, a);
+            if (variant == V_ARGMAX)
+                hipLaunchKernelGGL(k_head_argmax, dim3(1), dim3(1024), 0, m->stream, m->logits, V, m->d_sp, m->d_ring,
+                                   (int)c.seq);
+            else
+                hipLaunchKernelGGL(k_advance, dim3(1), dim3(1), 0, m->stream, m->d_sp);
+        }
+        if (variant == V_TOPK)
+            hipLaunchKernelGGL(k_head_topk, dim3(m->blocks), dim3(256), 0, m->stream, m->logits, V, m->d_sp,
+                               m->d_topk_vals, m->d_topk_idxs);
+        else if (variant == V_STATS)
+            hipLaunchKernelGGL(k_head_block_stats, dim3(m->blocks), dim3(256), 0, m->stream, m->logits, V, m->d_sp,
+                               m->d_bmax, m->d_bsum);
+        return;
+    }
     if (m->embed_wt == WT_F32)
         hipLaunchKernelGGL(k_embed<WT_F32>, dim3((D + 255) / 256), dim3(256), 0, m->stream, m->embed, m->x_in,
                            m->d_sp, m->x_a, D);
@@ -262,11 +325,27 @@ StepParams base_params(hipdec_model *m, uint32_t token) {
     return p;
 }
 
+// stream sync after a step; a persistent-kernel wait that timed out shows up as an error here
+int sync_checked(hipdec_model *m) {
+    HCHK(hipStreamSynchronize(m->stream));
+    if (m->mega_ok) {
+        unsigned flag = 0;
+        HCHK(hipMemcpy(&flag, m->d_epochs + 2, 4, hipMemcpyDeviceToHost));
+        if (flag) {
+            HCHK(hipMemset(m->d_epochs + 2, 0, 4));
+            m->err = "persistent decode kernel: a wait on another workgroup timed out (grid not co-resident?)";
+            return HIPDEC_ERR_HIP;
+        }
+    }
+    return HIPDEC_OK;
+}
+#define SYNC_CHECKED(m) do { int rc_ = sync_checked(m); if (rc_ != HIPDEC_OK) return rc_; } while (0)
+
 int softcap_out(hipdec_model *m, int start, int n, float cap, float *host_out) {
     hipLaunchKernelGGL(k_softcap_copy, dim3((n + 255) / 256), dim3(256), 0, m->stream, m->logits, m->d_out, start, n, cap);
     HCHK(hipGetLastError());
     HCHK(hipMemcpyAsync(m->h_out, m->d_out, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, m->stream));
-    HCHK(hipStreamSynchronize(m->stream));
+    SYNC_CHECKED(m);
     memcpy(host_out, m->h_out, (size_t)n * sizeof(float));
     return HIPDEC_OK;
 }
@@ -371,6 +450,85 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
     TRY(dalloc(m, &m->d_bmax, (size_t)m->blocks * 4));
     TRY(dalloc(m, &m->d_bsum, (size_t)m->blocks * 4));
     TRY(dalloc(m, &m->d_ring, S * 4));
+    // ---- persistent per-token kernel: exchange buffers, layer table, eligibility
+    {
+        const int G = m->num_cu;
+        const int epl = wt == WT_F32 ? 4 : wt == WT_BF16 ? 8 : wt == WT_FP8 ? 16 : 32;
+        auto tasks_of = [&](size_t rows, size_t K) {
+            size_t pairs = rows / 2, npl = (pairs + G - 1) / G;
+            size_t segs = (K / epl + MEGA_SEG_PIECES - 1) / MEGA_SEG_PIECES;
+            return npl * segs;
+        };
+        const bool head_inside = (wt == m->embed_wt);
+        size_t max_tasks = tasks_of(Q + 2 * KV, D);
+        max_tasks = std::max(max_tasks, tasks_of(D, Q));
+        max_tasks = std::max(max_tasks, tasks_of(2 * H, D));
+        max_tasks = std::max(max_tasks, tasks_of(D, H));
+        if (head_inside) max_tasks = std::max(max_tasks, tasks_of(V, D));
+        const size_t kesz = m->kvbf16 ? 2 : 4;
+        const int slots = MEGA_THREADS / (int)(c.hd / (16 / kesz));
+        int ns_max = G / (int)c.heads;
+        const int ns_lds = (int)((48 * 1024) / ((size_t)c.heads * (c.hd + MEGA_PREC) * 4));
+        if (ns_max > ns_lds) ns_max = ns_lds;
+        if (ns_max > 32) ns_max = 32;
+        const size_t Kmax = std::max(std::max(D, Q), H);
+        const size_t stage_floats = std::max((size_t)c.heads * (ns_max > 0 ? ns_max : 1) * (c.hd + MEGA_PREC),
+                                             (size_t)slots * (c.hd + MEGA_PREC) + 3 * c.hd);
+        const size_t xres_floats = 2 * ((D / 2 + G - 1) / G) + 2;
+        const size_t rope_floats = 2 * (((Q + 2 * KV) / 2 + G - 1) / G) + 2;
+        m->mega_lds = (Kmax + stage_floats + MEGA_PART_MAX + xres_floats + rope_floats) * 4 +
+                      (size_t)MEGA_LPTR * c.nlayers * sizeof(void *);
+        const char *env = getenv("HIPDEC_NO_MEGA");
+        bool want = !(m->opt.flags & HIPDEC_FLAG_NO_MEGA) && !(env && env[0] == '1');
+        bool fits = ns_max >= 1 && 2 * max_tasks <= MEGA_PART_MAX && m->mega_lds <= 160 * 1024 - 2048 &&
+                    (V % 2 == 0) && (int)c.heads <= G;
+        if (want && fits) {
+            std::vector<MegaLayer> hl(c.nlayers);
+            for (uint32_t l = 0; l < c.nlayers; ++l) {
+                const DevLayer &L = m->layers[l];
+                hl[l].w[0] = L.wqkv; hl[l].w[1] = L.wo; hl[l].w[2] = L.w13; hl[l].w[3] = L.w2;
+                hl[l].sc[0] = L.s_qkv; hl[l].sc[1] = L.s_wo; hl[l].sc[2] = L.s_w13; hl[l].sc[3] = L.s_w2;
+                hl[l].g1 = L.g1; hl[l].g2 = L.g2; hl[l].kc = L.kc; hl[l].vc = L.vc;
+            }
+            MegaLayer *dl = nullptr;
+            TRY(dalloc(m, &dl, sizeof(MegaLayer) * c.nlayers));
+            HCHK(hipMemcpy(dl, hl.data(), sizeof(MegaLayer) * c.nlayers, hipMemcpyHostToDevice));
+            MegaArgs &a = m->mega;
+            a.layers = dl; a.embed = m->embed; a.gfinal = m->gfinal; a.x_in = m->x_in;
+            a.X = m->x_a; a.logits = m->logits; a.sp = m->d_sp; a.ring = m->d_ring; a.ring_cap = (int)S;
+            TRY(dalloc(m, &a.QKV, (Q + 2 * KV) * 4));
+            TRY(dalloc(m, &a.PART, (size_t)c.heads * ns_max * (c.hd + MEGA_PREC) * 4));
+            TRY(dalloc(m, &a.X2, D * 4));
+            TRY(dalloc(m, &a.GATE, H * 4));
+            TRY(dalloc(m, &a.CAND, (size_t)G * 8));
+            TRY(dalloc(m, &m->d_epochs, 16));
+            HCHK(hipMemset(a.QKV, 0, (Q + 2 * KV) * 4));
+            HCHK(hipMemset(a.PART, 0, (size_t)c.heads * ns_max * (c.hd + MEGA_PREC) * 4));
+            HCHK(hipMemset(a.X2, 0, D * 4));
+            HCHK(hipMemset(a.GATE, 0, H * 4));
+            HCHK(hipMemset(a.CAND, 0, (size_t)G * 8));
+            HCHK(hipMemset(m->d_epochs, 0, 16));
+            HCHK(hipMemset(m->x_a, 0, D * 4));
+            a.epochs = m->d_epochs;
+            a.D = (int)D; a.Q = (int)Q; a.KV = (int)KV; a.H = (int)H; a.V = (int)V; a.L = (int)c.nlayers;
+            a.hd = (int)c.hd; a.heads = (int)c.heads; a.gqa = c.gqa_ratio ? (int)c.gqa_ratio : 1;
+            a.act = (int)m->opt.ffn_activation; a.ns_max = ns_max; a.seq = (int)S; a.alpha = m->alpha;
+            m->mega_grid = G;
+            hipError_t e;
+            switch (wt) {
+                case WT_F32: e = mega_set_lds_t<WT_F32>(m); break;
+                case WT_BF16: e = mega_set_lds_t<WT_BF16>(m); break;
+                case WT_FP8: e = mega_set_lds_t<WT_FP8>(m); break;
+                default: e = mega_set_lds_t<WT_INT4>(m); break;
+            }
+            m->mega_ok = (e == hipSuccess);
+            if (e != hipSuccess) (void)hipGetLastError();
+        }
+        if (const char *v = getenv("HIPDEC_VERBOSE"))
+            if (v[0] == '1')
+                fprintf(stderr, "hipdec: persistent step kernel %s (wanted %d, fits %d, grid %d, lds %zu B, ns_max %d, tasks %zu)\n",
+                        m->mega_ok ? "on" : "off", (int)want, (int)fits, G, m->mega_lds, ns_max, max_tasks);
+    }
 #undef TRY
     // RoPE table, theta = pos / 10000^(2i/hd) (engine/src/kernels/sdpa_fwd.rs:18-33, lib.rs:1401)
     {
@@ -386,13 +544,15 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
         rc = dalloc(m, &m->rope_sin, S * hp * 4); if (rc) return done(rc);
         HCHK(hipMemcpy(m->rope_cos, ct.data(), S * hp * 4, hipMemcpyHostToDevice));
         HCHK(hipMemcpy(m->rope_sin, st.data(), S * hp * 4, hipMemcpyHostToDevice));
+        m->mega.rope_cos = m->rope_cos;
+        m->mega.rope_sin = m->rope_sin;
     }
     HCHK(hipHostMalloc((void **)&m->h_sp, sizeof(StepParams) * (S + 1), hipHostMallocDefault));
     m->h_out_elems = V > 2 * (size_t)m->blocks * HIPDEC_MAX_GPU_TOPK ? V : 2 * (size_t)m->blocks * HIPDEC_MAX_GPU_TOPK;
     if (m->h_out_elems < S) m->h_out_elems = S;
     if (m->h_out_elems < D) m->h_out_elems = D;
     HCHK(hipHostMalloc((void **)&m->h_out, m->h_out_elems * 4, hipHostMallocDefault));
-    HCHK(hipStreamSynchronize(m->stream));
+    SYNC_CHECKED(m);
     return done(HIPDEC_OK);
 }
 
@@ -470,7 +630,7 @@ int hipdec_seed_layer_cache_from_channel_first(hipdec_model *m, size_t layer_idx
 
 static int read_x(hipdec_model *m, float *x_out) {
     HCHK(hipMemcpyAsync(m->h_out, m->x_a, (size_t)m->cfg.dim * 4, hipMemcpyDeviceToHost, m->stream));
-    HCHK(hipStreamSynchronize(m->stream));
+    SYNC_CHECKED(m);
     memcpy(x_out, m->h_out, (size_t)m->cfg.dim * 4);
     return HIPDEC_OK;
 }
@@ -506,7 +666,7 @@ int hipdec_decode_token_from_id(hipdec_model *m, uint32_t token, float *x_out) {
 
 static int finish_argmax(hipdec_model *m, uint32_t *out_token) {
     HCHK(hipMemcpyAsync(m->h_out, m->d_ring, 4, hipMemcpyDeviceToHost, m->stream));
-    HCHK(hipStreamSynchronize(m->stream));
+    SYNC_CHECKED(m);
     memcpy(out_token, m->h_out, 4);
     m->len += 1;
     return HIPDEC_OK;
@@ -544,7 +704,7 @@ int hipdec_decode_token_topk_from_id(hipdec_model *m, uint32_t token, uint32_t t
     if ((rc = step_with(m, V_TOPK, 0, p))) return rc;
     HCHK(hipMemcpyAsync(m->h_out, m->d_topk_vals, count * 4, hipMemcpyDeviceToHost, m->stream));
     HCHK(hipMemcpyAsync(m->h_out + count, m->d_topk_idxs, count * 4, hipMemcpyDeviceToHost, m->stream));
-    HCHK(hipStreamSynchronize(m->stream));
+    SYNC_CHECKED(m);
     memcpy(out_vals, m->h_out, count * 4);
     memcpy(out_idxs, m->h_out + count, count * 4);
     if (out_count) *out_count = count;
@@ -564,7 +724,7 @@ int hipdec_decode_token_block_stats_from_id(hipdec_model *m, uint32_t token, flo
     if ((rc = step_with(m, V_STATS, 0, p))) return rc;
     HCHK(hipMemcpyAsync(m->h_out, m->d_bmax, B * 4, hipMemcpyDeviceToHost, m->stream));
     HCHK(hipMemcpyAsync(m->h_out + B, m->d_bsum, B * 4, hipMemcpyDeviceToHost, m->stream));
-    HCHK(hipStreamSynchronize(m->stream));
+    SYNC_CHECKED(m);
     memcpy(out_maxes, m->h_out, B * 4);
     memcpy(out_sums, m->h_out + B, B * 4);
     if (out_count) *out_count = B;
@@ -615,7 +775,7 @@ int hipdec_prefill(hipdec_model *m, const uint32_t *ids, size_t n, float softcap
         int rc = softcap_out(m, 0, (int)m->cfg.vocab, softcap, last_logits);
         if (rc) return rc;
     } else {
-        HCHK(hipStreamSynchronize(m->stream));
+        SYNC_CHECKED(m);
     }
     HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
     m->len += n;
@@ -635,7 +795,7 @@ int hipdec_decode_greedy_run(hipdec_model *m, uint32_t token, size_t n_steps, ui
         if ((rc = run_step(m, V_ARGMAX))) return rc;
     HCHK(hipEventRecord(m->ev1, m->stream));
     HCHK(hipMemcpyAsync(m->h_out, m->d_ring, n_steps * 4, hipMemcpyDeviceToHost, m->stream));
-    HCHK(hipStreamSynchronize(m->stream));
+    SYNC_CHECKED(m);
     HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
     memcpy(out_tokens, m->h_out, n_steps * 4);
     m->len += n_steps;
@@ -658,6 +818,32 @@ int hipdec_bytes_per_token(const hipdec_model *m, size_t kv_len, uint64_t *out_b
     uint64_t b = L * per_layer + mat(m->embed_wt, V, D) + wt_row_bytes(m->embed_wt, D) + (2 * L + 1) * D * 4 +
                  L * 2 * (uint64_t)kv_len * KV * kvsz + L * 2 * KV * kvsz;
     *out_bytes = b;
+    return HIPDEC_OK;
+}
+
+int hipdec_debug_step_profile(hipdec_model *m, uint32_t token, uint64_t *out, size_t cap, size_t *out_count) {
+    int rc = check_step(m, token, true);
+    if (rc) return rc;
+    if (!m->mega_ok) return fail(m, HIPDEC_ERR_UNSUPPORTED, "persistent step kernel is off");
+    const size_t n = (size_t)(m->cfg.nlayers + 1) * MEGA_PROF_SLOTS;
+    if (!out || cap < n) return fail(m, HIPDEC_ERR_ARG, "profile buffer too small");
+    unsigned long long *d = nullptr;
+    HCHK(hipMalloc((void **)&d, n * 8));
+    HCHK(hipMemset(d, 0, n * 8));
+    m->h_sp[0] = base_params(m, token);
+    HCHK(hipMemcpyAsync(m->d_sp, &m->h_sp[0], sizeof(StepParams), hipMemcpyHostToDevice, m->stream));
+    m->mega.prof = d;
+    launch_mega(m, m->wt == m->embed_wt ? 1 : 0, 1);
+    m->mega.prof = nullptr;
+    rc = sync_checked(m);
+    if (rc == HIPDEC_OK) {
+        hipError_t e = hipMemcpy(out, d, n * 8, hipMemcpyDeviceToHost);
+        if (e != hipSuccess) { m->err = hipGetErrorString(e); rc = HIPDEC_ERR_HIP; }
+    }
+    (void)hipFree(d);
+    if (rc) return rc;
+    if (out_count) *out_count = n;
+    m->len += 1;
     return HIPDEC_OK;
 }
 

@@ -1,0 +1,668 @@
+// One-launch-per-token decode step for gfx950: a persistent kernel with one workgroup per CU.
+//
+// A batch-1 token step is a chain of ~5 dependent matrix-vector products per layer, each only a
+// few microseconds of HBM streaming on this machine; launched as separate kernels the chain is
+// bound by launch/ramp latency, not by bandwidth.  Here every workgroup stays resident for the
+// whole step and the layers' phases are separated by data exchanges through device memory:
+//
+//  * every activation vector a phase hands to the next one (residual stream, q/k/v of the new
+//    token, attention partials, gate vector) is written with device-coherent stores and carries an
+//    epoch bit in the least significant mantissa bit of each fp32 value; a consumer polls the
+//    values themselves (128-bit device-coherent loads, every 32-bit word self-validating) until
+//    every element shows the expected epoch, so one store->load round trip replaces
+//    "write, fence, signal, wait, fence, read";
+//  * weight addresses do not depend on activations, so each wave requests its next round of
+//    16-byte weight loads before it leaves the current phase: while a workgroup waits for its
+//    inputs the HBM stream for the next phase is already running;
+//  * the phases of all layers run through ONE copy of the polling / streaming / reduction code
+//    (a loop over phases with a small switch per phase), which keeps the loop body inside the
+//    instruction cache.
+//
+// All reductions run in a fixed order, so a step is bit-reproducible.  Every wait is bounded:
+// a workgroup that spins too long raises an abort flag that makes every other workgroup leave too.
+#pragma once
+#include "hipdec_kernels.h"
+
+#define MEGA_THREADS 512
+#define MEGA_WAVES 8
+#define MEGA_DEPTH 4            // tasks per round (16 loads of 16 bytes in flight per lane)
+#define MEGA_SEG_PIECES 128     // 16-byte pieces of one row per task: 2 per lane
+#define MEGA_SPIN_LIMIT (1u << 22)
+#define MEGA_PART_MAX 2048      // floats of per-task partial sums in LDS
+#define MEGA_PREC 4             // attention partial record = HD + 4 floats (acc[HD], max, sum, 0, 0)
+#define MEGA_PROF_SLOTS 32      // timestamps per layer when profiling
+#define MEGA_LPTR 12            // pointers per layer in the LDS copy of the layer table
+
+enum { MK_QKV = 0, MK_WO = 1, MK_W13 = 2, MK_W2 = 3, MK_HEAD = 4, MK_KINDS = 5 };
+
+struct MegaLayer {
+    const void *w[4];        // wqkv, wo, w13, w2 (out-major)
+    const void *sc[4];       // scales (fp8 / int4)
+    const float *g1, *g2;
+    void *kc, *vc;
+};
+
+struct MegaArgs {
+    const MegaLayer *layers;
+    const void *embed;
+    const float *gfinal, *x_in, *rope_cos, *rope_sin;
+    float *X, *QKV, *PART, *X2, *GATE, *logits;      // exchange buffers (device memory, zeroed at creation)
+    unsigned long long *CAND;                        // [grid] argmax candidates
+    StepParams *sp;
+    uint32_t *ring;
+    unsigned *epochs;                                // [0] per-layer exchange counter, [1] head counter, [2] abort
+    unsigned long long *prof;                        // nullable: workgroup 0 writes wall-clock stamps here
+    int ring_cap;
+    int D, Q, KV, H, V, L, hd, heads, gqa, act, do_head, advance, ns_max, seq;
+    float alpha;
+};
+
+struct MegaKind {            // per-workgroup view of one GEMV kind
+    int pieces, segs, pair0, npl, ntasks, K;
+    size_t row_bytes;
+};
+
+typedef unsigned mega_u4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ unsigned ld_u32_coherent(const unsigned *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_stamped(float *p, float v, unsigned par) {
+    unsigned u = (__float_as_uint(v) & ~1u) | par;
+    __hip_atomic_store((unsigned *)p, u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// 128-bit load that bypasses the non-coherent cache levels (sc1: device scope on gfx94x/gfx950)
+__device__ __forceinline__ mega_u4 ld16_coherent(__amdgpu_buffer_rsrc_t r, int byte_off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 16);
+}
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ bool stamp_bad(const mega_u4 &v, unsigned pm) {
+    return (((v.x ^ pm) | (v.y ^ pm) | (v.z ^ pm) | (v.w ^ pm)) & 1u) != 0;
+}
+// one 16-byte slot: reload until all four words carry the expected stamp (bounded)
+__device__ __forceinline__ bool repoll16(mega_u4 &v, __amdgpu_buffer_rsrc_t r, int byte_off, unsigned pm, unsigned *abortf) {
+    unsigned spins = 0;
+    while (stamp_bad(v, pm)) {
+        if ((++spins & 127u) == 0) {
+            if (ld_u32_coherent(abortf)) return false;
+            if (spins > MEGA_SPIN_LIMIT) {
+                __hip_atomic_store(abortf, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                return false;
+            }
+        }
+        v = ld16_coherent(r, byte_off);
+    }
+    return true;
+}
+
+// Polls n stamped floats (n % 4 == 0, src 16-byte aligned) with the whole workgroup into dst (LDS):
+// dst[i] = src[i] * (gamma ? gamma[i] : 1); elements with index in [r0, r0 + nres) are also copied
+// raw to res[i - r0].  Returns this thread's sum of squares of the raw values; *ok = false on
+// abort/timeout.  One copy of this code serves every exchange.
+__device__ __noinline__ float mega_poll_vec(const float *src, int n, unsigned par, unsigned *abortf, float *dst,
+                                            const float *gamma, float *res, int r0, int nres, bool *ok) {
+    const int tid = threadIdx.x;
+    const int n4 = n >> 2;
+    constexpr int NB = 4;
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(src, n * 4);
+    const unsigned pm = par ? 0xffffffffu : 0u;
+    float ss = 0.0f;
+    bool good = true;
+    for (int base = 0; base < n4 && good; base += MEGA_THREADS * NB) {
+        mega_u4 v[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const int i = base + b * MEGA_THREADS + tid;
+            if (i < n4) v[b] = ld16_coherent(r, i * 16);
+        }
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const int i = base + b * MEGA_THREADS + tid;
+            if (i < n4 && good) {
+                good = repoll16(v[b], r, i * 16, pm, abortf);
+                float x[4] = {__uint_as_float(v[b].x), __uint_as_float(v[b].y), __uint_as_float(v[b].z), __uint_as_float(v[b].w)};
+                float4 o;
+                float4 gm = gamma ? *(const float4 *)(gamma + 4 * i) : make_float4(1.0f, 1.0f, 1.0f, 1.0f);
+                o.x = x[0] * gm.x; o.y = x[1] * gm.y; o.z = x[2] * gm.z; o.w = x[3] * gm.w;
+                *(float4 *)(dst + 4 * i) = o;
+                ss += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int j = 4 * i + e - r0;
+                    if (j >= 0 && j < nres) res[j] = x[e];
+                }
+            }
+        }
+    }
+    *ok = good;
+    return ss;
+}
+
+// Sum over the 64 lanes of a wave with data-parallel-primitive moves (no LDS round trips);
+// the total is valid in lane 63.  Fixed order: quads, halves of 8, rows of 16, then the rows.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_get(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v += dpp_get<0xB1, 0xf>(v);      // quad_perm [1,0,3,2]
+    v += dpp_get<0x4E, 0xf>(v);      // quad_perm [2,3,0,1]
+    v += dpp_get<0x141, 0xf>(v);     // row_half_mirror
+    v += dpp_get<0x140, 0xf>(v);     // row_mirror: every lane of a row now holds the row's sum
+    v += dpp_get<0x142, 0xa>(v);     // row_bcast:15 into rows 1 and 3
+    v += dpp_get<0x143, 0xc>(v);     // row_bcast:31 into rows 2 and 3
+    return v;
+}
+// sum over aligned groups of N lanes (8, 16 or 32); every lane of the group receives it
+template <int N> __device__ __forceinline__ float group_sum_dpp(float v) {
+    v += dpp_get<0xB1, 0xf>(v);
+    v += dpp_get<0x4E, 0xf>(v);
+    v += dpp_get<0x141, 0xf>(v);
+    if (N >= 16) v += dpp_get<0x140, 0xf>(v);
+    if (N >= 32) v += __shfl_xor(v, 16, WAVE);
+    return v;
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
+// outstanding global load, which would stall each phase on the weight loads requested for the
+// next one; nothing in this kernel passes data between the waves of a workgroup through global
+// memory, so the LDS-only form is sufficient.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+template <int WT> struct MegaStage {
+    uint4 w[2][2];           // [row of the pair][piece j]
+    uint32_t sc[2][2];       // int4 group scales (bf16 bits)
+};
+
+template <int WT, int KVBF16, int HD>
+__global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
+    constexpr int EPL = WS<WT>::EPL;
+    constexpr int KESZ = KVBF16 ? 2 : 4;
+    constexpr int KEPL = 16 / KESZ;
+    constexpr int LPR = HD / KEPL;               // lanes per cache row
+    constexpr int SLOTS = MEGA_THREADS / LPR;    // cache rows per pass
+    constexpr int PRE = 4;                       // passes prefetched
+    constexpr int REC = HD + MEGA_PREC;          // floats per attention partial record
+    extern __shared__ __align__(16) float smem[];
+    __shared__ MegaKind kinds[MK_KINDS];
+    __shared__ float s_red[MEGA_WAVES];
+    __shared__ int s_bad;                        // set once by any thread whose wait was aborted
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid == 0) s_bad = 0;
+    const int G = gridDim.x, b = blockIdx.x;
+    const int D = a.D, Q = a.Q, KV = a.KV, H = a.H, V = a.V, L = a.L;
+    const int Kmax = max(max(D, Q), H);
+    float *xs = smem;                                        // [Kmax] staged input vector
+    float *stage = xs + Kmax;                                // attention partials / slots
+    const int stage_floats = max(a.heads * a.ns_max * REC, SLOTS * REC + 3 * HD);
+    float *partial = stage + stage_floats;                   // [MEGA_PART_MAX]
+    float *xres = partial + MEGA_PART_MAX;                   // residual inputs of this workgroup's wo/w2 rows
+    float *ropes = xres + 2 * ((D / 2 + G - 1) / G) + 2;     // (cos, sin) of this workgroup's q/k row pairs
+    // weight / scale pointers of every layer, copied once so that computing a load address never
+    // waits on device memory: [L][MEGA_LPTR] = w[4], sc[4], g1, g2, kc, vc
+    const void **lptr = (const void **)(ropes + 2 * (((Q + 2 * KV) / 2 + G - 1) / G) + 2);
+    for (int i = threadIdx.x; i < MEGA_LPTR * L; i += MEGA_THREADS) {
+        const int l = i / MEGA_LPTR, j = i - l * MEGA_LPTR;
+        const MegaLayer &ml = a.layers[l];
+        lptr[i] = j < 4 ? ml.w[j] : j < 8 ? ml.sc[j - 4] : j == 8 ? (const void *)ml.g1 : j == 9 ? (const void *)ml.g2
+                                                         : j == 10 ? (const void *)ml.kc : (const void *)ml.vc;
+    }
+
+    // ---- per-workgroup partition of each GEMV kind
+    if (tid < MK_KINDS) {
+        int rows, K;
+        switch (tid) {
+            case MK_QKV: rows = Q + 2 * KV; K = D; break;
+            case MK_WO: rows = D; K = Q; break;
+            case MK_W13: rows = 2 * H; K = D; break;
+            case MK_W2: rows = D; K = H; break;
+            default: rows = V; K = D; break;
+        }
+        int npairs = rows >> 1, base = npairs / G, rem = npairs % G;
+        MegaKind &k = kinds[tid];
+        k.K = K;
+        k.pieces = K / EPL;
+        k.segs = (k.pieces + MEGA_SEG_PIECES - 1) / MEGA_SEG_PIECES;
+        k.pair0 = b * base + min(b, rem);
+        k.npl = base + (b < rem ? 1 : 0);
+        k.ntasks = k.npl * k.segs;
+        k.row_bytes = WS<WT>::row_bytes(K);
+    }
+    const int pos = a.sp->pos, tok = a.sp->tok, use_x_in = a.sp->use_x_in;
+    const unsigned ep_layer = a.epochs[0], ep_head = a.epochs[1];
+    unsigned *abortf = a.epochs + 2;
+    __syncthreads();
+
+    if (wave == 0) {
+        const MegaKind &k = kinds[MK_QKV];
+        for (int p = lane; p < k.npl; p += 64) {
+            const int row0 = 2 * (k.pair0 + p);
+            const int rr = row0 < Q ? row0 : row0 - Q;
+            const int pi2 = (rr % HD) >> 1;
+            ropes[2 * p] = a.rope_cos[(size_t)pos * (HD / 2) + pi2];
+            ropes[2 * p + 1] = a.rope_sin[(size_t)pos * (HD / 2) + pi2];
+        }
+    }
+
+    unsigned long long *prof = (a.prof && b == 0 && tid == 0) ? a.prof : nullptr;
+    int prof_n = 0;
+    auto mark = [&]() { if (prof) prof[prof_n++] = wall_clock64(); };
+
+    // Tasks of a GEMV phase: (row pair, segment of MEGA_SEG_PIECES pieces).  Wave w owns the local
+    // pairs w, w+8, ... and walks each pair's segments in order, so both the streaming side and the
+    // prefetch side advance with two counters and no division.
+    auto n_mine = [&](int kind) {
+        const int npl = kinds[kind].npl;
+        return npl > wave ? ((npl - wave + MEGA_WAVES - 1) / MEGA_WAVES) * kinds[kind].segs : 0;
+    };
+    const int last_ph = a.do_head ? 4 * L : 4 * L - 1;       // GEMV phase sequence: l*4 + kind, then the head
+
+    // ---- weight prefetch: one register set holding the next round of MEGA_DEPTH tasks
+    MegaStage<WT> st[MEGA_DEPTH];
+    int p_ph = -1, p_left = 0, p_pl = 0, p_sg = 0;           // prefetch cursor
+    int p_pieces = 1, p_segs = 1, p_pair0 = 0, p_kg = 0;
+    size_t p_rb = 0;
+    const char *p_W = (const char *)a.embed;
+    const uint16_t *p_SC = nullptr;
+    // Requests the next round of this wave (a round never mixes phases).  Lanes past the end of
+    // a row and padding tasks re-read a valid address (served from cache) and are ignored when
+    // the round is consumed.
+    auto issue_round = [&]() {
+        while (p_left == 0 && p_ph < last_ph) {
+            ++p_ph;
+            const int kind = p_ph == 4 * L ? MK_HEAD : (p_ph & 3);
+            const MegaKind &k = kinds[kind];
+            p_left = n_mine(kind);
+            p_pieces = k.pieces; p_segs = k.segs; p_pair0 = k.pair0; p_rb = k.row_bytes; p_kg = k.K / 128;
+            p_pl = wave; p_sg = 0;
+            if (kind == MK_HEAD) { p_W = (const char *)a.embed; p_SC = nullptr; }
+            else { p_W = (const char *)lptr[(p_ph >> 2) * MEGA_LPTR + kind]; p_SC = (const uint16_t *)lptr[(p_ph >> 2) * MEGA_LPTR + 4 + kind]; }
+        }
+        // a skipped load is not free if it is issued anyway (it still occupies the address unit),
+        // so padding tasks and lanes past the row end issue nothing
+#pragma unroll
+        for (int s = 0; s < MEGA_DEPTH; ++s) {
+            if (p_left > 0) {
+                const size_t row = (size_t)2 * (p_pair0 + p_pl);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int piece = p_sg * MEGA_SEG_PIECES + j * 64 + lane;
+                    if (piece < p_pieces) {
+#pragma unroll
+                        for (int r = 0; r < 2; ++r) {
+                            st[s].w[r][j] = *(const uint4 *)(p_W + (row + r) * p_rb + (size_t)piece * 16);
+                            if (WT == WT_INT4) st[s].sc[r][j] = p_SC[(row + r) * p_kg + (piece >> 2)];   // 4-bit models keep the head outside
+                        }
+                    }
+                }
+                --p_left;
+                if (++p_sg == p_segs) { p_sg = 0; p_pl += MEGA_WAVES; }
+            }
+        }
+    };
+    issue_round();
+
+    const int wo_row0 = 2 * kinds[MK_WO].pair0, wo_rows = 2 * kinds[MK_WO].npl;   // same partition for w2
+    const int n_att = pos + 1;
+    int NS = (n_att + SLOTS * PRE - 1) / (SLOTS * PRE);
+    NS = max(1, min(NS, a.ns_max));
+    const int chunk = (n_att + NS - 1) / NS;
+    const float att_scale = 1.0f / sqrtf((float)HD);
+    const unsigned par_c = (ep_head + 1u) & 1u;
+
+    for (int ph = 0; ph <= last_ph; ++ph) {
+        const int l = min(ph >> 2, L - 1);
+        const int kind = ph == 4 * L ? MK_HEAD : (ph & 3);
+        const unsigned par = (ep_layer + (unsigned)l + 1u) & 1u;      // stamp of layer l's exchanges
+        const float *g1 = (const float *)lptr[l * MEGA_LPTR + 8], *g2 = (const float *)lptr[l * MEGA_LPTR + 9];
+        void *kcl = (void *)lptr[l * MEGA_LPTR + 10], *vcl = (void *)lptr[l * MEGA_LPTR + 11];
+        if (prof && (kind == MK_QKV || kind == MK_HEAD)) prof_n = (ph >> 2) * MEGA_PROF_SLOTS;
+        mark();
+
+        // ================= attention (before the output projection): item (split, head) on workgroup b
+        if (kind == MK_WO && b < a.heads * NS) {
+            const int sidx = b / a.heads, h = b - sidx * a.heads, g = h / a.gqa;
+            const int t0 = sidx * chunk, t1 = min(n_att, t0 + chunk);
+            float *qs = stage + SLOTS * REC, *kcur = qs + HD, *vcur = kcur + HD;
+            const int sub = tid % LPR, slot = tid / LPR;
+            const char *kb = (const char *)kcl + ((size_t)g * HD + sub * KEPL) * KESZ;
+            const char *vb = (const char *)vcl + ((size_t)g * HD + sub * KEPL) * KESZ;
+            const size_t rowb = (size_t)KV * KESZ;
+            uint4 kr[PRE], vr[PRE];
+            // rows older than the new token are already in the cache: fetch before q arrives
+#pragma unroll
+            for (int i = 0; i < PRE; ++i) {
+                const int t = t0 + slot + i * SLOTS;
+                kr[i] = make_uint4(0, 0, 0, 0); vr[i] = make_uint4(0, 0, 0, 0);
+                if (t < t1 && t != pos) { kr[i] = *(const uint4 *)(kb + (size_t)t * rowb); vr[i] = *(const uint4 *)(vb + (size_t)t * rowb); }
+            }
+            {
+                // q of head h, k and v of kv-head g: three HD-float pieces of the QKV exchange vector
+                bool ok = true;
+                if (tid < 3 * (HD / 4)) {
+                    const int which = tid / (HD / 4), i4 = tid - which * (HD / 4);
+                    const float *src = a.QKV + (which == 0 ? h * HD : which == 1 ? Q + g * HD : Q + KV + g * HD);
+                    float *dst = which == 0 ? qs : which == 1 ? kcur : vcur;
+                    const float mul = which == 0 ? att_scale : 1.0f;
+                    const __amdgpu_buffer_rsrc_t r = make_rsrc(src, HD * 4);
+                    mega_u4 v = ld16_coherent(r, i4 * 16);
+                    ok = repoll16(v, r, i4 * 16, par ? 0xffffffffu : 0u, abortf);
+                    dst[4 * i4] = __uint_as_float(v.x) * mul; dst[4 * i4 + 1] = __uint_as_float(v.y) * mul;
+                    dst[4 * i4 + 2] = __uint_as_float(v.z) * mul; dst[4 * i4 + 3] = __uint_as_float(v.w) * mul;
+                }
+                if (!ok) s_bad = 1;
+                lds_barrier();
+                if (s_bad) return;
+            }
+            mark();
+            float qv[KEPL];
+#pragma unroll
+            for (int e = 0; e < KEPL; ++e) qv[e] = qs[sub * KEPL + e];
+            float m = -1e30f, lsum = 0.0f, acc[KEPL];
+#pragma unroll
+            for (int e = 0; e < KEPL; ++e) acc[e] = 0.0f;
+            for (int tb = t0; tb < t1; tb += SLOTS * PRE) {
+                if (tb != t0) {
+#pragma unroll
+                    for (int i = 0; i < PRE; ++i) {
+                        const int t = tb + slot + i * SLOTS;
+                        if (t < t1 && t != pos) { kr[i] = *(const uint4 *)(kb + (size_t)t * rowb); vr[i] = *(const uint4 *)(vb + (size_t)t * rowb); }
+                    }
+                }
+                // the PRE scores of this pass first (independent chains), then one softmax update
+                float d[PRE];
+#pragma unroll
+                for (int i = 0; i < PRE; ++i) {
+                    const int t = tb + slot + i * SLOTS;
+                    float kf[KEPL];
+                    if (t == pos) {
+#pragma unroll
+                        for (int e = 0; e < KEPL; ++e) kf[e] = kcur[sub * KEPL + e];
+                    } else {
+                        WS<KVBF16 ? WT_BF16 : WT_F32>::decode(kr[i], kf);
+                    }
+                    float dd = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < KEPL; ++e) dd = fmaf(qv[e], kf[e], dd);
+                    d[i] = dd;
+                }
+#pragma unroll
+                for (int i = 0; i < PRE; ++i) d[i] = group_sum_dpp<LPR>(d[i]);
+                float mn = m;
+#pragma unroll
+                for (int i = 0; i < PRE; ++i)
+                    if (tb + slot + i * SLOTS < t1) mn = fmaxf(mn, d[i]);
+                const float corr = __expf(m - mn);
+                lsum *= corr;
+#pragma unroll
+                for (int e = 0; e < KEPL; ++e) acc[e] *= corr;
+                m = mn;
+#pragma unroll
+                for (int i = 0; i < PRE; ++i) {
+                    const int t = tb + slot + i * SLOTS;
+                    if (t < t1) {
+                        float vf[KEPL];
+                        if (t == pos) {
+#pragma unroll
+                            for (int e = 0; e < KEPL; ++e) vf[e] = vcur[sub * KEPL + e];
+                        } else {
+                            WS<KVBF16 ? WT_BF16 : WT_F32>::decode(vr[i], vf);
+                        }
+                        const float p = __expf(d[i] - mn);
+                        lsum += p;
+#pragma unroll
+                        for (int e = 0; e < KEPL; ++e) acc[e] = fmaf(p, vf[e], acc[e]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < KEPL; ++e) stage[slot * REC + sub * KEPL + e] = acc[e];
+            if (sub == 0) { stage[slot * REC + HD] = m; stage[slot * REC + HD + 1] = lsum; }
+            lds_barrier();
+            if (tid < HD) {
+                float M = -1e30f;
+                for (int k2 = 0; k2 < SLOTS; ++k2) M = fmaxf(M, stage[k2 * REC + HD]);
+                float Ls = 0.0f, A = 0.0f;
+                for (int k2 = 0; k2 < SLOTS; ++k2) {
+                    const float w = __expf(stage[k2 * REC + HD] - M);
+                    Ls += stage[k2 * REC + HD + 1] * w;
+                    A += stage[k2 * REC + tid] * w;
+                }
+                float *pp = a.PART + ((size_t)sidx * a.heads + h) * REC;
+                st_stamped(pp + tid, A, par);
+                if (tid < MEGA_PREC) st_stamped(pp + HD + tid, tid == 0 ? M : tid == 1 ? Ls : 0.0f, par);
+            }
+            lds_barrier();
+            mark();
+        }
+
+        // ================= stage this phase's input vector in xs
+        float ss = 0.0f;
+        bool ok = true;
+        if (kind == MK_QKV && l == 0) {
+            for (int i = tid; i < D; i += MEGA_THREADS) {
+                float v;
+                if (use_x_in) v = a.x_in[i];
+                else if (WT == WT_F32) v = ((const float *)a.embed)[(size_t)tok * D + i];
+                else v = bf16_to_f32(((const uint16_t *)a.embed)[(size_t)tok * D + i]);
+                xs[i] = v * g1[i];
+                ss += v * v;
+                if (i >= wo_row0 && i < wo_row0 + wo_rows) xres[i - wo_row0] = v;
+            }
+        } else {
+            // QKV / head: X of the previous layer; WO: attention partials; W13: X2; W2: gate
+            const float *src = kind == MK_WO ? a.PART : kind == MK_W13 ? a.X2 : kind == MK_W2 ? a.GATE : a.X;
+            const int n = kind == MK_WO ? NS * a.heads * REC : kind == MK_W2 ? H : D;
+            const float *gm = kind == MK_QKV ? g1 : kind == MK_W13 ? g2 : kind == MK_HEAD ? a.gfinal : nullptr;
+            float *dst = kind == MK_WO ? stage : xs;
+            const unsigned pr = kind == MK_QKV ? (par ^ 1u) : kind == MK_HEAD ? ((ep_layer + (unsigned)L) & 1u) : par;
+            const int nres = (kind == MK_QKV || kind == MK_W13) ? wo_rows : 0;
+            ss = mega_poll_vec(src, n, pr, abortf, dst, gm, xres, wo_row0, nres, &ok);
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) s_red[wave] = ss;
+        if (!ok) s_bad = 1;
+        lds_barrier();
+        if (s_bad) return;
+        mark();
+        if (kind == MK_WO) {
+            // fold the split partials of every head into the attention output vector
+            const int sstride = a.heads * REC;
+            if (tid < a.heads) {          // per head: the weight of each split, exp(m_s - M) / L
+                float *hp2 = stage + tid * REC;
+                float M = -1e30f;
+                for (int s = 0; s < NS; ++s) M = fmaxf(M, hp2[s * sstride + HD]);
+                float Ls = 0.0f;
+                for (int s = 0; s < NS; ++s) Ls += hp2[s * sstride + HD + 1] * __expf(hp2[s * sstride + HD] - M);
+                const float rl = Ls > 0.0f ? 1.0f / Ls : 0.0f;
+                for (int s = 0; s < NS; ++s) hp2[s * sstride + HD + 2] = __expf(hp2[s * sstride + HD] - M) * rl;
+            }
+            lds_barrier();
+            for (int i = tid; i < Q; i += MEGA_THREADS) {
+                const int h = i / HD, j = i - h * HD;
+                const float *hp2 = stage + h * REC;
+                float A = 0.0f;
+                for (int s = 0; s < NS; ++s) A = fmaf(hp2[s * sstride + j], hp2[s * sstride + HD + 2], A);
+                xs[i] = A;
+            }
+            lds_barrier();
+            mark();
+        }
+        float inv;
+        {
+            float t = 0.0f;
+#pragma unroll
+            for (int w = 0; w < MEGA_WAVES; ++w) t += s_red[w];
+            inv = 1.0f / sqrtf(t * (1.0f / (float)D) + 1e-5f);
+        }
+
+        // ================= stream this workgroup's rows in rounds of MEGA_DEPTH tasks.  The round's
+        // weights were requested one round (or one phase) earlier; once consumed, the registers are
+        // refilled with the next round, which after the last round is the first round of the NEXT
+        // phase.  Overlap inside a phase comes from the eight waves running out of step.  The
+        // 2*MEGA_DEPTH cross-lane sums of a round are reduced together so their latencies overlap.
+        {
+            const MegaKind k = kinds[kind];
+            const int nm = n_mine(kind);
+            int c_pl = wave, c_sg = 0;                        // (local pair, segment) of the next task
+            for (int i = 0; i < nm; i += MEGA_DEPTH) {
+                float acc[MEGA_DEPTH][2];
+                int slot_of[MEGA_DEPTH];                      // index of the task's partial-sum pair in LDS
+#pragma unroll
+                for (int s = 0; s < MEGA_DEPTH; ++s) {
+                    acc[s][0] = 0.0f; acc[s][1] = 0.0f;
+                    slot_of[s] = -1;
+                    if (i + s < nm) {
+                        const int sg = c_sg;
+                        slot_of[s] = c_pl * k.segs + c_sg;
+                        if (++c_sg == k.segs) { c_sg = 0; c_pl += MEGA_WAVES; }
+#pragma unroll
+                        for (int j = 0; j < 2; ++j) {
+                            const int piece = sg * MEGA_SEG_PIECES + j * 64 + lane;
+                            if (piece < k.pieces) {
+                                float xv[EPL];
+#pragma unroll
+                                for (int e = 0; e < EPL; e += 4) {
+                                    float4 tq = *(const float4 *)(xs + piece * EPL + e);
+                                    xv[e] = tq.x; xv[e + 1] = tq.y; xv[e + 2] = tq.z; xv[e + 3] = tq.w;
+                                }
+                                float w0[EPL], w1[EPL];
+                                WS<WT>::decode(st[s].w[0][j], w0);
+                                WS<WT>::decode(st[s].w[1][j], w1);
+                                float p0 = 0.0f, p1 = 0.0f;
+#pragma unroll
+                                for (int e = 0; e < EPL; ++e) { p0 = fmaf(w0[e], xv[e], p0); p1 = fmaf(w1[e], xv[e], p1); }
+                                if (WT == WT_INT4) { p0 *= bf16_to_f32(st[s].sc[0][j]); p1 *= bf16_to_f32(st[s].sc[1][j]); }
+                                acc[s][0] += p0; acc[s][1] += p1;
+                            }
+                        }
+                    }
+                }
+                if (i == 0) mark();
+                issue_round();
+                if (i == 0) mark();
+#pragma unroll
+                for (int s = 0; s < MEGA_DEPTH; ++s) {
+                    acc[s][0] = wave_sum_dpp(acc[s][0]);
+                    acc[s][1] = wave_sum_dpp(acc[s][1]);
+                }
+                if (lane == 63) {
+#pragma unroll
+                    for (int s = 0; s < MEGA_DEPTH; ++s)
+                        if (slot_of[s] >= 0) { partial[2 * slot_of[s]] = acc[s][0]; partial[2 * slot_of[s] + 1] = acc[s][1]; }
+                }
+            }
+        }
+        lds_barrier();
+        mark();
+
+        // ================= finish and publish this workgroup's outputs (wave 0)
+        if (wave == 0) {
+            const MegaKind &k = kinds[kind];
+            const float *fsc = (WT == WT_FP8 && kind != MK_HEAD) ? (const float *)lptr[l * MEGA_LPTR + 4 + kind] : nullptr;
+            float bv = -INFINITY; uint32_t bi = 0x7fffffffu;
+            for (int p = lane; p < k.npl; p += 64) {
+                float s0 = 0.0f, s1 = 0.0f;
+                for (int sg = 0; sg < k.segs; ++sg) { s0 += partial[2 * (p * k.segs + sg)]; s1 += partial[2 * (p * k.segs + sg) + 1]; }
+                const int row0 = 2 * (k.pair0 + p);
+                if (fsc) { s0 *= fsc[row0]; s1 *= fsc[row0 + 1]; }
+                if (kind == MK_QKV) {
+                    s0 *= inv; s1 *= inv;
+                    if (row0 < Q + KV) {            // q and k rows: RoPE on the pair
+                        const float c = ropes[2 * p], s = ropes[2 * p + 1];
+                        const float e = s0 * c - s1 * s, o = s1 * c + s0 * s;
+                        s0 = e; s1 = o;
+                    }
+                    if (row0 >= Q) {                // k and v rows enter the cache (and the exchange) in cache precision
+                        const bool isk = row0 < Q + KV;
+                        const int rr = isk ? row0 - Q : row0 - Q - KV;
+                        void *cache = isk ? kcl : vcl;
+                        if (KVBF16) {
+                            const uint16_t eb = f32_to_bf16_rne(s0), ob = f32_to_bf16_rne(s1);
+                            uint16_t *cp = (uint16_t *)cache + (size_t)pos * KV + rr;
+                            cp[0] = eb; cp[1] = ob;
+                            s0 = bf16_to_f32(eb); s1 = bf16_to_f32(ob);
+                        } else {
+                            float *cp = (float *)cache + (size_t)pos * KV + rr;
+                            cp[0] = s0; cp[1] = s1;
+                        }
+                    }
+                    st_stamped(a.QKV + row0, s0, par);
+                    st_stamped(a.QKV + row0 + 1, s1, par);
+                } else if (kind == MK_WO || kind == MK_W2) {
+                    float *dstv = kind == MK_WO ? a.X2 : a.X;
+                    st_stamped(dstv + row0, xres[2 * p] + a.alpha * s0, par);
+                    st_stamped(dstv + row0 + 1, xres[2 * p + 1] + a.alpha * s1, par);
+                } else if (kind == MK_W13) {
+                    const float h1 = s0 * inv, h3 = s1 * inv;
+                    float gte;
+                    if (a.act == 1) { const float lr = h1 > 0.0f ? h1 : 0.5f * h1; gte = lr * lr * h3; }
+                    else { const float sig = 1.0f / (1.0f + expf(-h1)); gte = h1 * sig * h3; }
+                    st_stamped(a.GATE + (k.pair0 + p), gte, par);
+                } else {
+                    s0 *= inv; s1 *= inv;
+                    a.logits[row0] = s0; a.logits[row0 + 1] = s1;
+                    if (better(s0, (uint32_t)row0, bv, bi)) { bv = s0; bi = (uint32_t)row0; }
+                    if (better(s1, (uint32_t)row0 + 1, bv, bi)) { bv = s1; bi = (uint32_t)row0 + 1; }
+                }
+            }
+            if (kind == MK_HEAD) {
+                wave_argbest(bv, bi);
+                if (lane == 0) {
+                    unsigned long long c = (unsigned long long)__float_as_uint(bv) | ((unsigned long long)(bi | (par_c << 31)) << 32);
+                    __hip_atomic_store(a.CAND + b, c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+        mark();
+    }
+
+    if (!a.do_head) {
+        if (b == 0 && tid == 0) {
+            if (a.advance) a.sp->pos = pos + 1;
+            a.epochs[0] = ep_layer + (unsigned)L;
+        }
+        return;
+    }
+    // ================= workgroup 0 folds the per-workgroup argmax candidates and advances the step state
+    if (b == 0 && wave == 0) {
+        float fv = -INFINITY; uint32_t fi = 0x7fffffffu;
+        bool ok = true;
+        for (int i = lane; i < G && ok; i += 64) {
+            unsigned spins = 0;
+            unsigned long long c;
+            for (;;) {
+                c = __hip_atomic_load(a.CAND + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((((unsigned)(c >> 63)) ^ par_c) == 0) break;
+                if ((++spins & 127u) == 0) {
+                    if (ld_u32_coherent(abortf)) { ok = false; break; }
+                    if (spins > MEGA_SPIN_LIMIT) { __hip_atomic_store(abortf, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); ok = false; break; }
+                }
+            }
+            if (ok) {
+                const float v = __uint_as_float((unsigned)c);
+                const uint32_t ix = (uint32_t)(c >> 32) & 0x7fffffffu;
+                if (better(v, ix, fv, fi)) { fv = v; fi = ix; }
+            }
+        }
+        wave_argbest(fv, fi);
+        const int bad = __any(!ok);
+        if (lane == 0 && !bad) {
+            const int stp = a.sp->step;
+            if (stp >= 0 && stp < a.ring_cap) a.ring[stp] = fi;
+            a.sp->tok = (int)fi;
+            a.sp->pos = pos + 1;
+            a.sp->step = stp + 1;
+            a.epochs[0] = ep_layer + (unsigned)L;
+            a.epochs[1] = ep_head + 1u;
+        }
+        mark();
+    }
+}

@@ -25,7 +25,7 @@ EXPORTS = [
     "hipdec_decode_token_argmax", "hipdec_decode_token_argmax_from_id", "hipdec_decode_token_topk_from_id",
     "hipdec_decode_token_block_stats_from_id", "hipdec_materialize_current_logits_block",
     "hipdec_decode_logits_from_id", "hipdec_prefill", "hipdec_decode_greedy_run", "hipdec_last_device_ms",
-    "hipdec_bytes_per_token", "hipdec_export_weight",
+    "hipdec_bytes_per_token", "hipdec_export_weight", "hipdec_debug_step_profile",
 ]
 
 
@@ -115,6 +115,8 @@ def load_library(path=None):
     lib.hipdec_last_device_ms.argtypes = [C.c_void_p, fp]
     lib.hipdec_bytes_per_token.argtypes = [C.c_void_p, C.c_size_t, C.POINTER(C.c_uint64)]
     lib.hipdec_export_weight.argtypes = [C.c_void_p, C.c_size_t, C.c_uint32, fp, C.c_size_t]
+    lib.hipdec_debug_step_profile.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(C.c_uint64), C.c_size_t,
+                                              C.POINTER(C.c_size_t)]
     if path is None:
         _LIB = lib
     return lib
@@ -264,6 +266,14 @@ class HipDecodeModel:
         b = C.c_uint64()
         self._chk(self._lib.hipdec_bytes_per_token(self._h, kv_len, C.byref(b)))
         return b.value
+
+    def debug_step_profile(self, token):
+        n = (self.cfg.nlayers + 1) * 32
+        out = np.zeros(n, np.uint64)
+        cnt = C.c_size_t()
+        self._chk(self._lib.hipdec_debug_step_profile(self._h, token, out.ctypes.data_as(C.POINTER(C.c_uint64)), n,
+                                                      C.byref(cnt)))
+        return out.reshape(self.cfg.nlayers + 1, 32)
 
     def export_weight(self, layer_idx, which):
         c = self.cfg
