@@ -1,0 +1,189 @@
+// Plain-C view of the host engine for ctypes (tests, benchmark).  Thin: every function forwards
+// to the C++ classes of model.h / decode_context.h / inference.h.
+#include <stdint.h>
+#include <string.h>
+
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "inference.h"
+
+using namespace rustane;
+
+extern "C" {
+
+struct rs_config {
+    uint64_t dim, hidden, heads, kv_heads, hd, seq, nlayers, vocab;
+    uint32_t ffn_activation;
+};
+struct rs_request {
+    uint32_t backend;            // 0 auto, 1 naive, 2 hip
+    uint64_t steps;
+    float temperature;
+    uint64_t top_k, samples, seed;
+};
+struct rs_batch_info {
+    uint32_t mode;               // 0 prefill_only, 1 naive_full_context, 2 kv_cache_hip
+    const char *fallback_reason, *auto_reason;
+    double base_prefill_s, request_prefill_s, prefill_s, total_decode_s, avg_decode_s, total_s;
+    uint64_t n_results;
+};
+struct rs_weights { ModelWeights w; };
+struct rs_session {
+    std::unique_ptr<InferenceSession> s;
+    GenerationBatch last;
+    size_t stream_count = 0;
+};
+
+static ModelConfig to_cfg(const rs_config *c) {
+    return ModelConfig::make(c->dim, c->hidden, c->heads, c->kv_heads, c->hd, c->seq, c->nlayers, c->vocab,
+                             (FfnActivation)c->ffn_activation);
+}
+static void put_err(char *buf, size_t cap, const std::string &e) {
+    if (buf && cap) { strncpy(buf, e.c_str(), cap - 1); buf[cap - 1] = 0; }
+}
+
+uint64_t rs_param_count(const rs_config *c) { return to_cfg(c).param_count(); }
+
+rs_weights *rs_weights_synthetic(const rs_config *c, uint64_t seed, float std, int round_bf16) {
+    rs_weights *w = new rs_weights();
+    w->w = ModelWeights::synthetic(to_cfg(c), seed, std, round_bf16 != 0);
+    return w;
+}
+// layer_ptrs: nlayers * 9 pointers in the order wq wk wv wo w1 w3 w2 gamma1 gamma2 (copied)
+rs_weights *rs_weights_from_arrays(const rs_config *c, const float *const *layer_ptrs, const float *gamma_final,
+                                   const float *embed) {
+    ModelConfig cfg = to_cfg(c);
+    rs_weights *w = new rs_weights();
+    const size_t D = cfg.dim, Q = cfg.q_dim, KV = cfg.kv_dim, H = cfg.hidden;
+    const size_t sizes[9] = {D * Q, D * KV, D * KV, Q * D, D * H, D * H, D * H, D, D};
+    w->w.embed.assign(embed, embed + cfg.vocab * D);
+    w->w.gamma_final.assign(gamma_final, gamma_final + D);
+    w->w.layers.resize(cfg.nlayers);
+    for (size_t l = 0; l < cfg.nlayers; ++l) {
+        LayerWeights &L = w->w.layers[l];
+        std::vector<float> *dst[9] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.w1, &L.w3, &L.w2, &L.gamma1, &L.gamma2};
+        for (int k = 0; k < 9; ++k) dst[k]->assign(layer_ptrs[l * 9 + k], layer_ptrs[l * 9 + k] + sizes[k]);
+    }
+    return w;
+}
+void rs_weights_free(rs_weights *w) { delete w; }
+
+rs_session *rs_session_new(const rs_config *c, const rs_weights *w, const uint32_t *prompt, size_t n, float softcap,
+                           uint32_t weight_dtype, uint32_t kv_dtype, uint32_t flags, char *err, size_t errcap) {
+    SessionOptions o;
+    o.weight_dtype = (WeightDtype)weight_dtype;
+    o.kv_dtype = (KvDtype)kv_dtype;
+    o.flags = flags;
+    std::string e;
+    std::unique_ptr<rs_session> s(new rs_session());
+    s->s.reset(new InferenceSession(to_cfg(c), w->w, std::vector<uint32_t>(prompt, prompt + n), softcap, o, &e));
+    if (!s->s->ok()) { put_err(err, errcap, e); return nullptr; }
+    return s.release();
+}
+void rs_session_free(rs_session *s) { delete s; }
+
+uint64_t rs_session_prompt_len(const rs_session *s) { return s->s->prompt_len(); }
+double rs_session_prefill_s(const rs_session *s) { return s->s->prefill_elapsed(); }
+void rs_session_prompt_logits(const rs_session *s, float *out) {
+    memcpy(out, s->s->prompt_logits().data(), s->s->prompt_logits().size() * sizeof(float));
+}
+
+// stream: 0 = generate_with_suffix; 1 = generate_stream_with_suffix whose callback returns an error
+// once it has been handed `abort_after` tokens (0 = never)
+int rs_session_generate(rs_session *s, const rs_request *r, const uint32_t *suffix, size_t n_suffix, int stream,
+                        uint64_t abort_after, rs_batch_info *info, char *err, size_t errcap) {
+    GenerationRequest req;
+    req.decode_backend = r->backend == 1 ? DecodeBackendRequest::Naive
+                         : r->backend == 2 ? DecodeBackendRequest::Hip : DecodeBackendRequest::Auto;
+    req.steps = r->steps; req.temperature = r->temperature; req.top_k = r->top_k; req.samples = r->samples;
+    req.seed = r->seed;
+    std::vector<uint32_t> suf(suffix, suffix + n_suffix);
+    std::string e;
+    bool ok;
+    s->stream_count = 0;
+    if (stream) {
+        StreamCallback cb = [&](uint32_t, const std::vector<uint32_t> &sampled, const std::vector<uint32_t> &) {
+            s->stream_count = sampled.size();
+            if (abort_after && sampled.size() >= abort_after) return std::string("callback asked to stop");
+            return std::string();
+        };
+        ok = s->s->generate_stream_with_suffix(req, suf, cb, &s->last, &e);
+    } else {
+        ok = s->s->generate_with_suffix(req, suf, &s->last, &e);
+    }
+    if (!ok) { put_err(err, errcap, e); return 1; }
+    const GenerationBatch &b = s->last;
+    info->mode = (uint32_t)b.decode_selection.mode;
+    info->fallback_reason = b.decode_selection.fallback_reason;
+    info->auto_reason = b.decode_selection.auto_reason;
+    info->base_prefill_s = b.base_prefill_elapsed; info->request_prefill_s = b.request_prefill_elapsed;
+    info->prefill_s = b.prefill_elapsed; info->total_decode_s = b.total_decode_elapsed;
+    info->avg_decode_s = b.avg_decode_elapsed; info->total_s = b.total_elapsed;
+    info->n_results = b.results.size();
+    return 0;
+}
+uint64_t rs_session_stream_count(const rs_session *s) { return s->stream_count; }
+uint64_t rs_session_result_len(const rs_session *s, size_t i, int which) {
+    const SampleResult &r = s->last.results[i];
+    return which ? r.generated.size() : r.sampled.size();
+}
+void rs_session_result_copy(const rs_session *s, size_t i, int which, uint32_t *out) {
+    const SampleResult &r = s->last.results[i];
+    const std::vector<uint32_t> &v = which ? r.generated : r.sampled;
+    memcpy(out, v.data(), v.size() * sizeof(uint32_t));
+}
+double rs_session_result_decode_s(const rs_session *s, size_t i) { return s->last.results[i].decode_elapsed; }
+uint64_t rs_session_result_seed(const rs_session *s, size_t i) { return s->last.results[i].seed; }
+
+void rs_select_decode_mode(const rs_config *c, uint32_t requested, uint64_t ctx_len, uint64_t steps, uint32_t *mode,
+                           const char **fallback_reason, const char **auto_reason) {
+    DecodeBackendRequest rq = requested == 1 ? DecodeBackendRequest::Naive
+                              : requested == 2 ? DecodeBackendRequest::Hip : DecodeBackendRequest::Auto;
+    DecodeSelection s = select_decode_mode(to_cfg(c), rq, ctx_len, steps);
+    *mode = (uint32_t)s.mode;
+    *fallback_reason = s.fallback_reason;
+    *auto_reason = s.auto_reason;
+}
+int rs_parse_decode_backend(const char *raw, uint32_t *out) {
+    DecodeBackendRequest r;
+    if (!parse_decode_backend(raw, &r)) return 0;
+    *out = r == DecodeBackendRequest::Naive ? 1 : r == DecodeBackendRequest::Hip ? 2 : 0;
+    return 1;
+}
+
+uint64_t rs_next_u64(uint64_t *state) { return next_u64(state); }
+float rs_next_f32(uint64_t *state) { return next_f32(state); }
+uint32_t rs_sample_next(const float *logits, size_t n, float t, size_t top_k, uint64_t *rng) {
+    return sample_next(logits, n, t, top_k, rng, nullptr);
+}
+uint32_t rs_sample_topk_candidates(const uint32_t *idxs, const float *logits, size_t n, float t, uint64_t *rng) {
+    return sample_topk_candidates(idxs, logits, n, t, rng);
+}
+uint64_t rs_sample_block_from_stats(const float *maxes, const float *sums, size_t n, uint64_t *rng) {
+    return sample_block_from_stats(maxes, sums, n, rng);
+}
+uint64_t rs_sample_softmax_index(const float *logits, size_t n, float t, uint64_t *rng) {
+    return sample_softmax_index(logits, n, t, rng);
+}
+uint32_t rs_sample_block_logits(uint32_t base, const float *logits, size_t n, float t, uint64_t *rng) {
+    return sample_block_logits(base, logits, n, t, rng);
+}
+uint64_t rs_merge_topk_candidates(const float *vals, const uint32_t *idxs, size_t count, size_t top_k, float *out_vals,
+                                  uint32_t *out_idxs) {
+    return merge_topk_candidates(vals, idxs, count, top_k, out_vals, out_idxs);
+}
+int rs_validate_token_ids(const uint32_t *ids, size_t n, size_t vocab, const char *source, char *err, size_t errcap) {
+    std::string e = validate_token_ids(ids, n, vocab, source);
+    put_err(err, errcap, e);
+    return e.empty() ? 0 : 1;
+}
+uint64_t rs_fill_input_window(const uint32_t *generated, size_t n, size_t seq, uint32_t *input) {
+    std::vector<uint32_t> in;
+    size_t cnt = fill_input_window(std::vector<uint32_t>(generated, generated + n), seq, &in);
+    memcpy(input, in.data(), seq * sizeof(uint32_t));
+    return cnt;
+}
+
+}  // extern "C"

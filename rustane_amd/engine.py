@@ -1,0 +1,254 @@
+"""ctypes view of the host engine (librustane_engine.so): the session API of the reference's
+`engine::inference` (crates/engine/src/inference.rs) over the HIP decode backend, its samplers and
+its backend selection.  Names follow the reference."""
+import ctypes as C
+import enum
+
+import numpy as np
+
+from .synth import load_engine
+
+fp = C.POINTER(C.c_float)
+u32p = C.POINTER(C.c_uint32)
+u64p = C.POINTER(C.c_uint64)
+
+AUTO_KV_PARAM_THRESHOLD = 20_000_000       # inference.rs:9
+MAX_GPU_TOPK = 32
+
+
+class DecodeBackendRequest(enum.IntEnum):
+    AUTO = 0
+    NAIVE = 1
+    HIP = 2
+
+
+class DecodeMode(enum.IntEnum):
+    PREFILL_ONLY = 0
+    NAIVE_FULL_CONTEXT = 1
+    KV_CACHE_HIP = 2
+
+
+class RsConfig(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in ("dim", "hidden", "heads", "kv_heads", "hd", "seq", "nlayers", "vocab")] + \
+               [("ffn_activation", C.c_uint32)]
+
+    @classmethod
+    def of(cls, cfg, ffn_activation=0):
+        return cls(cfg.dim, cfg.hidden, cfg.heads, cfg.kv_heads, cfg.hd, cfg.seq, cfg.nlayers, cfg.vocab,
+                   ffn_activation)
+
+
+class RsRequest(C.Structure):
+    _fields_ = [("backend", C.c_uint32), ("steps", C.c_uint64), ("temperature", C.c_float), ("top_k", C.c_uint64),
+                ("samples", C.c_uint64), ("seed", C.c_uint64)]
+
+
+class RsBatchInfo(C.Structure):
+    _fields_ = [("mode", C.c_uint32), ("fallback_reason", C.c_char_p), ("auto_reason", C.c_char_p),
+                ("base_prefill_s", C.c_double), ("request_prefill_s", C.c_double), ("prefill_s", C.c_double),
+                ("total_decode_s", C.c_double), ("avg_decode_s", C.c_double), ("total_s", C.c_double),
+                ("n_results", C.c_uint64)]
+
+
+_bound = False
+
+
+def lib():
+    global _bound
+    L = load_engine()
+    if not _bound:
+        L.rs_param_count.restype = C.c_uint64
+        L.rs_param_count.argtypes = [C.POINTER(RsConfig)]
+        L.rs_weights_synthetic.restype = C.c_void_p
+        L.rs_weights_synthetic.argtypes = [C.POINTER(RsConfig), C.c_uint64, C.c_float, C.c_int]
+        L.rs_weights_from_arrays.restype = C.c_void_p
+        L.rs_weights_from_arrays.argtypes = [C.POINTER(RsConfig), C.POINTER(fp), fp, fp]
+        L.rs_weights_free.argtypes = [C.c_void_p]
+        L.rs_session_new.restype = C.c_void_p
+        L.rs_session_new.argtypes = [C.POINTER(RsConfig), C.c_void_p, u32p, C.c_size_t, C.c_float, C.c_uint32,
+                                     C.c_uint32, C.c_uint32, C.c_char_p, C.c_size_t]
+        L.rs_session_free.argtypes = [C.c_void_p]
+        L.rs_session_prompt_len.restype = C.c_uint64
+        L.rs_session_prompt_len.argtypes = [C.c_void_p]
+        L.rs_session_prefill_s.restype = C.c_double
+        L.rs_session_prefill_s.argtypes = [C.c_void_p]
+        L.rs_session_prompt_logits.argtypes = [C.c_void_p, fp]
+        L.rs_session_generate.argtypes = [C.c_void_p, C.POINTER(RsRequest), u32p, C.c_size_t, C.c_int, C.c_uint64,
+                                          C.POINTER(RsBatchInfo), C.c_char_p, C.c_size_t]
+        L.rs_session_stream_count.restype = C.c_uint64
+        L.rs_session_stream_count.argtypes = [C.c_void_p]
+        L.rs_session_result_len.restype = C.c_uint64
+        L.rs_session_result_len.argtypes = [C.c_void_p, C.c_size_t, C.c_int]
+        L.rs_session_result_copy.argtypes = [C.c_void_p, C.c_size_t, C.c_int, u32p]
+        L.rs_session_result_decode_s.restype = C.c_double
+        L.rs_session_result_decode_s.argtypes = [C.c_void_p, C.c_size_t]
+        L.rs_session_result_seed.restype = C.c_uint64
+        L.rs_session_result_seed.argtypes = [C.c_void_p, C.c_size_t]
+        L.rs_select_decode_mode.argtypes = [C.POINTER(RsConfig), C.c_uint32, C.c_uint64, C.c_uint64, u32p,
+                                            C.POINTER(C.c_char_p), C.POINTER(C.c_char_p)]
+        L.rs_parse_decode_backend.argtypes = [C.c_char_p, u32p]
+        L.rs_next_u64.restype = C.c_uint64
+        L.rs_next_u64.argtypes = [u64p]
+        L.rs_next_f32.restype = C.c_float
+        L.rs_next_f32.argtypes = [u64p]
+        L.rs_sample_next.restype = C.c_uint32
+        L.rs_sample_next.argtypes = [fp, C.c_size_t, C.c_float, C.c_size_t, u64p]
+        L.rs_sample_topk_candidates.restype = C.c_uint32
+        L.rs_sample_topk_candidates.argtypes = [u32p, fp, C.c_size_t, C.c_float, u64p]
+        L.rs_sample_block_from_stats.restype = C.c_uint64
+        L.rs_sample_block_from_stats.argtypes = [fp, fp, C.c_size_t, u64p]
+        L.rs_sample_softmax_index.restype = C.c_uint64
+        L.rs_sample_softmax_index.argtypes = [fp, C.c_size_t, C.c_float, u64p]
+        L.rs_sample_block_logits.restype = C.c_uint32
+        L.rs_sample_block_logits.argtypes = [C.c_uint32, fp, C.c_size_t, C.c_float, u64p]
+        L.rs_merge_topk_candidates.restype = C.c_uint64
+        L.rs_merge_topk_candidates.argtypes = [fp, u32p, C.c_size_t, C.c_size_t, fp, u32p]
+        L.rs_validate_token_ids.argtypes = [u32p, C.c_size_t, C.c_size_t, C.c_char_p, C.c_char_p, C.c_size_t]
+        L.rs_fill_input_window.restype = C.c_uint64
+        L.rs_fill_input_window.argtypes = [u32p, C.c_size_t, C.c_size_t, u32p]
+        _bound = True
+    return L
+
+
+def param_count(cfg):
+    return lib().rs_param_count(C.byref(RsConfig.of(cfg)))
+
+
+def parse_decode_backend(raw):
+    out = C.c_uint32()
+    return DecodeBackendRequest(out.value) if lib().rs_parse_decode_backend(raw.encode(), C.byref(out)) else None
+
+
+class DecodeSelection:
+    def __init__(self, mode, fallback_reason, auto_reason):
+        self.mode = DecodeMode(mode)
+        self.fallback_reason = fallback_reason.decode() if fallback_reason else None
+        self.auto_reason = auto_reason.decode() if auto_reason else None
+
+
+def select_decode_mode(cfg, requested, effective_context_len, steps):
+    """inference.rs:458-528."""
+    mode = C.c_uint32()
+    fb, ar = C.c_char_p(), C.c_char_p()
+    lib().rs_select_decode_mode(C.byref(RsConfig.of(cfg)), int(requested), effective_context_len, steps,
+                                C.byref(mode), C.byref(fb), C.byref(ar))
+    return DecodeSelection(mode.value, fb.value, ar.value)
+
+
+class GenerationRequest:
+    """inference.rs:61-82 (same defaults)."""
+
+    def __init__(self, decode_backend=DecodeBackendRequest.AUTO, steps=32, temperature=0.0, top_k=0, samples=1, seed=1):
+        self.decode_backend, self.steps, self.temperature = decode_backend, steps, temperature
+        self.top_k, self.samples, self.seed = top_k, samples, seed
+
+    def _c(self):
+        return RsRequest(int(self.decode_backend), self.steps, self.temperature, self.top_k, self.samples, self.seed)
+
+
+class SampleResult:
+    def __init__(self, seed, generated, sampled, decode_elapsed):
+        self.seed, self.generated, self.sampled, self.decode_elapsed = seed, generated, sampled, decode_elapsed
+
+
+class GenerationBatch:
+    def __init__(self, info, results):
+        self.decode_selection = DecodeSelection(info.mode, info.fallback_reason, info.auto_reason)
+        self.base_prefill_elapsed = info.base_prefill_s
+        self.request_prefill_elapsed = info.request_prefill_s
+        self.prefill_elapsed = info.prefill_s
+        self.total_decode_elapsed = info.total_decode_s
+        self.avg_decode_elapsed = info.avg_decode_s
+        self.total_elapsed = info.total_s
+        self.results = results
+
+
+class SessionError(RuntimeError):
+    pass
+
+
+class InferenceSession:
+    """inference.rs:107-452 over the HIP backend.  weights: the dict layout of rustane_amd.synth.make_weights."""
+
+    def __init__(self, cfg, weights, prompt_ids, softcap=0.0, weight_dtype=0, kv_dtype=0, flags=0, ffn_activation=0):
+        L = lib()
+        self._L = L
+        self.cfg = cfg
+        rc = RsConfig.of(cfg, ffn_activation)
+        names = ("wq", "wk", "wv", "wo", "w1", "w3", "w2", "gamma1", "gamma2")
+        keep, ptrs = [], (fp * (9 * cfg.nlayers))()
+        for l, lw in enumerate(weights["layers"]):
+            for k, nme in enumerate(names):
+                a = np.ascontiguousarray(lw[nme], np.float32)
+                keep.append(a)
+                ptrs[l * 9 + k] = a.ctypes.data_as(fp)
+        gf = np.ascontiguousarray(weights["gamma_final"], np.float32)
+        em = np.ascontiguousarray(weights["embed"], np.float32)
+        self._w = C.c_void_p(L.rs_weights_from_arrays(C.byref(rc), ptrs, gf.ctypes.data_as(fp), em.ctypes.data_as(fp)))
+        ids = np.ascontiguousarray(prompt_ids, np.uint32)
+        err = C.create_string_buffer(512)
+        self._s = C.c_void_p(L.rs_session_new(C.byref(rc), self._w, ids.ctypes.data_as(u32p), ids.size, softcap,
+                                              int(weight_dtype), int(kv_dtype), flags, err, 512))
+        if not self._s.value:
+            L.rs_weights_free(self._w)
+            self._w = None
+            raise SessionError(err.value.decode())
+
+    def close(self):
+        if getattr(self, "_s", None) and self._s.value:
+            self._L.rs_session_free(self._s)
+            self._s = C.c_void_p()
+        if getattr(self, "_w", None):
+            self._L.rs_weights_free(self._w)
+            self._w = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def prompt_len(self):
+        return int(self._L.rs_session_prompt_len(self._s))
+
+    def prefill_elapsed(self):
+        return self._L.rs_session_prefill_s(self._s)
+
+    def prompt_logits(self):
+        out = np.empty(self.cfg.vocab, np.float32)
+        self._L.rs_session_prompt_logits(self._s, out.ctypes.data_as(fp))
+        return out
+
+    def _run(self, req, suffix, stream, abort_after):
+        suf = np.ascontiguousarray(suffix, np.uint32)
+        info = RsBatchInfo()
+        err = C.create_string_buffer(512)
+        rc = self._L.rs_session_generate(self._s, C.byref(req._c()), suf.ctypes.data_as(u32p), suf.size, int(stream),
+                                         abort_after, C.byref(info), err, 512)
+        if rc:
+            raise SessionError(err.value.decode())
+        results = []
+        for i in range(info.n_results):
+            arrs = []
+            for which in (0, 1):
+                n = self._L.rs_session_result_len(self._s, i, which)
+                a = np.empty(max(n, 1), np.uint32)
+                self._L.rs_session_result_copy(self._s, i, which, a.ctypes.data_as(u32p))
+                arrs.append(a[:n])
+            results.append(SampleResult(self._L.rs_session_result_seed(self._s, i), arrs[1], arrs[0],
+                                        self._L.rs_session_result_decode_s(self._s, i)))
+        return GenerationBatch(info, results)
+
+    def generate(self, req):
+        return self._run(req, (), False, 0)
+
+    def generate_with_suffix(self, req, prompt_suffix):
+        return self._run(req, prompt_suffix, False, 0)
+
+    def generate_stream_with_suffix(self, req, prompt_suffix, abort_after=0):
+        """Streams through a callback inside the engine; it fails the generation once it has seen
+        `abort_after` tokens (0 = never).  stream_count() tells how many tokens it was handed."""
+        return self._run(req, prompt_suffix, True, abort_after)
+
+    def stream_count(self):
+        return int(self._L.rs_session_stream_count(self._s))
