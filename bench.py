@@ -64,6 +64,8 @@ def main():
     ap.add_argument("--workload", default="c2_600m_bf16_bs1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="also run 4 launches of a plain copy kernel of this size (for scaling traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this decode path runs on one GPU (no sharding); --gpus %d is not supported" % args.gpus,
@@ -104,6 +106,9 @@ def main():
         dev_ms += dev.last_device_ms()
         kv_sum += sum(range(n_prompt + 1, n_prompt + n + 1))
         done += n
+    if args.calibrate_copy:
+        from rustane_amd.hipdec import calibration_copy
+        calibration_copy(args.calibrate_copy << 20, 4)
     mean_kv = kv_sum // max(done, 1)
     bytes_per_step = dev.bytes_per_token(mean_kv)
     achieved = bytes_per_step * K / (dev_ms * 1e-3) / 1e9

@@ -155,6 +155,10 @@ int hipdec_export_weight(hipdec_model *m, size_t layer_idx, uint32_t which, floa
  * (100 MHz ticks) workgroup 0 took at its phase boundaries: (nlayers + 1) * 32 slots, unused ones 0. */
 int hipdec_debug_step_profile(hipdec_model *m, uint32_t token, uint64_t *out, size_t cap, size_t *out_count);
 
+/* Diagnostic: `reps` launches of a plain device-to-device copy kernel (k_calib_copy) of `bytes` bytes,
+ * the known-size yardstick that hardware memory-traffic counters are scaled by. */
+int hipdec_debug_calibration_copy(size_t bytes, int reps);
+
 #ifdef __cplusplus
 }
 #endif

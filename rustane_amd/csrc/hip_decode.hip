@@ -821,6 +821,21 @@ int hipdec_bytes_per_token(const hipdec_model *m, size_t kv_len, uint64_t *out_b
     return HIPDEC_OK;
 }
 
+int hipdec_debug_calibration_copy(size_t bytes, int reps) {
+    if (bytes < 16 || reps < 1) return HIPDEC_ERR_ARG;
+    uint4 *src = nullptr, *dst = nullptr;
+    if (hipMalloc((void **)&src, bytes) != hipSuccess) return HIPDEC_ERR_HIP;
+    if (hipMalloc((void **)&dst, bytes) != hipSuccess) { (void)hipFree(src); return HIPDEC_ERR_HIP; }
+    (void)hipMemset(src, 1, bytes);
+    (void)hipMemset(dst, 0, bytes);
+    for (int i = 0; i < reps; ++i)
+        hipLaunchKernelGGL(k_calib_copy, dim3(2048), dim3(256), 0, nullptr, src, dst, bytes / 16);
+    hipError_t e = hipDeviceSynchronize();
+    (void)hipFree(src);
+    (void)hipFree(dst);
+    return e == hipSuccess ? HIPDEC_OK : HIPDEC_ERR_HIP;
+}
+
 int hipdec_debug_step_profile(hipdec_model *m, uint32_t token, uint64_t *out, size_t cap, size_t *out_count) {
     int rc = check_step(m, token, true);
     if (rc) return rc;

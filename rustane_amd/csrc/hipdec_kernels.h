@@ -350,6 +350,13 @@ __global__ void k_softcap_copy(const float *__restrict__ logits, float *__restri
 // bump the position after a step whose head does not do it itself
 __global__ void k_advance(StepParams *sp) { sp->pos = sp->pos + 1; }
 
+// plain device copy of a known size: the yardstick the memory-traffic counters are scaled by
+__global__ __launch_bounds__(256) void k_calib_copy(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n16) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n16; i += stride) dst[i] = src[i];
+}
+
 // ---------------------------------------------------------------- weight load (one-time)
 // [rows][cols] fp32 -> [cols][rows] fp32 through a 32x32 LDS tile
 __global__ void k_transpose_f32(const float *__restrict__ in, float *__restrict__ out, int rows, int cols) {

@@ -25,7 +25,7 @@ EXPORTS = [
     "hipdec_decode_token_argmax", "hipdec_decode_token_argmax_from_id", "hipdec_decode_token_topk_from_id",
     "hipdec_decode_token_block_stats_from_id", "hipdec_materialize_current_logits_block",
     "hipdec_decode_logits_from_id", "hipdec_prefill", "hipdec_decode_greedy_run", "hipdec_last_device_ms",
-    "hipdec_bytes_per_token", "hipdec_export_weight", "hipdec_debug_step_profile",
+    "hipdec_bytes_per_token", "hipdec_export_weight", "hipdec_debug_step_profile", "hipdec_debug_calibration_copy",
 ]
 
 
@@ -117,9 +117,17 @@ def load_library(path=None):
     lib.hipdec_export_weight.argtypes = [C.c_void_p, C.c_size_t, C.c_uint32, fp, C.c_size_t]
     lib.hipdec_debug_step_profile.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(C.c_uint64), C.c_size_t,
                                               C.POINTER(C.c_size_t)]
+    lib.hipdec_debug_calibration_copy.argtypes = [C.c_size_t, C.c_int]
     if path is None:
         _LIB = lib
     return lib
+
+
+def calibration_copy(nbytes, reps=1):
+    """Runs the plain copy kernel (k_calib_copy) of a known size: the yardstick for traffic counters."""
+    rc = load_library().hipdec_debug_calibration_copy(nbytes, reps)
+    if rc != OK:
+        raise HipDecodeError(rc, "calibration copy failed")
 
 
 def _fptr(a):
