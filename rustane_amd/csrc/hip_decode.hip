@@ -467,21 +467,26 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
         if (head_inside) max_tasks = std::max(max_tasks, tasks_of(V, D));
         const size_t kesz = m->kvbf16 ? 2 : 4;
         const int slots = MEGA_THREADS / (int)(c.hd / (16 / kesz));
-        int ns_max = G / (int)c.heads;
-        const int ns_lds = (int)((48 * 1024) / ((size_t)c.heads * (c.hd + MEGA_PREC) * 4));
-        if (ns_max > ns_lds) ns_max = ns_lds;
-        if (ns_max > 32) ns_max = 32;
-        const size_t Kmax = std::max(std::max(D, Q), H);
-        const size_t stage_floats = std::max((size_t)c.heads * (ns_max > 0 ? ns_max : 1) * (c.hd + MEGA_PREC),
-                                             (size_t)slots * (c.hd + MEGA_PREC) + 3 * c.hd);
+        // LDS of the persistent kernel: the staged input vector twice (even phases read D floats, odd
+        // phases max(Q, H)), the attention staging area, the residual inputs twice, the RoPE pairs
+        // and the per-layer pointer table.  The attention split count takes what is left.
+        const size_t lds_cap = 160 * 1024 - 2048;
+        const size_t xs_floats = D + std::max(Q, H);
         const size_t xres_floats = 2 * ((D / 2 + G - 1) / G) + 2;
         const size_t rope_floats = 2 * (((Q + 2 * KV) / 2 + G - 1) / G) + 2;
-        m->mega_lds = (Kmax + stage_floats + MEGA_PART_MAX + xres_floats + rope_floats) * 4 +
-                      (size_t)MEGA_LPTR * c.nlayers * sizeof(void *);
+        const size_t fixed_lds = (xs_floats + 2 * xres_floats + rope_floats) * 4 + (size_t)MEGA_LPTR * c.nlayers * sizeof(void *);
+        const size_t rec_bytes = (size_t)c.heads * (c.hd + MEGA_PREC) * 4;
+        int ns_max = G / (int)c.heads;
+        const int ns_lds = fixed_lds < lds_cap ? (int)((lds_cap - fixed_lds) / rec_bytes) : 0;
+        if (ns_max > ns_lds) ns_max = ns_lds;
+        if (ns_max > 32) ns_max = 32;
+        const size_t stage_floats = std::max((size_t)c.heads * (ns_max > 0 ? ns_max : 1) * (c.hd + MEGA_PREC),
+                                             (size_t)slots * (c.hd + MEGA_PREC) + 3 * c.hd);
+        m->mega_lds = fixed_lds + stage_floats * 4;
         const char *env = getenv("HIPDEC_NO_MEGA");
         bool want = !(m->opt.flags & HIPDEC_FLAG_NO_MEGA) && !(env && env[0] == '1');
-        bool fits = ns_max >= 1 && 2 * max_tasks <= MEGA_PART_MAX && m->mega_lds <= 160 * 1024 - 2048 &&
-                    (V % 2 == 0) && (int)c.heads <= G;
+        bool fits = ns_max >= 1 && m->mega_lds <= lds_cap && (V % 2 == 0) && (int)c.heads <= G &&
+                    D % 4 == 0;
         if (want && fits) {
             std::vector<MegaLayer> hl(c.nlayers);
             for (uint32_t l = 0; l < c.nlayers; ++l) {

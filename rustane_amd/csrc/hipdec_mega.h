@@ -28,7 +28,9 @@
 #define MEGA_DEPTH 4            // tasks per round (16 loads of 16 bytes in flight per lane)
 #define MEGA_SEG_PIECES 128     // 16-byte pieces of one row per task: 2 per lane
 #define MEGA_SPIN_LIMIT (1u << 22)
-#define MEGA_PART_MAX 2048      // floats of per-task partial sums in LDS
+#define MEGA_POLLERS 0          // waves that only wait for and stage exchanged vectors (they request no weights,
+                                // so their loads are never queued behind a round of weight loads)
+#define MEGA_SW (MEGA_WAVES - MEGA_POLLERS)   // waves that stream weight rows
 #define MEGA_PREC 4             // attention partial record = HD + 4 floats (acc[HD], max, sum, 0, 0)
 #define MEGA_PROF_SLOTS 32      // timestamps per layer when profiling
 #define MEGA_LPTR 12            // pointers per layer in the LDS copy of the layer table
@@ -64,6 +66,17 @@ struct MegaKind {            // per-workgroup view of one GEMV kind
 
 typedef unsigned mega_u4 __attribute__((ext_vector_type(4)));
 
+// Loads through pointers that were themselves loaded from a table have an unknown address space
+// and compile to flat loads, which the compiler can only wait for with a full counter drain (and
+// which it also drains before issuing more).  These helpers state that the memory is global.
+__device__ __forceinline__ uint4 ldg_u4(const void *p) {
+    const mega_u4 v = *(const __attribute__((address_space(1))) mega_u4 *)p;
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint16_t ldg_u16(const void *p) {
+    return *(const __attribute__((address_space(1))) uint16_t *)p;
+}
+
 __device__ __forceinline__ unsigned ld_u32_coherent(const unsigned *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -97,34 +110,47 @@ __device__ __forceinline__ bool repoll16(mega_u4 &v, __amdgpu_buffer_rsrc_t r, i
     return true;
 }
 
-// Polls n stamped floats (n % 4 == 0, src 16-byte aligned) with the whole workgroup into dst (LDS):
-// dst[i] = src[i] * (gamma ? gamma[i] : 1); elements with index in [r0, r0 + nres) are also copied
-// raw to res[i - r0].  Returns this thread's sum of squares of the raw values; *ok = false on
-// abort/timeout.  One copy of this code serves every exchange.
+// Polls n stamped floats (n % 4 == 0, src 16-byte aligned) with the polling waves (thread pt of
+// MEGA_PT) into dst (LDS): dst[i] = src[i] * (gamma ? gamma[i] : 1); elements with index in
+// [r0, r0 + nres) are also copied raw to res[i - r0].  Returns this thread's sum of squares of
+// the raw values, or a negative value when the wait was aborted (a flag returned through memory
+// would live in scratch memory).  Kept out of line: inlined, the compiler sinks each poll load next
+// to its use and the loads of one thread stop overlapping.  The price is that a called function
+// starts by waiting for every outstanding load of the wave, the requested weights included; loads
+// return in order, so the polled values could not be seen before those anyway.
+#define MEGA_P0 (MEGA_POLLERS ? MEGA_SW * 64 : 0)   // first polling thread
+#define MEGA_PT (MEGA_THREADS - MEGA_P0)            // polling threads
 __device__ __noinline__ float mega_poll_vec(const float *src, int n, unsigned par, unsigned *abortf, float *dst,
-                                            const float *gamma, float *res, int r0, int nres, bool *ok) {
-    const int tid = threadIdx.x;
+                                            const float *gamma, float *res, int r0, int nres, int pt) {
     const int n4 = n >> 2;
-    constexpr int NB = 4;
+    constexpr int NB = 2048 / MEGA_PT;
     const __amdgpu_buffer_rsrc_t r = make_rsrc(src, n * 4);
     const unsigned pm = par ? 0xffffffffu : 0u;
     float ss = 0.0f;
     bool good = true;
-    for (int base = 0; base < n4 && good; base += MEGA_THREADS * NB) {
-        mega_u4 v[NB];
+    for (int base = 0; base < n4 && good; base += MEGA_PT * NB) {
+        mega_u4 v[NB], g[NB];
+        // the norm weights do not depend on the exchange: request them first so that they are
+        // there when the stamped values arrive
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            const int i = base + b * MEGA_THREADS + tid;
+            const int i = base + b * MEGA_PT + pt;
+            g[b] = mega_u4{0x3f800000u, 0x3f800000u, 0x3f800000u, 0x3f800000u};
+            if (gamma && i < n4) g[b] = *(const __attribute__((address_space(1))) mega_u4 *)(gamma + 4 * i);
+        }
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const int i = base + b * MEGA_PT + pt;
             if (i < n4) v[b] = ld16_coherent(r, i * 16);
         }
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            const int i = base + b * MEGA_THREADS + tid;
+            const int i = base + b * MEGA_PT + pt;
             if (i < n4 && good) {
                 good = repoll16(v[b], r, i * 16, pm, abortf);
                 float x[4] = {__uint_as_float(v[b].x), __uint_as_float(v[b].y), __uint_as_float(v[b].z), __uint_as_float(v[b].w)};
                 float4 o;
-                float4 gm = gamma ? *(const float4 *)(gamma + 4 * i) : make_float4(1.0f, 1.0f, 1.0f, 1.0f);
+                const float4 gm = make_float4(__uint_as_float(g[b].x), __uint_as_float(g[b].y), __uint_as_float(g[b].z), __uint_as_float(g[b].w));
                 o.x = x[0] * gm.x; o.y = x[1] * gm.y; o.z = x[2] * gm.z; o.w = x[3] * gm.w;
                 *(float4 *)(dst + 4 * i) = o;
                 ss += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
@@ -136,8 +162,7 @@ __device__ __noinline__ float mega_poll_vec(const float *src, int n, unsigned pa
             }
         }
     }
-    *ok = good;
-    return ss;
+    return good ? ss : -1.0f;
 }
 
 // Sum over the 64 lanes of a wave with data-parallel-primitive moves (no LDS round trips);
@@ -191,20 +216,25 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     constexpr int REC = HD + MEGA_PREC;          // floats per attention partial record
     extern __shared__ __align__(16) float smem[];
     __shared__ MegaKind kinds[MK_KINDS];
-    __shared__ float s_red[MEGA_WAVES];
-    __shared__ int s_bad;                        // set once by any thread whose wait was aborted
+    __shared__ float s_red[2][MEGA_WAVES];       // per-wave sums of squares, by phase parity
+    __shared__ float s_cand_v[MEGA_WAVES];       // per-wave argmax candidates of the head phase
+    __shared__ uint32_t s_cand_i[MEGA_WAVES];
+    __shared__ int s_bad;                       // set once by any thread whose wait was aborted
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: per-wave bookkeeping stays on the scalar unit
     if (tid == 0) s_bad = 0;
     const int G = gridDim.x, b = blockIdx.x;
     const int D = a.D, Q = a.Q, KV = a.KV, H = a.H, V = a.V, L = a.L;
-    const int Kmax = max(max(D, Q), H);
-    float *xs = smem;                                        // [Kmax] staged input vector
-    float *stage = xs + Kmax;                                // attention partials / slots
+    // the staged input vector is double-buffered by phase parity: a wave may still read phase p's
+    // vector while another already stages phase p+1's.  Even phases (qkv, w13, head) read D floats,
+    // odd phases (wo, w2) max(Q, H).
+    float *xsb = smem;                                       // [D] then [max(Q, H)]
+    float *stage = xsb + D + max(Q, H);                      // attention partials / slots
     const int stage_floats = max(a.heads * a.ns_max * REC, SLOTS * REC + 3 * HD);
-    float *partial = stage + stage_floats;                   // [MEGA_PART_MAX]
-    float *xres = partial + MEGA_PART_MAX;                   // residual inputs of this workgroup's wo/w2 rows
-    float *ropes = xres + 2 * ((D / 2 + G - 1) / G) + 2;     // (cos, sin) of this workgroup's q/k row pairs
+    const int xres_n = 2 * ((D / 2 + G - 1) / G) + 2;
+    float *xresb = stage + stage_floats;                     // [2][xres_n] residual inputs of this workgroup's wo / w2 rows
+    float *ropes = xresb + 2 * xres_n;                       // (cos, sin) of this workgroup's q/k row pairs
     // weight / scale pointers of every layer, copied once so that computing a load address never
     // waits on device memory: [L][MEGA_LPTR] = w[4], sc[4], g1, g2, kc, vc
     const void **lptr = (const void **)(ropes + 2 * (((Q + 2 * KV) / 2 + G - 1) / G) + 2);
@@ -255,12 +285,16 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     int prof_n = 0;
     auto mark = [&]() { if (prof) prof[prof_n++] = wall_clock64(); };
 
-    // Tasks of a GEMV phase: (row pair, segment of MEGA_SEG_PIECES pieces).  Wave w owns the local
-    // pairs w, w+8, ... and walks each pair's segments in order, so both the streaming side and the
-    // prefetch side advance with two counters and no division.
+    // Tasks of a GEMV phase: (row pair, segment of MEGA_SEG_PIECES pieces).  Streaming wave w owns
+    // the local pairs w, w+MEGA_SW, ... and walks each pair's segments in order, so both the
+    // streaming side and the prefetch side advance with two counters and no division.  The last
+    // MEGA_POLLERS waves stream nothing: they wait for and stage the exchanged vectors.
+    const bool streams = wave < MEGA_SW;
+    const int pt = tid - MEGA_P0;                            // index among the polling threads (negative: not one)
+    const bool polls = pt >= 0;
     auto n_mine = [&](int kind) {
         const int npl = kinds[kind].npl;
-        return npl > wave ? ((npl - wave + MEGA_WAVES - 1) / MEGA_WAVES) * kinds[kind].segs : 0;
+        return (streams && npl > wave) ? ((npl - wave + MEGA_SW - 1) / MEGA_SW) * kinds[kind].segs : 0;
     };
     const int last_ph = a.do_head ? 4 * L : 4 * L - 1;       // GEMV phase sequence: l*4 + kind, then the head
 
@@ -297,17 +331,21 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                     if (piece < p_pieces) {
 #pragma unroll
                         for (int r = 0; r < 2; ++r) {
-                            st[s].w[r][j] = *(const uint4 *)(p_W + (row + r) * p_rb + (size_t)piece * 16);
-                            if (WT == WT_INT4) st[s].sc[r][j] = p_SC[(row + r) * p_kg + (piece >> 2)];   // 4-bit models keep the head outside
+                            st[s].w[r][j] = ldg_u4(p_W + (row + r) * p_rb + (size_t)piece * 16);
+                            if (WT == WT_INT4) st[s].sc[r][j] = ldg_u16(p_SC + (row + r) * p_kg + (piece >> 2));   // 4-bit models keep the head outside
                         }
                     }
                 }
                 --p_left;
-                if (++p_sg == p_segs) { p_sg = 0; p_pl += MEGA_WAVES; }
+                if (++p_sg == p_segs) { p_sg = 0; p_pl += MEGA_SW; }
             }
         }
     };
-    issue_round();
+    // Drain the set-up loads here, once: a load still pending on entry to the phase loop would make
+    // the compiler wait for "everything outstanding" at the top of every iteration, which later
+    // includes the weights requested for the phase.
+    __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0)
+    if (streams) issue_round();
 
     const int wo_row0 = 2 * kinds[MK_WO].pair0, wo_rows = 2 * kinds[MK_WO].npl;   // same partition for w2
     const int n_att = pos + 1;
@@ -323,6 +361,11 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         const unsigned par = (ep_layer + (unsigned)l + 1u) & 1u;      // stamp of layer l's exchanges
         const float *g1 = (const float *)lptr[l * MEGA_LPTR + 8], *g2 = (const float *)lptr[l * MEGA_LPTR + 9];
         void *kcl = (void *)lptr[l * MEGA_LPTR + 10], *vcl = (void *)lptr[l * MEGA_LPTR + 11];
+        float *xs = xsb + (ph & 1) * D;
+        // residual inputs: the qkv stage keeps x for the wo epilogue in buffer 0, the w13 stage keeps
+        // x2 for the w2 epilogue in buffer 1
+        float *xres_w = xresb + (kind == MK_W13 ? xres_n : 0);
+        const float *xres_r = xresb + (kind == MK_W2 ? xres_n : 0);
         if (prof && (kind == MK_QKV || kind == MK_HEAD)) prof_n = (ph >> 2) * MEGA_PROF_SLOTS;
         mark();
 
@@ -336,18 +379,23 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             const char *vb = (const char *)vcl + ((size_t)g * HD + sub * KEPL) * KESZ;
             const size_t rowb = (size_t)KV * KESZ;
             uint4 kr[PRE], vr[PRE];
-            // rows older than the new token are already in the cache: fetch before q arrives
 #pragma unroll
-            for (int i = 0; i < PRE; ++i) {
-                const int t = t0 + slot + i * SLOTS;
-                kr[i] = make_uint4(0, 0, 0, 0); vr[i] = make_uint4(0, 0, 0, 0);
-                if (t < t1 && t != pos) { kr[i] = *(const uint4 *)(kb + (size_t)t * rowb); vr[i] = *(const uint4 *)(vb + (size_t)t * rowb); }
-            }
+            for (int i = 0; i < PRE; ++i) { kr[i] = make_uint4(0, 0, 0, 0); vr[i] = make_uint4(0, 0, 0, 0); }
+            // rows older than the new token are already in the cache: the streaming waves fetch
+            // them before q arrives, the polling waves after they have seen it
+            auto kv_first = [&]() {
+#pragma unroll
+                for (int i = 0; i < PRE; ++i) {
+                    const int t = t0 + slot + i * SLOTS;
+                    if (t < t1 && t != pos) { kr[i] = ldg_u4(kb + (size_t)t * rowb); vr[i] = ldg_u4(vb + (size_t)t * rowb); }
+                }
+            };
+            if (streams) kv_first();
             {
                 // q of head h, k and v of kv-head g: three HD-float pieces of the QKV exchange vector
                 bool ok = true;
-                if (tid < 3 * (HD / 4)) {
-                    const int which = tid / (HD / 4), i4 = tid - which * (HD / 4);
+                if (pt >= 0 && pt < 3 * (HD / 4)) {
+                    const int which = pt / (HD / 4), i4 = pt - which * (HD / 4);
                     const float *src = a.QKV + (which == 0 ? h * HD : which == 1 ? Q + g * HD : Q + KV + g * HD);
                     float *dst = which == 0 ? qs : which == 1 ? kcur : vcur;
                     const float mul = which == 0 ? att_scale : 1.0f;
@@ -357,6 +405,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                     dst[4 * i4] = __uint_as_float(v.x) * mul; dst[4 * i4 + 1] = __uint_as_float(v.y) * mul;
                     dst[4 * i4 + 2] = __uint_as_float(v.z) * mul; dst[4 * i4 + 3] = __uint_as_float(v.w) * mul;
                 }
+                if (!streams) kv_first();
                 if (!ok) s_bad = 1;
                 lds_barrier();
                 if (s_bad) return;
@@ -373,7 +422,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
 #pragma unroll
                     for (int i = 0; i < PRE; ++i) {
                         const int t = tb + slot + i * SLOTS;
-                        if (t < t1 && t != pos) { kr[i] = *(const uint4 *)(kb + (size_t)t * rowb); vr[i] = *(const uint4 *)(vb + (size_t)t * rowb); }
+                        if (t < t1 && t != pos) { kr[i] = ldg_u4(kb + (size_t)t * rowb); vr[i] = ldg_u4(vb + (size_t)t * rowb); }
                     }
                 }
                 // the PRE scores of this pass first (independent chains), then one softmax update
@@ -454,7 +503,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                 else v = bf16_to_f32(((const uint16_t *)a.embed)[(size_t)tok * D + i]);
                 xs[i] = v * g1[i];
                 ss += v * v;
-                if (i >= wo_row0 && i < wo_row0 + wo_rows) xres[i - wo_row0] = v;
+                if (i >= wo_row0 && i < wo_row0 + wo_rows) xres_w[i - wo_row0] = v;
             }
         } else {
             // QKV / head: X of the previous layer; WO: attention partials; W13: X2; W2: gate
@@ -464,10 +513,13 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             float *dst = kind == MK_WO ? stage : xs;
             const unsigned pr = kind == MK_QKV ? (par ^ 1u) : kind == MK_HEAD ? ((ep_layer + (unsigned)L) & 1u) : par;
             const int nres = (kind == MK_QKV || kind == MK_W13) ? wo_rows : 0;
-            ss = mega_poll_vec(src, n, pr, abortf, dst, gm, xres, wo_row0, nres, &ok);
+            if (polls) {
+                ss = mega_poll_vec(src, n, pr, abortf, dst, gm, xres_w, wo_row0, nres, pt);
+                if (ss < 0.0f) { ok = false; ss = 0.0f; }
+            }
         }
         ss = wave_sum(ss);
-        if (lane == 0) s_red[wave] = ss;
+        if (lane == 0) s_red[ph & 1][wave] = ss;
         if (!ok) s_bad = 1;
         lds_barrier();
         if (s_bad) return;
@@ -499,30 +551,32 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         {
             float t = 0.0f;
 #pragma unroll
-            for (int w = 0; w < MEGA_WAVES; ++w) t += s_red[w];
+            for (int w = 0; w < MEGA_WAVES; ++w) t += s_red[ph & 1][w];
             inv = 1.0f / sqrtf(t * (1.0f / (float)D) + 1e-5f);
         }
 
         // ================= stream this workgroup's rows in rounds of MEGA_DEPTH tasks.  The round's
         // weights were requested one round (or one phase) earlier; once consumed, the registers are
         // refilled with the next round, which after the last round is the first round of the NEXT
-        // phase.  Overlap inside a phase comes from the eight waves running out of step.  The
-        // 2*MEGA_DEPTH cross-lane sums of a round are reduced together so their latencies overlap.
+        // phase.  A wave owns whole row pairs: it keeps per-lane partial sums across the segments
+        // of a pair, reduces them across lanes once, and its last lane finishes and publishes the
+        // two outputs, so the waves of a workgroup never wait for each other after staging.
+        float bv = -INFINITY; uint32_t bi = 0x7fffffffu;      // head phase: best logit seen by this wave (lane 63)
         {
             const MegaKind k = kinds[kind];
             const int nm = n_mine(kind);
-            int c_pl = wave, c_sg = 0;                        // (local pair, segment) of the next task
+            const float *fsc = (WT == WT_FP8 && kind != MK_HEAD) ? (const float *)lptr[l * MEGA_LPTR + 4 + kind] : nullptr;
+            int c_pl = wave, c_sg = 0;                        // (local pair, segment) of the next task to fold
+            int f_sg = 0;                                     // segment of the next task to multiply
+            float run0 = 0.0f, run1 = 0.0f;                   // per-lane sums of the pair being walked
             for (int i = 0; i < nm; i += MEGA_DEPTH) {
                 float acc[MEGA_DEPTH][2];
-                int slot_of[MEGA_DEPTH];                      // index of the task's partial-sum pair in LDS
 #pragma unroll
                 for (int s = 0; s < MEGA_DEPTH; ++s) {
                     acc[s][0] = 0.0f; acc[s][1] = 0.0f;
-                    slot_of[s] = -1;
                     if (i + s < nm) {
-                        const int sg = c_sg;
-                        slot_of[s] = c_pl * k.segs + c_sg;
-                        if (++c_sg == k.segs) { c_sg = 0; c_pl += MEGA_WAVES; }
+                        const int sg = f_sg;
+                        if (++f_sg == k.segs) f_sg = 0;
 #pragma unroll
                         for (int j = 0; j < 2; ++j) {
                             const int piece = sg * MEGA_SEG_PIECES + j * 64 + lane;
@@ -546,31 +600,20 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                     }
                 }
                 if (i == 0) mark();
-                issue_round();
-                if (i == 0) mark();
+                // inside a phase the next round is requested before the sums are finished (its
+                // latency overlaps them); at the end of a phase the outputs other workgroups wait
+                // for go out first
+                const bool last_round = i + MEGA_DEPTH >= nm;
+                if (!last_round) issue_round();
 #pragma unroll
                 for (int s = 0; s < MEGA_DEPTH; ++s) {
-                    acc[s][0] = wave_sum_dpp(acc[s][0]);
-                    acc[s][1] = wave_sum_dpp(acc[s][1]);
-                }
-                if (lane == 63) {
-#pragma unroll
-                    for (int s = 0; s < MEGA_DEPTH; ++s)
-                        if (slot_of[s] >= 0) { partial[2 * slot_of[s]] = acc[s][0]; partial[2 * slot_of[s] + 1] = acc[s][1]; }
-                }
-            }
-        }
-        lds_barrier();
-        mark();
-
-        // ================= finish and publish this workgroup's outputs (wave 0)
-        if (wave == 0) {
-            const MegaKind &k = kinds[kind];
-            const float *fsc = (WT == WT_FP8 && kind != MK_HEAD) ? (const float *)lptr[l * MEGA_LPTR + 4 + kind] : nullptr;
-            float bv = -INFINITY; uint32_t bi = 0x7fffffffu;
-            for (int p = lane; p < k.npl; p += 64) {
-                float s0 = 0.0f, s1 = 0.0f;
-                for (int sg = 0; sg < k.segs; ++sg) { s0 += partial[2 * (p * k.segs + sg)]; s1 += partial[2 * (p * k.segs + sg) + 1]; }
+                  if (i + s < nm) {
+                    run0 += acc[s][0]; run1 += acc[s][1];
+                    if (++c_sg == k.segs) {
+                      float s0 = wave_sum_dpp(run0), s1 = wave_sum_dpp(run1);
+                      const int p = c_pl;
+                      run0 = 0.0f; run1 = 0.0f; c_sg = 0; c_pl += MEGA_SW;
+                      if (lane == 63) {
                 const int row0 = 2 * (k.pair0 + p);
                 if (fsc) { s0 *= fsc[row0]; s1 *= fsc[row0 + 1]; }
                 if (kind == MK_QKV) {
@@ -598,8 +641,8 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                     st_stamped(a.QKV + row0 + 1, s1, par);
                 } else if (kind == MK_WO || kind == MK_W2) {
                     float *dstv = kind == MK_WO ? a.X2 : a.X;
-                    st_stamped(dstv + row0, xres[2 * p] + a.alpha * s0, par);
-                    st_stamped(dstv + row0 + 1, xres[2 * p + 1] + a.alpha * s1, par);
+                    st_stamped(dstv + row0, xres_r[2 * p] + a.alpha * s0, par);
+                    st_stamped(dstv + row0 + 1, xres_r[2 * p + 1] + a.alpha * s1, par);
                 } else if (kind == MK_W13) {
                     const float h1 = s0 * inv, h3 = s1 * inv;
                     float gte;
@@ -612,11 +655,24 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                     if (better(s0, (uint32_t)row0, bv, bi)) { bv = s0; bi = (uint32_t)row0; }
                     if (better(s1, (uint32_t)row0 + 1, bv, bi)) { bv = s1; bi = (uint32_t)row0 + 1; }
                 }
+                      }
+                    }
+                  }
+                }
+                if (last_round) issue_round();
             }
-            if (kind == MK_HEAD) {
-                wave_argbest(bv, bi);
+        }
+        mark();
+        if (kind == MK_HEAD) {
+            // the eight per-wave candidates meet in LDS; wave 0 publishes the workgroup's best
+            if (lane == 63) { s_cand_v[wave] = bv; s_cand_i[wave] = bi; }
+            lds_barrier();
+            if (wave == 0) {
+                float cv = lane < MEGA_WAVES ? s_cand_v[lane] : -INFINITY;
+                uint32_t ci = lane < MEGA_WAVES ? s_cand_i[lane] : 0x7fffffffu;
+                wave_argbest(cv, ci);
                 if (lane == 0) {
-                    unsigned long long c = (unsigned long long)__float_as_uint(bv) | ((unsigned long long)(bi | (par_c << 31)) << 32);
+                    unsigned long long c = (unsigned long long)__float_as_uint(cv) | ((unsigned long long)(ci | (par_c << 31)) << 32);
                     __hip_atomic_store(a.CAND + b, c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
