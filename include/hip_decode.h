@@ -74,6 +74,8 @@ typedef struct {
 
 #define HIPDEC_FLAG_NO_GRAPH 1u   /* launch kernels eagerly instead of replaying a captured hipGraph */
 #define HIPDEC_FLAG_NO_MEGA 2u    /* one kernel per matrix product instead of the persistent per-token kernel */
+#define HIPDEC_FLAG_PREFILL_STEPS 4u /* hipdec_prefill runs one token step per prompt row instead of the
+                                        chunked matrix-core path (which bf16 and e4m3 weights use by default) */
 
 typedef struct hipdec_model hipdec_model;
 

@@ -2,6 +2,7 @@
 // conversion, hipGraph-captured decode steps and the head variants.
 #include "../../include/hip_decode.h"
 #include "hipdec_mega.h"
+#include "hipdec_prefill.h"
 
 #include <math.h>
 #include <stdio.h>
@@ -23,6 +24,18 @@ struct DevLayer {
 };
 
 std::string g_create_error;
+
+// Workspace of the chunked prompt prefill (hipdec_prefill.h), allocated at the first prefill.
+struct PrefillWork {
+    int rows = 0;                        // chunk capacity in prompt rows
+    uint32_t *ids = nullptr;
+    float *x = nullptr, *x2 = nullptr, *q = nullptr;
+    uint16_t *xn_hi = nullptr, *xn_lo = nullptr, *att_hi = nullptr, *att_lo = nullptr, *gate_hi = nullptr,
+             *gate_lo = nullptr;
+    float *P = nullptr;                  // split-K partial planes
+    size_t P_floats = 0;
+    uint32_t *h_ids = nullptr;           // pinned
+};
 
 }  // namespace
 
@@ -56,6 +69,7 @@ struct hipdec_model {
     int mega_grid = 0;
     size_t mega_lds = 0;
     unsigned *d_epochs = nullptr;
+    PrefillWork pf;
     std::vector<void *> allocs;
     std::string err;
 };
@@ -350,6 +364,149 @@ int softcap_out(hipdec_model *m, int start, int n, float cap, float *host_out) {
     return HIPDEC_OK;
 }
 
+// ---- chunked prompt prefill on the matrix cores (hipdec_prefill.h)
+constexpr int kPrefillMaxRows = 1024;     // prompt rows per chunk
+constexpr int kPrefillMinRows = 8;        // shorter prompts go through the token step
+
+bool prefill_batched_ok(const hipdec_model *m, size_t n) {
+    const hipdec_config &c = m->cfg;
+    if (m->opt.flags & HIPDEC_FLAG_PREFILL_STEPS) return false;
+    if (n < (size_t)kPrefillMinRows) return false;
+    if (m->wt != WT_BF16 && m->wt != WT_FP8) return false;          // fp32 and 4-bit weights: token steps
+    if (c.dim % PF_BK || c.q_dim % PF_BK || c.hidden % PF_BK) return false;
+    if (c.hd != 64 && c.hd != 128) return false;
+    return true;
+}
+
+struct PfSplit { int splits, steps_per_split; };
+PfSplit pf_split_k(const hipdec_model *m, int T, int N, int K) {
+    const int tiles = ((N + PF_BN - 1) / PF_BN) * ((T + PF_BM - 1) / PF_BM);
+    const int nsteps = K / PF_BK;
+    int s = (2 * m->num_cu + tiles - 1) / tiles;
+    s = std::min(s, 8);
+    s = std::min(s, std::max(1, nsteps / 8));
+    s = std::max(s, 1);
+    const int sps = (nsteps + s - 1) / s;
+    return PfSplit{(nsteps + sps - 1) / sps, sps};
+}
+
+int pf_ensure(hipdec_model *m, int T) {
+    const hipdec_config &c = m->cfg;
+    const size_t D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden;
+    PrefillWork &w = m->pf;
+    int rc;
+    if (w.rows < T) {
+        const size_t R = (size_t)std::min<size_t>(kPrefillMaxRows, c.seq);
+        if ((rc = dalloc(m, &w.ids, R * 4))) return rc;
+        if ((rc = dalloc(m, &w.x, R * D * 4))) return rc;
+        if ((rc = dalloc(m, &w.x2, R * D * 4))) return rc;
+        if ((rc = dalloc(m, &w.q, R * Q * 4))) return rc;
+        if ((rc = dalloc(m, &w.xn_hi, R * D * 2))) return rc;
+        if ((rc = dalloc(m, &w.xn_lo, R * D * 2))) return rc;
+        if ((rc = dalloc(m, &w.att_hi, R * Q * 2))) return rc;
+        if ((rc = dalloc(m, &w.att_lo, R * Q * 2))) return rc;
+        if ((rc = dalloc(m, &w.gate_hi, R * H * 2))) return rc;
+        if ((rc = dalloc(m, &w.gate_lo, R * H * 2))) return rc;
+        if (!w.h_ids) HCHK(hipHostMalloc((void **)&w.h_ids, R * 4));
+        w.rows = (int)R;
+    }
+    size_t need = 0;
+    const int dims[4][2] = {{(int)(Q + 2 * KV), (int)D}, {(int)D, (int)Q}, {(int)(2 * H), (int)D}, {(int)D, (int)H}};
+    for (auto &d : dims) need = std::max(need, (size_t)pf_split_k(m, T, d[0], d[1]).splits * T * d[0]);
+    if (need > w.P_floats) {
+        if ((rc = dalloc(m, &w.P, need * 4))) return rc;
+        w.P_floats = need;
+    }
+    return HIPDEC_OK;
+}
+
+// P[z][t][n] = sum over the z-th K slice of A[t][k] * W[n][k]; returns the number of planes
+int pf_gemm(hipdec_model *m, const uint16_t *Ahi, const uint16_t *Alo, const void *W, int T, int N, int K) {
+    const PfSplit sp = pf_split_k(m, T, N, K);
+    PfGemm g{Ahi, Alo, W, m->pf.P, T, N, K, sp.steps_per_split};
+    dim3 grid((N + PF_BN - 1) / PF_BN, (T + PF_BM - 1) / PF_BM, sp.splits), block(256);
+    if (m->wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm<WT_BF16>, grid, block, 0, m->stream, g);
+    else hipLaunchKernelGGL(k_pf_gemm<WT_FP8>, grid, block, 0, m->stream, g);
+    return sp.splits;
+}
+
+// Runs prompt rows ids[0..n) at positions len .. len+n-1 through every layer, chunk by chunk; on
+// return the caches hold their keys and values and *x_last points at the residual stream of the
+// last row (device memory).
+int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float **x_last) {
+    const hipdec_config &c = m->cfg;
+    const int D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden;
+    const int gqa = c.gqa_ratio ? c.gqa_ratio : 1;
+    const float scale = 1.0f / sqrtf((float)c.hd);
+    size_t done = 0;
+    while (done < n) {
+        const int T = (int)std::min<size_t>(n - done, kPrefillMaxRows);
+        const int pos0 = (int)(m->len + done);
+        int rc = pf_ensure(m, T);
+        if (rc) return rc;
+        PrefillWork &w = m->pf;
+        HCHK(hipStreamSynchronize(m->stream));                  // the pinned id buffer is free again
+        memcpy(w.h_ids, ids + done, (size_t)T * 4);
+        HCHK(hipMemcpyAsync(w.ids, w.h_ids, (size_t)T * 4, hipMemcpyHostToDevice, m->stream));
+        if (m->embed_wt == WT_F32)
+            hipLaunchKernelGGL(k_pf_embed_norm<WT_F32>, dim3(T), dim3(256), 0, m->stream, m->embed, w.ids, w.x,
+                               m->layers[0].g1, w.xn_hi, w.xn_lo, D);
+        else
+            hipLaunchKernelGGL(k_pf_embed_norm<WT_BF16>, dim3(T), dim3(256), 0, m->stream, m->embed, w.ids, w.x,
+                               m->layers[0].g1, w.xn_hi, w.xn_lo, D);
+        for (uint32_t l = 0; l < c.nlayers; ++l) {
+            const DevLayer &L = m->layers[l];
+            const bool fp8 = m->wt == WT_FP8;
+            // q/k/v projections, RoPE, cache append
+            int N = Q + 2 * KV;
+            int sp = pf_gemm(m, w.xn_hi, w.xn_lo, L.wqkv, T, N, D);
+            {
+                const size_t items = (size_t)T * (N / 2);
+                dim3 grid((unsigned)((items + 255) / 256)), block(256);
+                if (m->kvbf16)
+                    hipLaunchKernelGGL(k_pf_qkv_epi<1>, grid, block, 0, m->stream, w.P, sp, (size_t)T * N,
+                                       fp8 ? (const float *)L.s_qkv : nullptr, w.q, L.kc, L.vc, m->rope_cos, m->rope_sin,
+                                       T, Q, KV, (int)c.hd, pos0);
+                else
+                    hipLaunchKernelGGL(k_pf_qkv_epi<0>, grid, block, 0, m->stream, w.P, sp, (size_t)T * N,
+                                       fp8 ? (const float *)L.s_qkv : nullptr, w.q, L.kc, L.vc, m->rope_cos, m->rope_sin,
+                                       T, Q, KV, (int)c.hd, pos0);
+            }
+            // causal attention of the chunk's rows over positions 0 .. pos0 + t
+            {
+                dim3 grid((T + 31) / 32, c.heads), block(64);
+#define PFATT(KVB, HD)                                                                                             \
+    hipLaunchKernelGGL((k_pf_attn<KVB, HD>), grid, block, 0, m->stream, w.q, L.kc, L.vc, w.att_hi, w.att_lo, T, Q, KV, \
+                       gqa, pos0, (int)c.seq, scale)
+                if (m->kvbf16) { if (c.hd == 64) PFATT(1, 64); else PFATT(1, 128); }
+                else { if (c.hd == 64) PFATT(0, 64); else PFATT(0, 128); }
+#undef PFATT
+            }
+            // output projection, residual, second norm
+            sp = pf_gemm(m, w.att_hi, w.att_lo, L.wo, T, D, Q);
+            hipLaunchKernelGGL(k_pf_resid_norm, dim3(T), dim3(256), 0, m->stream, w.P, sp, (size_t)T * D,
+                               fp8 ? (const float *)L.s_wo : nullptr, w.x, m->alpha, w.x2, L.g2, w.xn_hi, w.xn_lo, D);
+            // gate/up, activation
+            sp = pf_gemm(m, w.xn_hi, w.xn_lo, L.w13, T, 2 * H, D);
+            {
+                const size_t items = (size_t)T * H;
+                hipLaunchKernelGGL(k_pf_gate_epi, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, m->stream, w.P, sp,
+                                   (size_t)T * 2 * H, fp8 ? (const float *)L.s_w13 : nullptr, w.gate_hi, w.gate_lo, T, H,
+                                   (int)m->opt.ffn_activation);
+            }
+            // down projection, residual, next layer's first norm
+            sp = pf_gemm(m, w.gate_hi, w.gate_lo, L.w2, T, D, H);
+            const float *gnext = l + 1 < c.nlayers ? m->layers[l + 1].g1 : nullptr;
+            hipLaunchKernelGGL(k_pf_resid_norm, dim3(T), dim3(256), 0, m->stream, w.P, sp, (size_t)T * D,
+                               fp8 ? (const float *)L.s_w2 : nullptr, w.x2, m->alpha, w.x, gnext, w.xn_hi, w.xn_lo, D);
+        }
+        HCHK(hipGetLastError());
+        *x_last = w.x + (size_t)(T - 1) * D;
+        done += T;
+    }
+    return HIPDEC_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -363,6 +520,7 @@ void hipdec_destroy(hipdec_model *m) {
     for (void *p : m->allocs) (void)hipFree(p);
     if (m->h_sp) (void)hipHostFree(m->h_sp);
     if (m->h_out) (void)hipHostFree(m->h_out);
+    if (m->pf.h_ids) (void)hipHostFree(m->pf.h_ids);
     if (m->ev0) (void)hipEventDestroy(m->ev0);
     if (m->ev1) (void)hipEventDestroy(m->ev1);
     if (m->stream) (void)hipStreamDestroy(m->stream);
@@ -588,6 +746,7 @@ int hipdec_create(const hipdec_config *cfg, const hipdec_layer_f32 *layers, size
     // HIPDEC_NO_GRAPH=1 in the environment forces eager launches (profilers that cannot follow
     // graph replays still see every kernel)
     if (const char *e = getenv("HIPDEC_NO_GRAPH")) if (e[0] == '1') o.flags |= HIPDEC_FLAG_NO_GRAPH;
+    if (const char *e = getenv("HIPDEC_PREFILL_STEPS")) if (e[0] == '1') o.flags |= HIPDEC_FLAG_PREFILL_STEPS;
     m->opt = o;
     m->wt = (int)o.weight_dtype;
     m->embed_wt = o.weight_dtype == HIPDEC_W_F32 ? WT_F32 : WT_BF16;
@@ -768,12 +927,26 @@ int hipdec_prefill(hipdec_model *m, const uint32_t *ids, size_t n, float softcap
     for (size_t i = 0; i < n; ++i)
         if (ids[i] >= m->cfg.vocab) return fail(m, HIPDEC_ERR_ARG, "token id must fit vocab");
     HCHK(hipEventRecord(m->ev0, m->stream));
-    for (size_t i = 0; i < n; ++i) {
-        StepParams p = base_params(m, ids[i]);
-        p.pos = (int)(m->len + i);
-        int variant = (i + 1 == n && last_logits) ? V_LOGITS : V_X;
-        int rc = step_with(m, variant, i, p);
+    if (prefill_batched_ok(m, n)) {
+        const float *x_last = nullptr;
+        int rc = prefill_batched(m, ids, n, &x_last);
         if (rc) return rc;
+        if (last_logits) {
+            // final RMSNorm + tied LM head on the last row only (full_model.rs:419-428 computes every row)
+            GemvArgs a{};
+            a.sp = m->d_sp; a.W = m->embed; a.in = x_last; a.gamma = m->gfinal; a.out = m->logits;
+            a.rows = (int)m->cfg.vocab; a.K = (int)m->cfg.dim;
+            launch_gemv<EPI_HEAD>(m, m->embed_wt, a);
+            HCHK(hipGetLastError());
+        }
+    } else {
+        for (size_t i = 0; i < n; ++i) {
+            StepParams p = base_params(m, ids[i]);
+            p.pos = (int)(m->len + i);
+            int variant = (i + 1 == n && last_logits) ? V_LOGITS : V_X;
+            int rc = step_with(m, variant, i, p);
+            if (rc) return rc;
+        }
     }
     HCHK(hipEventRecord(m->ev1, m->stream));
     if (last_logits) {

@@ -1,0 +1,423 @@
+// Prompt prefill for gfx950: all prompt rows of a chunk go through each layer together.
+//
+// The reference prefills on the Apple Neural Engine (engine/src/inference.rs:136-144, the graphs of
+// engine/src/kernels/sdpa_fwd.rs, dyn_matmul.rs, ffn_fused.rs); this file is the same arithmetic
+// (crates/engine/src/layer.rs:1287-1431) laid out for matrix cores:
+//
+//  * the four projections of a layer are GEMMs  P[t][n] = sum_k A[t][k] * W[n][k]  on the bf16 MFMA
+//    (32x32x16).  Activations stay fp32-grade: every activation is carried as the sum of two bf16
+//    numbers (hi = rne(v), lo = rne(v - hi), 16 mantissa bits together) and each weight tile is
+//    multiplied by both, so the products lose nothing against the fp32 token path beyond the
+//    accumulation order.  8-bit weights are widened to bf16 (exact) on their way into LDS and their
+//    per-row scale is applied to the finished sum;
+//  * a GEMM may be split along K over blockIdx.z; the partial planes are summed in a fixed order by
+//    the element-wise kernel that consumes them (RoPE + cache write, residual + RMSNorm, gate);
+//  * attention runs on the fp32 MFMA (32x32x2): one wave per (head, 32 query rows) walks the key
+//    tiles with an online softmax, scores kept transposed so that the probabilities are already in
+//    operand layout for the P.V product.
+#pragma once
+#include "hipdec_kernels.h"
+
+typedef __bf16 pf_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float pf_f32x16 __attribute__((ext_vector_type(16)));
+
+#define PF_BM 128           // prompt rows per GEMM workgroup tile
+#define PF_BN 128           // weight rows (output channels) per GEMM workgroup tile
+#define PF_BK 32            // reduction elements per step
+#define PF_LDS_STRIDE 40    // bf16 elements per LDS tile row (80 bytes: 16-byte aligned, spreads rows over banks)
+
+__device__ __forceinline__ void pf_split(float v, uint16_t &hi, uint16_t &lo) {
+    hi = f32_to_bf16_rne(v);
+    lo = f32_to_bf16_rne(v - bf16_to_f32(hi));
+}
+
+__device__ __forceinline__ float pf_block_sum(float v, float *red) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float t = 0.0f;
+    for (int w = 0; w < nw; ++w) t += red[w];
+    return t;
+}
+
+// x[t] = embed[ids[t]] (cpu/embedding.rs:8-16), then RMSNorm with the first layer's gamma1
+// (cpu/rmsnorm.rs:149-183) into the hi/lo activation pair.  One workgroup per prompt row.
+template <int EWT>
+__global__ __launch_bounds__(256) void k_pf_embed_norm(const void *__restrict__ embed, const uint32_t *__restrict__ ids,
+                                                       float *__restrict__ x, const float *__restrict__ gamma,
+                                                       uint16_t *__restrict__ hi, uint16_t *__restrict__ lo, int D) {
+    __shared__ float red[8];
+    const int t = blockIdx.x;
+    const size_t tok = ids[t];
+    float ss = 0.0f;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float v = EWT == WT_F32 ? ((const float *)embed)[tok * D + d] : bf16_to_f32(((const uint16_t *)embed)[tok * D + d]);
+        x[(size_t)t * D + d] = v;
+        ss += v * v;
+    }
+    ss = pf_block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss * (1.0f / (float)D) + 1e-5f);
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        const float v = x[(size_t)t * D + d] * inv * gamma[d];
+        pf_split(v, hi[(size_t)t * D + d], lo[(size_t)t * D + d]);
+    }
+}
+
+// out[t][d] = resid[t][d] + alpha * scale[d] * sum_z P[z][t][d]   (layer.rs:1397-1405, :1300), then
+// RMSNorm(out[t]) * gamma into the hi/lo pair for the next GEMM (gamma == nullptr: no norm output).
+__global__ __launch_bounds__(256) void k_pf_resid_norm(const float *__restrict__ P, int splits, size_t plane,
+                                                       const float *__restrict__ wscale, const float *__restrict__ resid,
+                                                       float alpha, float *__restrict__ out, const float *__restrict__ gamma,
+                                                       uint16_t *__restrict__ hi, uint16_t *__restrict__ lo, int D) {
+    __shared__ float red[8];
+    const int t = blockIdx.x;
+    float ss = 0.0f;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float s = 0.0f;
+        for (int z = 0; z < splits; ++z) s += P[z * plane + (size_t)t * D + d];
+        if (wscale) s *= wscale[d];
+        const float v = resid[(size_t)t * D + d] + alpha * s;
+        out[(size_t)t * D + d] = v;
+        ss += v * v;
+    }
+    if (!gamma) return;
+    ss = pf_block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss * (1.0f / (float)D) + 1e-5f);
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        const float v = out[(size_t)t * D + d] * inv * gamma[d];
+        pf_split(v, hi[(size_t)t * D + d], lo[(size_t)t * D + d]);
+    }
+}
+
+// q/k/v rows of the chunk: sum the split planes, scale (8-bit weights), RoPE on interleaved pairs
+// (kernels/sdpa_fwd.rs:18-33, :258-321), q kept as fp32, k and v written into the caches at
+// positions pos0 + t in cache precision.  One thread per (row, channel pair).
+template <int KVBF16>
+__global__ __launch_bounds__(256) void k_pf_qkv_epi(const float *__restrict__ P, int splits, size_t plane,
+                                                    const float *__restrict__ wscale, float *__restrict__ q,
+                                                    void *__restrict__ kc, void *__restrict__ vc,
+                                                    const float *__restrict__ rope_cos, const float *__restrict__ rope_sin,
+                                                    int T, int Q, int KV, int hd, int pos0) {
+    const int N = Q + 2 * KV, npairs = N >> 1;
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= (size_t)T * npairs) return;
+    const int t = (int)(gid / npairs), p = (int)(gid - (size_t)t * npairs), row0 = 2 * p;
+    float s0 = 0.0f, s1 = 0.0f;
+    for (int z = 0; z < splits; ++z) {
+        const float2 v = *(const float2 *)(P + z * plane + (size_t)t * N + row0);
+        s0 += v.x; s1 += v.y;
+    }
+    if (wscale) { s0 *= wscale[row0]; s1 *= wscale[row0 + 1]; }
+    const int pos = pos0 + t;
+    if (row0 < Q + KV) {
+        const int rr = row0 < Q ? row0 : row0 - Q;
+        const int pi2 = (rr % hd) >> 1;
+        const float c = rope_cos[(size_t)pos * (hd / 2) + pi2], s = rope_sin[(size_t)pos * (hd / 2) + pi2];
+        const float e = s0 * c - s1 * s, o = s1 * c + s0 * s;
+        s0 = e; s1 = o;
+    }
+    if (row0 < Q) {
+        *(float2 *)(q + (size_t)t * Q + row0) = make_float2(s0, s1);
+    } else {
+        const bool isk = row0 < Q + KV;
+        const int rr = isk ? row0 - Q : row0 - Q - KV;
+        void *cache = isk ? kc : vc;
+        if (KVBF16) {
+            uint16_t *cp = (uint16_t *)cache + (size_t)pos * KV + rr;
+            cp[0] = f32_to_bf16_rne(s0); cp[1] = f32_to_bf16_rne(s1);
+        } else {
+            float *cp = (float *)cache + (size_t)pos * KV + rr;
+            cp[0] = s0; cp[1] = s1;
+        }
+    }
+}
+
+// gate[t][j] = act(h1) * h3 with h1 = row 2j and h3 = row 2j+1 of the interleaved gate/up product
+// (kernels/ffn_fused.rs:114-150), written as the hi/lo pair the down projection reads.
+__global__ __launch_bounds__(256) void k_pf_gate_epi(const float *__restrict__ P, int splits, size_t plane,
+                                                     const float *__restrict__ wscale, uint16_t *__restrict__ hi,
+                                                     uint16_t *__restrict__ lo, int T, int H, int act) {
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= (size_t)T * H) return;
+    const int t = (int)(gid / H), j = (int)(gid - (size_t)t * H);
+    float h1 = 0.0f, h3 = 0.0f;
+    for (int z = 0; z < splits; ++z) {
+        const float2 v = *(const float2 *)(P + z * plane + (size_t)t * 2 * H + 2 * j);
+        h1 += v.x; h3 += v.y;
+    }
+    if (wscale) { h1 *= wscale[2 * j]; h3 *= wscale[2 * j + 1]; }
+    float g;
+    if (act == 1) { const float lr = h1 > 0.0f ? h1 : 0.5f * h1; g = lr * lr * h3; }
+    else { const float sig = 1.0f / (1.0f + expf(-h1)); g = h1 * sig * h3; }
+    pf_split(g, hi[gid], lo[gid]);
+}
+
+// ---------------------------------------------------------------- GEMM on the bf16 matrix cores
+struct PfGemm {
+    const uint16_t *Ahi, *Alo;   // activations [T][K], hi and lo parts
+    const void *W;               // weights [N][K], bf16 or e4m3
+    float *P;                    // partial planes [splits][T][N]
+    int T, N, K;
+    int steps_per_split;         // PF_BK-steps of the reduction each blockIdx.z covers
+};
+
+__device__ __forceinline__ pf_bf16x8 pf_frag(const uint16_t *p) {
+    const uint4 v = *(const uint4 *)p;
+    return __builtin_bit_cast(pf_bf16x8, v);
+}
+
+// 256 threads = 4 waves in a 2 x 2 arrangement; each wave owns a 64 (rows) x 64 (channels) tile =
+// 2 x 2 MFMA tiles.  Operand layout of v_mfma_f32_32x32x16_bf16: lane l supplies row (l % 32),
+// reduction elements 8 * (l / 32) .. + 7 of both operands; result register i of lane l is
+// C[8 * (i / 4) + 4 * (l / 32) + i % 4][l % 32].
+template <int WT>
+__global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
+    __shared__ __align__(16) uint16_t sAh[PF_BM * PF_LDS_STRIDE];
+    __shared__ __align__(16) uint16_t sAl[PF_BM * PF_LDS_STRIDE];
+    __shared__ __align__(16) uint16_t sW[PF_BN * PF_LDS_STRIDE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int n0 = blockIdx.x * PF_BN, t0 = blockIdx.y * PF_BM, z = blockIdx.z;
+    const int nsteps = g.K / PF_BK;
+    const int s_begin = z * g.steps_per_split, s_end = min(nsteps, s_begin + g.steps_per_split);
+
+    pf_f32x16 acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.0f;
+
+    // global -> register staging of the next tiles.  Activation tiles: 128 rows x 4 chunks of 8
+    // elements, two chunks per thread for hi and for lo.  Weight tile: bf16 the same; e4m3 128 rows
+    // x 2 chunks of 16 elements, one per thread.  Rows past the end re-read the last valid row;
+    // their results are not stored.
+    uint4 rah[2], ral[2], rw[2];
+    auto gload = [&](int step) {
+        const int k0 = step * PF_BK;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int c = tid + 256 * j, row = c >> 2, kc = c & 3;
+            const size_t ta = (size_t)min(t0 + row, g.T - 1);
+            rah[j] = *(const uint4 *)(g.Ahi + ta * g.K + k0 + kc * 8);
+            ral[j] = *(const uint4 *)(g.Alo + ta * g.K + k0 + kc * 8);
+            if (WT == WT_BF16) {
+                const size_t na = (size_t)min(n0 + row, g.N - 1);
+                rw[j] = *(const uint4 *)((const uint16_t *)g.W + na * g.K + k0 + kc * 8);
+            }
+        }
+        if (WT == WT_FP8) {
+            const int row = tid >> 1, half = tid & 1;
+            const size_t na = (size_t)min(n0 + row, g.N - 1);
+            rw[0] = *(const uint4 *)((const uint8_t *)g.W + na * g.K + k0 + half * 16);
+        }
+    };
+    auto lstore = [&]() {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int c = tid + 256 * j, row = c >> 2, kc = c & 3;
+            *(uint4 *)(sAh + row * PF_LDS_STRIDE + kc * 8) = rah[j];
+            *(uint4 *)(sAl + row * PF_LDS_STRIDE + kc * 8) = ral[j];
+            if (WT == WT_BF16) *(uint4 *)(sW + row * PF_LDS_STRIDE + kc * 8) = rw[j];
+        }
+        if (WT == WT_FP8) {
+            const int row = tid >> 1, half = tid & 1;
+            const uint32_t u[4] = {rw[0].x, rw[0].y, rw[0].z, rw[0].w};
+            uint32_t o[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                auto lo2 = __builtin_amdgcn_cvt_pk_f32_fp8(u[i], false);
+                auto hi2 = __builtin_amdgcn_cvt_pk_f32_fp8(u[i], true);
+                // e4m3 values are exact in bf16: keep the upper halves of the fp32 patterns
+                o[2 * i] = (__float_as_uint(lo2[0]) >> 16) | (__float_as_uint(lo2[1]) & 0xffff0000u);
+                o[2 * i + 1] = (__float_as_uint(hi2[0]) >> 16) | (__float_as_uint(hi2[1]) & 0xffff0000u);
+            }
+            uint16_t *dst = sW + row * PF_LDS_STRIDE + half * 16;
+            *(uint4 *)dst = make_uint4(o[0], o[1], o[2], o[3]);
+            *(uint4 *)(dst + 8) = make_uint4(o[4], o[5], o[6], o[7]);
+        }
+    };
+
+    if (s_begin < s_end) gload(s_begin);
+    for (int step = s_begin; step < s_end; ++step) {
+        __syncthreads();                       // the previous step's operand reads are done
+        lstore();
+        __syncthreads();
+        if (step + 1 < s_end) gload(step + 1); // in flight while this step multiplies
+        const int r = lane & 31, kq = 8 * (lane >> 5);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            pf_bf16x8 b[2], ah[2], al[2];
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) b[nt] = pf_frag(sW + (64 * wn + 32 * nt + r) * PF_LDS_STRIDE + 16 * j + kq);
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+                ah[mt] = pf_frag(sAh + (64 * wm + 32 * mt + r) * PF_LDS_STRIDE + 16 * j + kq);
+                al[mt] = pf_frag(sAl + (64 * wm + 32 * mt + r) * PF_LDS_STRIDE + 16 * j + kq);
+            }
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt) {
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mt], b[nt], acc[mt][nt], 0, 0, 0);
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], b[nt], acc[mt][nt], 0, 0, 0);
+                }
+        }
+    }
+
+    float *Pz = g.P + (size_t)z * g.T * g.N;
+    const int r = lane & 31, gq = lane >> 5;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+            const int n = n0 + 64 * wn + 32 * nt + r;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int t = t0 + 64 * wm + 32 * mt + 8 * (i >> 2) + 4 * gq + (i & 3);
+                if (t < g.T && n < g.N) Pz[(size_t)t * g.N + n] = acc[mt][nt][i];
+            }
+        }
+}
+
+// ---------------------------------------------------------------- causal attention over the chunk
+// One wave per (32 query rows, head).  S^T = K . Q^T on the fp32 MFMA (32x32x2: lane l supplies
+// row l % 32 and reduction element l / 32 of both operands), so lane (q = l % 32, g = l / 32) ends
+// up with the scores of query q against keys 8 * (i / 4) + 4 * g + i % 4, i = 0..15 -- exactly the
+// operand layout P needs in O += P . V.  Softmax statistics are per lane (+ one exchange with lane
+// l ^ 32); the rescale factors of the O rows travel through LDS.
+// (kernels/sdpa_fwd.rs:325-354: softmax(q . k^T / sqrt(hd) + causal mask) . v)
+template <int KVBF16, int HD>
+__global__ __launch_bounds__(64) void k_pf_attn(const float *__restrict__ q, const void *__restrict__ kc,
+                                                const void *__restrict__ vc, uint16_t *__restrict__ ohi,
+                                                uint16_t *__restrict__ olo, int T, int Q, int KV, int gqa, int pos0,
+                                                int seq, float scale) {
+    constexpr int HK = HD / 2;                 // reduction elements per lane group in S
+    constexpr int NT = HD / 32;                // 32-wide column tiles of O
+    constexpr int VS = HD + 8;                 // LDS row stride of the V tile (floats)
+    constexpr int KESZ = KVBF16 ? 2 : 4;
+    constexpr int CPR = HD * KESZ / 16;        // 16-byte chunks per cache row
+    constexpr int KCH = HK * KESZ / 16;        // chunks of this lane's half row
+    constexpr int VCH = 32 * CPR / 64;         // V-tile chunks per lane
+    __shared__ __align__(16) float sV[32 * VS];
+    __shared__ __align__(16) float sfac[32];
+    const int lane = threadIdx.x, r = lane & 31, g = lane >> 5;
+    const int q0 = blockIdx.x * 32, h = blockIdx.y, kvh = h / gqa;
+    const int tq = min(q0 + r, T - 1);
+    const int qpos = pos0 + q0 + r;            // position of this lane's query row
+
+    float qf[HK];
+    {
+        const float *qp = q + (size_t)tq * Q + h * HD + HK * g;
+#pragma unroll
+        for (int s = 0; s < HK; s += 4) {
+            const float4 v = *(const float4 *)(qp + s);
+            qf[s] = v.x * scale; qf[s + 1] = v.y * scale; qf[s + 2] = v.z * scale; qf[s + 3] = v.w * scale;
+        }
+    }
+    pf_f32x16 accO[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) accO[nt][i] = 0.0f;
+    float m_run = -1e30f, l_run = 0.0f;
+
+    const int last_pos = pos0 + min(q0 + 31, T - 1);
+    const char *kbase = (const char *)kc + (size_t)kvh * HD * KESZ;
+    const char *vbase = (const char *)vc + (size_t)kvh * HD * KESZ;
+    const size_t rowb = (size_t)KV * KESZ;
+    for (int kt0 = 0; kt0 <= last_pos; kt0 += 32) {
+        // this lane's key row (its half of the head dimension) and its share of the V tile
+        uint4 kr[KCH], vr[VCH];
+        {
+            const int krow = min(kt0 + r, seq - 1);
+            const char *kp = kbase + (size_t)krow * rowb + (size_t)g * HK * KESZ;
+#pragma unroll
+            for (int c = 0; c < KCH; ++c) kr[c] = *(const uint4 *)(kp + c * 16);
+#pragma unroll
+            for (int c = 0; c < VCH; ++c) {
+                const int ch = lane + 64 * c, vrow = min(kt0 + ch / CPR, seq - 1), cc = ch % CPR;
+                vr[c] = *(const uint4 *)(vbase + (size_t)vrow * rowb + cc * 16);
+            }
+        }
+        pf_f32x16 accS;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) accS[i] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < KCH; ++c) {
+            float kf[16 / KESZ];
+            WS<KVBF16 ? WT_BF16 : WT_F32>::decode(kr[c], kf);
+#pragma unroll
+            for (int e = 0; e < 16 / KESZ; ++e)
+                accS = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[c * (16 / KESZ) + e], accS, 0, 0, 0);
+        }
+        __syncthreads();                       // the previous tile's V reads are done
+#pragma unroll
+        for (int c = 0; c < VCH; ++c) {
+            const int ch = lane + 64 * c, vrow = ch / CPR, cc = ch % CPR;
+            float vf[16 / KESZ];
+            WS<KVBF16 ? WT_BF16 : WT_F32>::decode(vr[c], vf);
+            float *dst = sV + vrow * VS + cc * (16 / KESZ);
+#pragma unroll
+            for (int e = 0; e < 16 / KESZ; e += 4) *(float4 *)(dst + e) = make_float4(vf[e], vf[e + 1], vf[e + 2], vf[e + 3]);
+        }
+        // online softmax for query row r over this tile's 32 keys (16 here, 16 in lane r ^ 32)
+        float tmax = -1e30f;
+        bool valid[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int kpos = kt0 + 8 * (i >> 2) + 4 * g + (i & 3);
+            valid[i] = kpos <= qpos;
+            if (valid[i]) tmax = fmaxf(tmax, accS[i]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m_run, tmax);
+        const float corr = __expf(m_run - m_new);
+        float psum = 0.0f;
+        float p[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            p[i] = valid[i] ? __expf(accS[i] - m_new) : 0.0f;
+            psum += p[i];
+        }
+        psum += __shfl_xor(psum, 32, 64);
+        l_run = l_run * corr + psum;
+        m_run = m_new;
+        if (g == 0) sfac[r] = corr;
+        __syncthreads();                       // V tile and rescale factors are in LDS
+#pragma unroll
+        for (int j4 = 0; j4 < 4; ++j4) {
+            const float4 f = *(const float4 *)(sfac + 8 * j4 + 4 * g);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                accO[nt][4 * j4] *= f.x; accO[nt][4 * j4 + 1] *= f.y;
+                accO[nt][4 * j4 + 2] *= f.z; accO[nt][4 * j4 + 3] *= f.w;
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+            const int key = 8 * (s >> 2) + 4 * g + (s & 3);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+                accO[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(p[s], sV[key * VS + 32 * nt + r], accO[nt], 0, 0, 0);
+        }
+    }
+    __syncthreads();
+    if (g == 0) sfac[r] = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int qi = 8 * (i >> 2) + 4 * g + (i & 3), t = q0 + qi;
+        const float f = sfac[qi];
+        if (t < T) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const size_t o = (size_t)t * Q + h * HD + 32 * nt + r;
+                pf_split(accO[nt][i] * f, ohi[o], olo[o]);
+            }
+        }
+    }
+}

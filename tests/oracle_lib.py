@@ -286,3 +286,36 @@ class Rng:
     @property
     def ref(self):
         return C.byref(self.s)
+
+
+def dequantised_weights(cfg, weights, kind):
+    """The fp32 weight set a quantised model actually multiplies with: every linear matrix goes
+    through the oracle's quantise->de-quantise round trip (kind: "fp8" = e4m3 with a per-output-row
+    scale, "int4" = 4-bit groups of 128 along the reduction axis); embeddings and norms stay as they
+    are.  Also returns the out-major de-quantised matrices per layer (for bit-exact storage checks)."""
+    L = lib()
+    D, Q, KV, H = cfg.dim, cfg.q_dim, cfg.kv_dim, cfg.hidden
+
+    def out_major(a, rows_in, cols_in, transpose):
+        a = f32(a).reshape(rows_in, cols_in)
+        return np.ascontiguousarray(a.T) if transpose else a
+
+    def dq(m):
+        m = np.ascontiguousarray(m, np.float32)
+        out = np.empty_like(m)
+        fn = L.orc_quant_fp8_rows if kind == "fp8" else L.orc_quant_int4_g128
+        fn(P(m), m.shape[0], m.shape[1], None, None, P(out))
+        return out
+
+    shapes = dict(wq=(D, Q, True), wk=(D, KV, True), wv=(D, KV, True), wo=(Q, D, True), w1=(D, H, True),
+                  w3=(D, H, True), w2=(D, H, False))
+    out = {"embed": weights["embed"], "gamma_final": weights["gamma_final"], "layers": []}
+    mats_per_layer = []
+    for lw in weights["layers"]:
+        mats = {n: dq(out_major(lw[n], *shape)) for n, shape in shapes.items()}
+        lay = {n: np.ascontiguousarray(mats[n].T).ravel() for n in ("wq", "wk", "wv", "wo", "w1", "w3")}
+        lay["w2"] = mats["w2"].ravel()
+        lay["gamma1"], lay["gamma2"] = lw["gamma1"], lw["gamma2"]
+        out["layers"].append(lay)
+        mats_per_layer.append(mats)
+    return out, mats_per_layer

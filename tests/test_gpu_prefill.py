@@ -1,0 +1,90 @@
+"""GPU parity of the chunked matrix-core prompt prefill (hipdec_prefill through the C ABI) against
+the CPU oracle's full-window forward (crates/engine/src/full_model.rs:336-437) and against the
+backend's own token-step prefill.  The prefill keeps activations fp32-grade (two bf16 parts), so
+the fp32-cache tolerance is the reference's 1e-4 on logits (crates/engine/tests/auto_kv_decode.rs:67-215);
+with a bf16 cache a 1-ulp difference can flip a cached value's rounding (2e-3)."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from rustane_amd import synth
+from rustane_amd.hipdec import Config, HipDecodeModel, KvDtype, WeightDtype
+
+pytestmark = pytest.mark.gpu
+
+FLAG_PREFILL_STEPS = 4
+
+
+def rel_err(a, b):
+    return float(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64)).max() / max(np.abs(b).max(), 1e-30))
+
+
+def make(cfg, wdt=WeightDtype.BF16, kvdt=KvDtype.F32, std=0.06, seed=31, act=0, flags=0):
+    w = synth.make_weights(cfg, seed=seed, std=std, round_bf16=True)
+    wo = w
+    if wdt == WeightDtype.FP8_E4M3:
+        wo, _ = O.dequantised_weights(cfg, w, "fp8")
+    orc = O.Oracle(cfg, wo, kv_round_bf16=(kvdt == KvDtype.BF16), ffn_activation=act)
+    dev = HipDecodeModel(cfg, w, weight_dtype=wdt, kv_dtype=kvdt, ffn_activation=act, flags=flags)
+    return w, orc, dev
+
+
+def check_prefill_then_decode(cfg, n_prompt, tol, n_decode=4, **kw):
+    w, orc, dev = make(cfg, **kw)
+    ids = synth.make_prompt(3, cfg.vocab, n_prompt)
+    lg_o, _, _ = orc.forward_window(ids)
+    lg_d = dev.prefill(ids)
+    assert dev.len() == n_prompt
+    assert rel_err(lg_d, lg_o[0]) < tol
+    # the caches the prefill wrote must carry the following cached steps
+    tok = int(O.argmax_lower(lg_o[0]))
+    for _ in range(n_decode):
+        a = orc.decode_logits_from_id(tok)
+        b = dev.decode_logits_from_id(tok)
+        assert rel_err(b, a) < tol
+        tok = int(O.argmax_lower(a))
+
+
+@pytest.mark.parametrize("n_prompt", [8, 33, 70, 128])
+def test_prefill_bf16_weights_f32_cache(n_prompt):
+    cfg = Config.make(dim=256, hidden=640, heads=2, hd=128, seq=160, nlayers=2, vocab=320)
+    check_prefill_then_decode(cfg, n_prompt, 1e-4)
+
+
+def test_prefill_hd64_gqa_and_leaky_relu():
+    cfg = Config.make(dim=256, hidden=384, heads=4, hd=64, seq=96, nlayers=3, vocab=512, kv_heads=2)
+    check_prefill_then_decode(cfg, 45, 1e-4, act=1)
+
+
+def test_prefill_bf16_cache():
+    cfg = Config.make(dim=512, hidden=1024, heads=4, hd=128, seq=200, nlayers=2, vocab=512)
+    check_prefill_then_decode(cfg, 150, 2e-3, kvdt=KvDtype.BF16)
+
+
+def test_prefill_fp8_weights():
+    cfg = Config.make(dim=512, hidden=1024, heads=4, hd=128, seq=128, nlayers=2, vocab=512)
+    check_prefill_then_decode(cfg, 65, 2e-3, wdt=WeightDtype.FP8_E4M3, kvdt=KvDtype.BF16, std=0.05)
+
+
+def test_prefill_in_two_calls_equals_one():
+    cfg = Config.make(dim=256, hidden=640, heads=2, hd=128, seq=160, nlayers=2, vocab=320)
+    w, orc, dev = make(cfg)
+    ids = synth.make_prompt(9, cfg.vocab, 90)
+    lg_o, _, _ = orc.forward_window(ids)
+    dev.prefill(ids[:50], want_logits=False)
+    lg_d = dev.prefill(ids[50:])
+    assert dev.len() == 90
+    assert rel_err(lg_d, lg_o[0]) < 1e-4
+
+
+def test_chunked_prefill_matches_token_step_prefill():
+    cfg = Config.make(dim=512, hidden=1024, heads=4, hd=128, seq=256, nlayers=3, vocab=1024)
+    w = synth.make_weights(cfg, seed=5, std=0.06, round_bf16=True)
+    ids = synth.make_prompt(4, cfg.vocab, 130)
+    a = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.F32)
+    b = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.F32, flags=FLAG_PREFILL_STEPS)
+    la, lb = a.prefill(ids), b.prefill(ids)
+    assert rel_err(la, lb) < 2e-5
+    ta = a.decode_greedy_run(int(np.argmax(la)), 16)
+    tb = b.decode_greedy_run(int(np.argmax(lb)), 16)
+    np.testing.assert_array_equal(ta, tb)
