@@ -134,6 +134,37 @@ int hipdec_decode_logits_from_id(hipdec_model *m, uint32_t token, float softcap,
  * (nullable, [vocab]) receives the softcapped logits of the last position. */
 int hipdec_prefill(hipdec_model *m, const uint32_t *ids, size_t n, float softcap, float *last_logits);
 
+/* ---- multi-sample decode: n_rows continuations of one shared prefix, stepped together ----
+ *
+ * The reference draws its `samples` one after the other, re-seeding the KV cache from the shared
+ * prompt caches for each (engine/src/inference.rs:247-262, :561).  Here the rows share cache
+ * positions [0, len) as they are when hipdec_batch_begin is called and each row appends to a
+ * suffix cache of its own, so every weight matrix is streamed once per step for all rows.  Row r of
+ * every batched call returns what the single-row call of the same name would return for a model
+ * that had decoded row r's tokens alone.  Between begin and end only the *_batch calls may be
+ * used; hipdec_batch_end leaves len and the shared positions as they were.  1 <= n_rows <= 32;
+ * needs bf16 or e4m3 weights (HIPDEC_ERR_UNSUPPORTED otherwise). */
+int hipdec_batch_begin(hipdec_model *m, size_t n_rows);
+int hipdec_batch_end(hipdec_model *m);
+/* steps taken since hipdec_batch_begin (each row is at position len + steps) */
+int hipdec_batch_steps(const hipdec_model *m, size_t *out_steps);
+/* tokens[n_rows]; out_logits[n_rows][vocab]  (hipdec_decode_logits_from_id per row) */
+int hipdec_decode_logits_from_ids_batch(hipdec_model *m, const uint32_t *tokens, float softcap, float *out_logits);
+/* tokens[n_rows] -> out_tokens[n_rows]  (Model::decode_token_argmax_from_id per row, lib.rs:340-375) */
+int hipdec_decode_token_argmax_from_ids_batch(hipdec_model *m, const uint32_t *tokens, uint32_t *out_tokens);
+/* out_vals/out_idxs[n_rows][blocks*top_k], cap = capacity of each array in elements, *out_count =
+ * blocks*top_k per row  (Model::decode_token_topk_from_id per row, lib.rs:377-434) */
+int hipdec_decode_token_topk_from_ids_batch(hipdec_model *m, const uint32_t *tokens, uint32_t top_k,
+                                            float *out_vals, uint32_t *out_idxs, size_t cap, size_t *out_count);
+/* out_maxes/out_sums[n_rows][blocks], *out_count = blocks per row
+ * (Model::decode_token_block_stats_from_id per row, lib.rs:436-487) */
+int hipdec_decode_token_block_stats_from_ids_batch(hipdec_model *m, const uint32_t *tokens, float inv_temperature,
+                                                   float softcap, float *out_maxes, float *out_sums, size_t cap,
+                                                   size_t *out_count);
+/* Model::materialize_current_logits_block for one row of the last batched step (lib.rs:489-511) */
+int hipdec_materialize_current_logits_block_batch(hipdec_model *m, size_t row, size_t block_idx, float softcap,
+                                                  float *out_logits, size_t cap, size_t *out_valid);
+
 /* Greedy run without a host round trip per token (the loop of engine/src/inference.rs:576-585):
  * starting from `token`, performs n_steps argmax steps, each feeding its result to the next;
  * out_tokens[n_steps].  Equivalent to n_steps calls of hipdec_decode_token_argmax_from_id. */

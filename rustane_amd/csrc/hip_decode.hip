@@ -3,6 +3,7 @@
 #include "../../include/hip_decode.h"
 #include "hipdec_mega.h"
 #include "hipdec_prefill.h"
+#include "hipdec_batch.h"
 
 #include <math.h>
 #include <stdio.h>
@@ -35,6 +36,23 @@ struct PrefillWork {
     float *P = nullptr;                  // split-K partial planes
     size_t P_floats = 0;
     uint32_t *h_ids = nullptr;           // pinned
+};
+
+// State of the multi-sample decode (hipdec_batch.h): rows share cache positions [0, prefix) and
+// append to their own suffix caches.
+enum BatchVariant { B_LOGITS = 0, B_ARGMAX, B_TOPK, B_STATS };
+struct BatchState {
+    int rows = 0;                        // 0: no batch open
+    size_t prefix = 0, slot = 0;
+    int cap_rows = 0;                    // rows the buffers below were sized for
+    size_t suf_rows = 0;                 // capacity of one row's suffix cache
+    std::vector<void *> kc_suf, vc_suf;  // per layer [cap_rows][suf_rows][kv_dim]
+    BatchParams *d_bp = nullptr, *h_bp = nullptr;
+    float *logits = nullptr, *d_out = nullptr, *d_vals = nullptr, *d_bmax = nullptr, *d_bsum = nullptr;
+    uint32_t *d_idxs = nullptr, *d_tok = nullptr;
+    float *h_stage = nullptr;            // pinned, cap_rows * max(vocab, 2 * blocks * 32) floats
+    size_t h_stage_floats = 0;
+    bool have_logits = false;            // a step has run since hipdec_batch_begin
 };
 
 }  // namespace
@@ -70,6 +88,7 @@ struct hipdec_model {
     size_t mega_lds = 0;
     unsigned *d_epochs = nullptr;
     PrefillWork pf;
+    BatchState bt;
     std::vector<void *> allocs;
     std::string err;
 };
@@ -390,7 +409,7 @@ PfSplit pf_split_k(const hipdec_model *m, int T, int N, int K) {
     return PfSplit{(nsteps + sps - 1) / sps, sps};
 }
 
-int pf_ensure(hipdec_model *m, int T) {
+int pf_ensure(hipdec_model *m, int T, bool with_head = false) {
     const hipdec_config &c = m->cfg;
     const size_t D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden;
     PrefillWork &w = m->pf;
@@ -413,6 +432,7 @@ int pf_ensure(hipdec_model *m, int T) {
     size_t need = 0;
     const int dims[4][2] = {{(int)(Q + 2 * KV), (int)D}, {(int)D, (int)Q}, {(int)(2 * H), (int)D}, {(int)D, (int)H}};
     for (auto &d : dims) need = std::max(need, (size_t)pf_split_k(m, T, d[0], d[1]).splits * T * d[0]);
+    if (with_head) need = std::max(need, (size_t)pf_split_k(m, T, (int)c.vocab, (int)D).splits * T * c.vocab);
     if (need > w.P_floats) {
         if ((rc = dalloc(m, &w.P, need * 4))) return rc;
         w.P_floats = need;
@@ -421,11 +441,11 @@ int pf_ensure(hipdec_model *m, int T) {
 }
 
 // P[z][t][n] = sum over the z-th K slice of A[t][k] * W[n][k]; returns the number of planes
-int pf_gemm(hipdec_model *m, const uint16_t *Ahi, const uint16_t *Alo, const void *W, int T, int N, int K) {
+int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, const void *W, int T, int N, int K) {
     const PfSplit sp = pf_split_k(m, T, N, K);
     PfGemm g{Ahi, Alo, W, m->pf.P, T, N, K, sp.steps_per_split};
     dim3 grid((N + PF_BN - 1) / PF_BN, (T + PF_BM - 1) / PF_BM, sp.splits), block(256);
-    if (m->wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm<WT_BF16>, grid, block, 0, m->stream, g);
+    if (wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm<WT_BF16>, grid, block, 0, m->stream, g);
     else hipLaunchKernelGGL(k_pf_gemm<WT_FP8>, grid, block, 0, m->stream, g);
     return sp.splits;
 }
@@ -459,7 +479,7 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
             const bool fp8 = m->wt == WT_FP8;
             // q/k/v projections, RoPE, cache append
             int N = Q + 2 * KV;
-            int sp = pf_gemm(m, w.xn_hi, w.xn_lo, L.wqkv, T, N, D);
+            int sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.wqkv, T, N, D);
             {
                 const size_t items = (size_t)T * (N / 2);
                 dim3 grid((unsigned)((items + 255) / 256)), block(256);
@@ -483,11 +503,11 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
 #undef PFATT
             }
             // output projection, residual, second norm
-            sp = pf_gemm(m, w.att_hi, w.att_lo, L.wo, T, D, Q);
+            sp = pf_gemm(m, m->wt, w.att_hi, w.att_lo, L.wo, T, D, Q);
             hipLaunchKernelGGL(k_pf_resid_norm, dim3(T), dim3(256), 0, m->stream, w.P, sp, (size_t)T * D,
                                fp8 ? (const float *)L.s_wo : nullptr, w.x, m->alpha, w.x2, L.g2, w.xn_hi, w.xn_lo, D);
             // gate/up, activation
-            sp = pf_gemm(m, w.xn_hi, w.xn_lo, L.w13, T, 2 * H, D);
+            sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.w13, T, 2 * H, D);
             {
                 const size_t items = (size_t)T * H;
                 hipLaunchKernelGGL(k_pf_gate_epi, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, m->stream, w.P, sp,
@@ -495,7 +515,7 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
                                    (int)m->opt.ffn_activation);
             }
             // down projection, residual, next layer's first norm
-            sp = pf_gemm(m, w.gate_hi, w.gate_lo, L.w2, T, D, H);
+            sp = pf_gemm(m, m->wt, w.gate_hi, w.gate_lo, L.w2, T, D, H);
             const float *gnext = l + 1 < c.nlayers ? m->layers[l + 1].g1 : nullptr;
             hipLaunchKernelGGL(k_pf_resid_norm, dim3(T), dim3(256), 0, m->stream, w.P, sp, (size_t)T * D,
                                fp8 ? (const float *)L.s_w2 : nullptr, w.x2, m->alpha, w.x, gnext, w.xn_hi, w.xn_lo, D);
@@ -504,6 +524,140 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
         *x_last = w.x + (size_t)(T - 1) * D;
         done += T;
     }
+    return HIPDEC_OK;
+}
+
+// ---- multi-sample decode (hipdec_batch.h)
+constexpr int kBatchMaxRows = 32;
+
+int batch_alloc(hipdec_model *m, int rows) {
+    const hipdec_config &c = m->cfg;
+    BatchState &b = m->bt;
+    if (b.cap_rows >= rows) return HIPDEC_OK;
+    int rc;
+    const size_t esz = m->kvbf16 ? 2 : 4, V = c.vocab, blocks = (size_t)m->blocks;
+    b.suf_rows = c.seq;
+    b.kc_suf.assign(c.nlayers, nullptr);
+    b.vc_suf.assign(c.nlayers, nullptr);
+    for (uint32_t l = 0; l < c.nlayers; ++l) {
+        if ((rc = dalloc(m, &b.kc_suf[l], (size_t)rows * b.suf_rows * c.kv_dim * esz))) return rc;
+        if ((rc = dalloc(m, &b.vc_suf[l], (size_t)rows * b.suf_rows * c.kv_dim * esz))) return rc;
+    }
+    if (!b.d_bp) { if ((rc = dalloc(m, &b.d_bp, sizeof(BatchParams)))) return rc; }
+    if (!b.h_bp) HCHK(hipHostMalloc((void **)&b.h_bp, sizeof(BatchParams)));
+    if ((rc = dalloc(m, &b.logits, (size_t)rows * V * 4))) return rc;
+    if ((rc = dalloc(m, &b.d_out, (size_t)rows * V * 4))) return rc;
+    if ((rc = dalloc(m, &b.d_vals, (size_t)rows * blocks * HIPDEC_MAX_GPU_TOPK * 4))) return rc;
+    if ((rc = dalloc(m, &b.d_idxs, (size_t)rows * blocks * HIPDEC_MAX_GPU_TOPK * 4))) return rc;
+    if ((rc = dalloc(m, &b.d_bmax, (size_t)rows * blocks * 4))) return rc;
+    if ((rc = dalloc(m, &b.d_bsum, (size_t)rows * blocks * 4))) return rc;
+    if ((rc = dalloc(m, &b.d_tok, (size_t)rows * 4))) return rc;
+    if (b.h_stage) (void)hipHostFree(b.h_stage);
+    b.h_stage_floats = (size_t)rows * std::max(V, 2 * blocks * HIPDEC_MAX_GPU_TOPK);
+    HCHK(hipHostMalloc((void **)&b.h_stage, b.h_stage_floats * 4));
+    b.cap_rows = rows;
+    return HIPDEC_OK;
+}
+
+// one step of every open row: tokens[r] at position prefix + slot
+int batch_step(hipdec_model *m, const uint32_t *tokens, int variant, uint32_t top_k, float inv_t, float softcap) {
+    const hipdec_config &c = m->cfg;
+    BatchState &b = m->bt;
+    if (b.rows <= 0) return fail(m, HIPDEC_ERR_ARG, "no batch is open (hipdec_batch_begin)");
+    if (!tokens) return fail(m, HIPDEC_ERR_ARG, "null buffer");
+    if (b.prefix + b.slot >= c.seq) return fail(m, HIPDEC_ERR_FULL, "decode only supports lengths within cfg.seq");
+    const int R = b.rows;
+    for (int r = 0; r < R; ++r)
+        if (tokens[r] >= c.vocab) return fail(m, HIPDEC_ERR_ARG, "token id must fit vocab");
+    const int D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden, V = c.vocab;
+    const int gqa = c.gqa_ratio ? c.gqa_ratio : 1;
+    const float scale = 1.0f / sqrtf((float)c.hd);
+    int rc = pf_ensure(m, R, true);
+    if (rc) return rc;
+    PrefillWork &w = m->pf;
+    HCHK(hipStreamSynchronize(m->stream));                      // pinned staging is free again
+    memcpy(w.h_ids, tokens, (size_t)R * 4);
+    *b.h_bp = BatchParams{(int)(b.prefix + b.slot), (int)b.slot, (int)b.prefix, (int)top_k, inv_t, softcap};
+    HCHK(hipMemcpyAsync(w.ids, w.h_ids, (size_t)R * 4, hipMemcpyHostToDevice, m->stream));
+    HCHK(hipMemcpyAsync(b.d_bp, b.h_bp, sizeof(BatchParams), hipMemcpyHostToDevice, m->stream));
+    HCHK(hipEventRecord(m->ev0, m->stream));
+    if (m->embed_wt == WT_F32)
+        hipLaunchKernelGGL(k_pf_embed_norm<WT_F32>, dim3(R), dim3(256), 0, m->stream, m->embed, w.ids, w.x,
+                           m->layers[0].g1, w.xn_hi, w.xn_lo, D);
+    else
+        hipLaunchKernelGGL(k_pf_embed_norm<WT_BF16>, dim3(R), dim3(256), 0, m->stream, m->embed, w.ids, w.x,
+                           m->layers[0].g1, w.xn_hi, w.xn_lo, D);
+    const bool fp8 = m->wt == WT_FP8;
+    for (uint32_t l = 0; l < c.nlayers; ++l) {
+        const DevLayer &L = m->layers[l];
+        const int N = Q + 2 * KV;
+        int sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.wqkv, R, N, D);
+        {
+            const size_t items = (size_t)R * (N / 2);
+            dim3 grid((unsigned)((items + 255) / 256)), block(256);
+            if (m->kvbf16)
+                hipLaunchKernelGGL(k_bd_qkv_epi<1>, grid, block, 0, m->stream, w.P, sp, (size_t)R * N,
+                                   fp8 ? (const float *)L.s_qkv : nullptr, w.q, b.kc_suf[l], b.vc_suf[l], b.suf_rows,
+                                   m->rope_cos, m->rope_sin, b.d_bp, R, Q, KV, (int)c.hd);
+            else
+                hipLaunchKernelGGL(k_bd_qkv_epi<0>, grid, block, 0, m->stream, w.P, sp, (size_t)R * N,
+                                   fp8 ? (const float *)L.s_qkv : nullptr, w.q, b.kc_suf[l], b.vc_suf[l], b.suf_rows,
+                                   m->rope_cos, m->rope_sin, b.d_bp, R, Q, KV, (int)c.hd);
+        }
+        {
+            dim3 grid(c.heads, R), block(256);
+#define BDATT(KVB, HD)                                                                                             \
+    hipLaunchKernelGGL((k_bd_attn<KVB, HD>), grid, block, 0, m->stream, w.q, L.kc, L.vc, b.kc_suf[l], b.vc_suf[l], \
+                       b.suf_rows, b.d_bp, w.att_hi, w.att_lo, Q, KV, gqa, scale)
+            if (m->kvbf16) { if (c.hd == 64) BDATT(1, 64); else BDATT(1, 128); }
+            else { if (c.hd == 64) BDATT(0, 64); else BDATT(0, 128); }
+#undef BDATT
+        }
+        sp = pf_gemm(m, m->wt, w.att_hi, w.att_lo, L.wo, R, D, Q);
+        hipLaunchKernelGGL(k_pf_resid_norm, dim3(R), dim3(256), 0, m->stream, w.P, sp, (size_t)R * D,
+                           fp8 ? (const float *)L.s_wo : nullptr, w.x, m->alpha, w.x2, L.g2, w.xn_hi, w.xn_lo, D);
+        sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.w13, R, 2 * H, D);
+        {
+            const size_t items = (size_t)R * H;
+            hipLaunchKernelGGL(k_pf_gate_epi, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, m->stream, w.P, sp,
+                               (size_t)R * 2 * H, fp8 ? (const float *)L.s_w13 : nullptr, w.gate_hi, w.gate_lo, R, H,
+                               (int)m->opt.ffn_activation);
+        }
+        sp = pf_gemm(m, m->wt, w.gate_hi, w.gate_lo, L.w2, R, D, H);
+        // the last layer's residual kernel applies the final norm instead of the next layer's first one
+        const float *gnext = l + 1 < c.nlayers ? m->layers[l + 1].g1 : m->gfinal;
+        hipLaunchKernelGGL(k_pf_resid_norm, dim3(R), dim3(256), 0, m->stream, w.P, sp, (size_t)R * D,
+                           fp8 ? (const float *)L.s_w2 : nullptr, w.x2, m->alpha, w.x, gnext, w.xn_hi, w.xn_lo, D);
+    }
+    // tied LM head for every row (full_model.rs:419-428), then the per-row head kernel
+    {
+        const int sp = pf_gemm(m, m->embed_wt, w.xn_hi, w.xn_lo, m->embed, R, V, D);
+        const size_t n = (size_t)R * V;
+        hipLaunchKernelGGL(k_bd_sum_planes, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, m->stream, w.P, sp, n,
+                           b.logits, n);
+    }
+    if (variant == B_ARGMAX)
+        hipLaunchKernelGGL(k_bd_argmax, dim3(R), dim3(1024), 0, m->stream, b.logits, V, b.d_tok);
+    else if (variant == B_TOPK)
+        hipLaunchKernelGGL(k_bd_topk, dim3(m->blocks, R), dim3(256), 0, m->stream, b.logits, V, b.d_bp, b.d_vals, b.d_idxs);
+    else if (variant == B_STATS)
+        hipLaunchKernelGGL(k_bd_block_stats, dim3(m->blocks, R), dim3(256), 0, m->stream, b.logits, V, b.d_bp, b.d_bmax,
+                           b.d_bsum);
+    HCHK(hipGetLastError());
+    HCHK(hipEventRecord(m->ev1, m->stream));
+    b.slot += 1;
+    b.have_logits = true;
+    return HIPDEC_OK;
+}
+
+// copies `floats` values from device memory to the caller through the pinned staging buffer
+int batch_fetch(hipdec_model *m, const void *dev, void *host, size_t floats) {
+    BatchState &b = m->bt;
+    if (floats > b.h_stage_floats) return fail(m, HIPDEC_ERR_ARG, "internal: staging buffer too small");
+    HCHK(hipMemcpyAsync(b.h_stage, dev, floats * 4, hipMemcpyDeviceToHost, m->stream));
+    HCHK(hipStreamSynchronize(m->stream));
+    HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+    memcpy(host, b.h_stage, floats * 4);
     return HIPDEC_OK;
 }
 
@@ -521,6 +675,8 @@ void hipdec_destroy(hipdec_model *m) {
     if (m->h_sp) (void)hipHostFree(m->h_sp);
     if (m->h_out) (void)hipHostFree(m->h_out);
     if (m->pf.h_ids) (void)hipHostFree(m->pf.h_ids);
+    if (m->bt.h_bp) (void)hipHostFree(m->bt.h_bp);
+    if (m->bt.h_stage) (void)hipHostFree(m->bt.h_stage);
     if (m->ev0) (void)hipEventDestroy(m->ev0);
     if (m->ev1) (void)hipEventDestroy(m->ev1);
     if (m->stream) (void)hipStreamDestroy(m->stream);
@@ -957,6 +1113,99 @@ int hipdec_prefill(hipdec_model *m, const uint32_t *ids, size_t n, float softcap
     }
     HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
     m->len += n;
+    return HIPDEC_OK;
+}
+
+int hipdec_batch_begin(hipdec_model *m, size_t n_rows) {
+    if (!m) return HIPDEC_ERR_ARG;
+    if (n_rows == 0 || n_rows > (size_t)kBatchMaxRows) return fail(m, HIPDEC_ERR_ARG, "n_rows must be in 1..32");
+    if (!prefill_batched_ok(m, kPrefillMinRows))
+        return fail(m, HIPDEC_ERR_UNSUPPORTED, "multi-row decode needs bf16 or e4m3 weights and dimensions that are multiples of 32");
+    if (m->len >= m->cfg.seq) return fail(m, HIPDEC_ERR_FULL, "decode only supports lengths within cfg.seq");
+    int rc = batch_alloc(m, (int)n_rows);
+    if (rc) return rc;
+    m->bt.rows = (int)n_rows;
+    m->bt.prefix = m->len;
+    m->bt.slot = 0;
+    m->bt.have_logits = false;
+    return HIPDEC_OK;
+}
+
+int hipdec_batch_end(hipdec_model *m) {
+    if (!m) return HIPDEC_ERR_ARG;
+    m->bt.rows = 0;
+    m->bt.have_logits = false;
+    return HIPDEC_OK;
+}
+
+int hipdec_batch_steps(const hipdec_model *m, size_t *out_steps) {
+    if (!m || !out_steps) return HIPDEC_ERR_ARG;
+    *out_steps = m->bt.rows ? m->bt.slot : 0;
+    return HIPDEC_OK;
+}
+
+int hipdec_decode_logits_from_ids_batch(hipdec_model *m, const uint32_t *tokens, float softcap, float *out_logits) {
+    if (!m || !out_logits) return HIPDEC_ERR_ARG;
+    int rc = batch_step(m, tokens, B_LOGITS, 1, 1.0f, 0.0f);
+    if (rc) return rc;
+    const size_t n = (size_t)m->bt.rows * m->cfg.vocab;
+    hipLaunchKernelGGL(k_softcap_copy, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, m->stream, m->bt.logits,
+                       m->bt.d_out, 0, (int)n, softcap);
+    HCHK(hipGetLastError());
+    return batch_fetch(m, m->bt.d_out, out_logits, n);
+}
+
+int hipdec_decode_token_argmax_from_ids_batch(hipdec_model *m, const uint32_t *tokens, uint32_t *out_tokens) {
+    if (!m || !out_tokens) return HIPDEC_ERR_ARG;
+    int rc = batch_step(m, tokens, B_ARGMAX, 1, 1.0f, 0.0f);
+    if (rc) return rc;
+    return batch_fetch(m, m->bt.d_tok, out_tokens, (size_t)m->bt.rows);
+}
+
+int hipdec_decode_token_topk_from_ids_batch(hipdec_model *m, const uint32_t *tokens, uint32_t top_k, float *out_vals,
+                                            uint32_t *out_idxs, size_t cap, size_t *out_count) {
+    if (!m || !out_vals || !out_idxs) return HIPDEC_ERR_ARG;
+    if (top_k == 0 || top_k > HIPDEC_MAX_GPU_TOPK) return fail(m, HIPDEC_ERR_ARG, "gpu top-k only supports k in 1..32");
+    const size_t per_row = (size_t)m->blocks * top_k, n = per_row * (size_t)std::max(m->bt.rows, 1);
+    if (cap < n) return fail(m, HIPDEC_ERR_ARG, "top-k outputs must fit the per-block candidates of every row");
+    int rc = batch_step(m, tokens, B_TOPK, top_k, 1.0f, 0.0f);
+    if (rc) return rc;
+    if ((rc = batch_fetch(m, m->bt.d_vals, out_vals, n))) return rc;
+    if ((rc = batch_fetch(m, m->bt.d_idxs, out_idxs, n))) return rc;
+    if (out_count) *out_count = per_row;
+    return HIPDEC_OK;
+}
+
+int hipdec_decode_token_block_stats_from_ids_batch(hipdec_model *m, const uint32_t *tokens, float inv_temperature,
+                                                   float softcap, float *out_maxes, float *out_sums, size_t cap,
+                                                   size_t *out_count) {
+    if (!m || !out_maxes || !out_sums) return HIPDEC_ERR_ARG;
+    const size_t n = (size_t)m->blocks * (size_t)std::max(m->bt.rows, 1);
+    if (cap < n) return fail(m, HIPDEC_ERR_ARG, "block stats outputs must fit the vocab blocks of every row");
+    int rc = batch_step(m, tokens, B_STATS, 1, inv_temperature, softcap);
+    if (rc) return rc;
+    if ((rc = batch_fetch(m, m->bt.d_bmax, out_maxes, n))) return rc;
+    if ((rc = batch_fetch(m, m->bt.d_bsum, out_sums, n))) return rc;
+    if (out_count) *out_count = (size_t)m->blocks;
+    return HIPDEC_OK;
+}
+
+int hipdec_materialize_current_logits_block_batch(hipdec_model *m, size_t row, size_t block_idx, float softcap,
+                                                  float *out_logits, size_t cap, size_t *out_valid) {
+    if (!m || !out_logits) return HIPDEC_ERR_ARG;
+    BatchState &b = m->bt;
+    if (b.rows <= 0 || !b.have_logits) return fail(m, HIPDEC_ERR_ARG, "no batched step has run");
+    if (row >= (size_t)b.rows) return fail(m, HIPDEC_ERR_ARG, "row out of range");
+    if (block_idx >= (size_t)m->blocks) return fail(m, HIPDEC_ERR_ARG, "block index out of range");
+    const size_t V = m->cfg.vocab, start = block_idx * HIPDEC_HEAD_BLOCK;
+    const size_t valid = std::min<size_t>(HIPDEC_HEAD_BLOCK, V - start);
+    if (cap < valid) return fail(m, HIPDEC_ERR_ARG, "logits block output too small");
+    hipLaunchKernelGGL(k_softcap_copy, dim3(1), dim3(256), 0, m->stream, b.logits + row * V, b.d_out, (int)start, (int)valid,
+                       softcap);
+    HCHK(hipGetLastError());
+    int rc = batch_fetch(m, b.d_out, out_logits, valid);
+    if (rc) return rc;
+    if (out_valid) *out_valid = valid;
     return HIPDEC_OK;
 }
 

@@ -26,6 +26,9 @@ EXPORTS = [
     "hipdec_decode_token_block_stats_from_id", "hipdec_materialize_current_logits_block",
     "hipdec_decode_logits_from_id", "hipdec_prefill", "hipdec_decode_greedy_run", "hipdec_last_device_ms",
     "hipdec_bytes_per_token", "hipdec_export_weight", "hipdec_debug_step_profile", "hipdec_debug_calibration_copy",
+    "hipdec_batch_begin", "hipdec_batch_end", "hipdec_batch_steps", "hipdec_decode_logits_from_ids_batch",
+    "hipdec_decode_token_argmax_from_ids_batch", "hipdec_decode_token_topk_from_ids_batch",
+    "hipdec_decode_token_block_stats_from_ids_batch", "hipdec_materialize_current_logits_block_batch",
 ]
 
 
@@ -118,6 +121,17 @@ def load_library(path=None):
     lib.hipdec_debug_step_profile.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(C.c_uint64), C.c_size_t,
                                               C.POINTER(C.c_size_t)]
     lib.hipdec_debug_calibration_copy.argtypes = [C.c_size_t, C.c_int]
+    szp = C.POINTER(C.c_size_t)
+    lib.hipdec_batch_begin.argtypes = [C.c_void_p, C.c_size_t]
+    lib.hipdec_batch_end.argtypes = [C.c_void_p]
+    lib.hipdec_batch_steps.argtypes = [C.c_void_p, szp]
+    lib.hipdec_decode_logits_from_ids_batch.argtypes = [C.c_void_p, u32p, C.c_float, fp]
+    lib.hipdec_decode_token_argmax_from_ids_batch.argtypes = [C.c_void_p, u32p, u32p]
+    lib.hipdec_decode_token_topk_from_ids_batch.argtypes = [C.c_void_p, u32p, C.c_uint32, fp, u32p, C.c_size_t, szp]
+    lib.hipdec_decode_token_block_stats_from_ids_batch.argtypes = [C.c_void_p, u32p, C.c_float, C.c_float, fp, fp,
+                                                                   C.c_size_t, szp]
+    lib.hipdec_materialize_current_logits_block_batch.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_float, fp,
+                                                                  C.c_size_t, szp]
     if path is None:
         _LIB = lib
     return lib
@@ -171,6 +185,7 @@ class HipDecodeModel:
         if rc != OK:
             raise HipDecodeError(rc, (self._lib.hipdec_last_error(None) or b"").decode())
         self.blocks = (V + HEAD_BLOCK - 1) // HEAD_BLOCK
+        self._rows = 0
 
     def close(self):
         if getattr(self, "_h", None) and self._h.value:
@@ -264,6 +279,68 @@ class HipDecodeModel:
         self._chk(self._lib.hipdec_decode_greedy_run(self._h, token, n_steps,
                                                      out.ctypes.data_as(C.POINTER(C.c_uint32))))
         return out[:n_steps]
+
+    # ---- multi-sample decode: rows share positions [0, len) and step together
+    def batch_begin(self, n_rows):
+        self._chk(self._lib.hipdec_batch_begin(self._h, n_rows))
+        self._rows = int(n_rows)
+
+    def batch_end(self):
+        self._chk(self._lib.hipdec_batch_end(self._h))
+        self._rows = 0
+
+    def batch_steps(self):
+        n = C.c_size_t()
+        self._chk(self._lib.hipdec_batch_steps(self._h, C.byref(n)))
+        return n.value
+
+    def _toks(self, tokens):
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        if t.size != self._rows:
+            raise ValueError("expected %d tokens, got %d" % (self._rows, t.size))
+        return t
+
+    def decode_logits_from_ids_batch(self, tokens, softcap=0.0):
+        t = self._toks(tokens)
+        out = np.empty((self._rows, self.cfg.vocab), np.float32)
+        self._chk(self._lib.hipdec_decode_logits_from_ids_batch(self._h, t.ctypes.data_as(C.POINTER(C.c_uint32)), softcap,
+                                                               _fptr(out)))
+        return out
+
+    def decode_token_argmax_from_ids_batch(self, tokens):
+        t = self._toks(tokens)
+        out = np.empty(self._rows, np.uint32)
+        self._chk(self._lib.hipdec_decode_token_argmax_from_ids_batch(
+            self._h, t.ctypes.data_as(C.POINTER(C.c_uint32)), out.ctypes.data_as(C.POINTER(C.c_uint32))))
+        return out
+
+    def decode_token_topk_from_ids_batch(self, tokens, top_k):
+        t = self._toks(tokens)
+        per = self.blocks * max(int(top_k), 1)
+        vals = np.empty((self._rows, per), np.float32)
+        idxs = np.empty((self._rows, per), np.uint32)
+        cnt = C.c_size_t()
+        self._chk(self._lib.hipdec_decode_token_topk_from_ids_batch(
+            self._h, t.ctypes.data_as(C.POINTER(C.c_uint32)), top_k, _fptr(vals),
+            idxs.ctypes.data_as(C.POINTER(C.c_uint32)), vals.size, C.byref(cnt)))
+        return vals, idxs
+
+    def decode_token_block_stats_from_ids_batch(self, tokens, inv_temperature, softcap):
+        t = self._toks(tokens)
+        mx = np.empty((self._rows, self.blocks), np.float32)
+        sm = np.empty((self._rows, self.blocks), np.float32)
+        cnt = C.c_size_t()
+        self._chk(self._lib.hipdec_decode_token_block_stats_from_ids_batch(
+            self._h, t.ctypes.data_as(C.POINTER(C.c_uint32)), inv_temperature, softcap, _fptr(mx), _fptr(sm), mx.size,
+            C.byref(cnt)))
+        return mx, sm
+
+    def materialize_current_logits_block_batch(self, row, block_idx, softcap, cap=HEAD_BLOCK):
+        out = np.empty(max(cap, 1), np.float32)
+        valid = C.c_size_t()
+        self._chk(self._lib.hipdec_materialize_current_logits_block_batch(self._h, row, block_idx, softcap, _fptr(out),
+                                                                          cap, C.byref(valid)))
+        return out[:valid.value]
 
     def last_device_ms(self):
         ms = C.c_float()
