@@ -165,6 +165,79 @@ void DecodeContext::decode_greedy_run(uint32_t token, size_t n_steps, uint32_t *
     check(hipdec_decode_greedy_run(m_, token, n_steps, out), "decode_greedy_run");
 }
 
+bool DecodeContext::batch_begin(size_t rows) {
+    const int rc = hipdec_batch_begin(m_, rows);
+    if (rc == HIPDEC_ERR_UNSUPPORTED) return false;
+    check(rc, "batch_begin");
+    batch_rows_ = rows;
+    b_vals_.assign(rows * blocks_ * MAX_GPU_TOPK, 0.0f);
+    b_idxs_.assign(rows * blocks_ * MAX_GPU_TOPK, UINT32_MAX);
+    b_merged_vals_.assign(rows * MAX_GPU_TOPK, 0.0f);
+    b_merged_idxs_.assign(rows * MAX_GPU_TOPK, UINT32_MAX);
+    b_counts_.assign(rows, 0);
+    b_maxes_.assign(rows * blocks_, 0.0f);
+    b_sums_.assign(rows * blocks_, 0.0f);
+    return true;
+}
+
+void DecodeContext::batch_end() {
+    check(hipdec_batch_end(m_), "batch_end");
+    batch_rows_ = 0;
+}
+
+void DecodeContext::decode_next_greedy_tokens(const uint32_t *tokens, uint32_t *out) {
+    check(hipdec_decode_token_argmax_from_ids_batch(m_, tokens, out), "decode_next_greedy_tokens");
+}
+
+void DecodeContext::decode_next_topk_candidates_batch(const uint32_t *tokens, size_t top_k, float softcap,
+                                                      const uint32_t **idxs, const float **logits, const size_t **n) {
+    if (top_k > MAX_GPU_TOPK) top_k = MAX_GPU_TOPK;            // decode.rs:140
+    if (top_k > vocab_) top_k = vocab_;
+    size_t per_row = 0;
+    check(hipdec_decode_token_topk_from_ids_batch(m_, tokens, (uint32_t)top_k, b_vals_.data(), b_idxs_.data(),
+                                                  b_vals_.size(), &per_row),
+          "decode_next_topk_candidates_batch");
+    for (size_t r = 0; r < batch_rows_; ++r) {
+        float *mv = b_merged_vals_.data() + r * MAX_GPU_TOPK;
+        const size_t merged = merge_topk_candidates(b_vals_.data() + r * per_row, b_idxs_.data() + r * per_row, per_row,
+                                                    top_k, mv, b_merged_idxs_.data() + r * MAX_GPU_TOPK);
+        if (softcap > 0.0f)                                    // decode.rs:155-159
+            for (size_t i = 0; i < merged; ++i) mv[i] = softcap * tanhf(mv[i] / softcap);
+        b_counts_[r] = merged;
+    }
+    *idxs = b_merged_idxs_.data();
+    *logits = b_merged_vals_.data();
+    *n = b_counts_.data();
+}
+
+void DecodeContext::decode_next_fullvocab_block_stats_batch(const uint32_t *tokens, float temperature, float softcap,
+                                                            const float **maxes, const float **sums, size_t *blocks) {
+    const float t = temperature > std::numeric_limits<float>::min() ? temperature : std::numeric_limits<float>::min();
+    size_t count = 0;
+    check(hipdec_decode_token_block_stats_from_ids_batch(m_, tokens, 1.0f / t, softcap, b_maxes_.data(), b_sums_.data(),
+                                                         b_maxes_.size(), &count),
+          "decode_next_fullvocab_block_stats_batch");
+    *maxes = b_maxes_.data();
+    *sums = b_sums_.data();
+    *blocks = count;
+}
+
+void DecodeContext::materialize_current_logits_block_batch(size_t row, size_t block_idx, float softcap,
+                                                           const float **logits, size_t *n) {
+    size_t valid = 0;
+    check(hipdec_materialize_current_logits_block_batch(m_, row, block_idx, softcap, block_logits_.data(),
+                                                        block_logits_.size(), &valid),
+          "materialize_current_logits_block_batch");
+    *logits = block_logits_.data();
+    *n = valid;
+}
+
+const float *DecodeContext::decode_next_logits_batch(const uint32_t *tokens, float softcap) {
+    b_logits_.resize(batch_rows_ * vocab_);
+    check(hipdec_decode_logits_from_ids_batch(m_, tokens, softcap, b_logits_.data()), "decode_next_logits_batch");
+    return b_logits_.data();
+}
+
 float DecodeContext::last_device_ms() const {
     float ms = 0.0f;
     hipdec_last_device_ms(m_, &ms);

@@ -52,6 +52,24 @@ public:
     // not in the reference: prompt prefill on the GPU and greedy runs without per-token host round trips
     const std::vector<float> &prefill(const uint32_t *ids, size_t n, float softcap);
     void decode_greedy_run(uint32_t token, size_t n_steps, uint32_t *out);
+    // not in the reference: `rows` continuations of the current cache contents stepped together
+    // (the reference runs its samples one after the other, inference.rs:247-262).  batch_begin
+    // returns false when the backend has no multi-row path for this model.
+    bool batch_begin(size_t rows);
+    void batch_end();
+    size_t batch_rows() const { return batch_rows_; }
+    // tokens[rows] -> out[rows]
+    void decode_next_greedy_tokens(const uint32_t *tokens, uint32_t *out);
+    // row r's merged, softcapped candidates are at idxs + r * MAX_GPU_TOPK / logits + r * MAX_GPU_TOPK, n[r] of them
+    void decode_next_topk_candidates_batch(const uint32_t *tokens, size_t top_k, float softcap, const uint32_t **idxs,
+                                           const float **logits, const size_t **n);
+    // row r's block statistics are at maxes + r * blocks / sums + r * blocks
+    void decode_next_fullvocab_block_stats_batch(const uint32_t *tokens, float temperature, float softcap,
+                                                 const float **maxes, const float **sums, size_t *blocks);
+    void materialize_current_logits_block_batch(size_t row, size_t block_idx, float softcap, const float **logits,
+                                                size_t *n);
+    // row r's logits are at result + r * vocab
+    const float *decode_next_logits_batch(const uint32_t *tokens, float softcap);
     float last_device_ms() const;
     uint64_t bytes_per_token(size_t kv_len) const;
     hipdec_model *raw() { return m_; }
@@ -63,6 +81,11 @@ private:
     // decode.rs:19-31 DecodeWorkspace
     std::vector<float> logits_, block_maxes_, block_sums_, block_logits_, topk_vals_, merged_vals_;
     std::vector<uint32_t> topk_idxs_, merged_idxs_;
+    // multi-row workspace
+    size_t batch_rows_ = 0;
+    std::vector<float> b_logits_, b_vals_, b_merged_vals_, b_maxes_, b_sums_;
+    std::vector<uint32_t> b_idxs_, b_merged_idxs_;
+    std::vector<size_t> b_counts_;
 };
 
 }  // namespace rustane

@@ -196,7 +196,7 @@ size_t fill_input_window(const std::vector<uint32_t> &generated, size_t seq, std
 InferenceSession::InferenceSession(const ModelConfig &cfg, const ModelWeights &weights,
                                    const std::vector<uint32_t> &prompt_ids, float softcap, const SessionOptions &opts,
                                    std::string *err)
-    : cfg_(cfg), prompt_ids_(prompt_ids), softcap_(softcap) {
+    : cfg_(cfg), prompt_ids_(prompt_ids), softcap_(softcap), batch_samples_(opts.batch_samples) {
     err->clear();
     if (prompt_ids.empty()) { *err = "prompt must contain at least one token"; return; }           // inference.rs:131-133
     *err = validate_token_ids(prompt_ids.data(), prompt_ids.size(), cfg.vocab, "prompt");
@@ -275,7 +275,11 @@ bool InferenceSession::run_request(const GenerationRequest &req, const std::vect
             request_prefill = now_s() - t0;
         }
         out->results.clear();
-        for (size_t i = 0; i < req.samples; ++i) {
+        bool batched = false;
+        if (use_kv && !cb && req.samples > 1 && req.steps > 1 && batch_samples_) {
+            if (!run_cached_batch(eff_ids, prompt_logits, suffix, req, &out->results, &batched, err)) return false;
+        }
+        for (size_t i = 0; !batched && i < req.samples; ++i) {
             const uint64_t seed = cb ? req.seed : req.seed + (uint64_t)i;                          // :256, :414
             SampleResult r;
             const bool ok = use_kv ? run_cached_sample(eff_ids, prompt_logits, suffix, req, seed, cb, &r, err)
@@ -361,6 +365,68 @@ bool InferenceSession::run_cached_sample(const std::vector<uint32_t> &prompt, co
         }
     }
     out->decode_elapsed = now_s() - t0;
+    return true;
+}
+
+// The loop of run_cached_sample for every sample of the request at once: sample i keeps its own
+// RNG (seed + i, inference.rs:256) and its own token stream; one device step serves all of them.
+bool InferenceSession::run_cached_batch(const std::vector<uint32_t> &prompt, const std::vector<float> &prompt_logits,
+                                        const std::vector<uint32_t> &suffix, const GenerationRequest &req,
+                                        std::vector<SampleResult> *out, bool *done, std::string *err) {
+    (void)err;
+    *done = false;
+    const size_t R = req.samples;
+    if (R > 32) return true;                                                       // backend limit: fall back
+    restore_prompt_cache();
+    const double t0 = now_s();                                                     // :562
+    for (uint32_t tok : suffix) ctx_->decode_next_logits(tok, softcap_);          // :563-565
+    if (!ctx_->batch_begin(R)) return true;
+    std::vector<SampleResult> res(R);
+    std::vector<uint64_t> rng(R);
+    std::vector<uint32_t> cur(R), nxt(R);
+    for (size_t r = 0; r < R; ++r) {
+        res[r].seed = req.seed + (uint64_t)r;
+        res[r].generated = prompt;
+        res[r].sampled.reserve(req.steps);
+        rng[r] = res[r].seed;
+        cur[r] = sample_next(prompt_logits.data(), prompt_logits.size(), req.temperature, req.top_k, &rng[r],
+                             &sampler_scratch_);
+        res[r].generated.push_back(cur[r]);
+        res[r].sampled.push_back(cur[r]);
+    }
+    for (size_t i = 1; i < req.steps; ++i) {
+        if (req.temperature <= 0.0f || req.top_k == 1) {                           // :576-585
+            ctx_->decode_next_greedy_tokens(cur.data(), nxt.data());
+        } else if (req.top_k > 0 && req.top_k <= MAX_GPU_TOPK) {                   // :586-599
+            const uint32_t *idxs; const float *lg; const size_t *n;
+            ctx_->decode_next_topk_candidates_batch(cur.data(), req.top_k, softcap_, &idxs, &lg, &n);
+            for (size_t r = 0; r < R; ++r)
+                nxt[r] = sample_topk_candidates(idxs + r * MAX_GPU_TOPK, lg + r * MAX_GPU_TOPK, n[r], req.temperature, &rng[r]);
+        } else if (req.top_k == 0) {                                               // :600-625
+            const float *mx, *sm; size_t nb;
+            ctx_->decode_next_fullvocab_block_stats_batch(cur.data(), req.temperature, softcap_, &mx, &sm, &nb);
+            for (size_t r = 0; r < R; ++r) {
+                const size_t blk = sample_block_from_stats(mx + r * nb, sm + r * nb, nb, &rng[r]);
+                const float *bl; size_t nv;
+                ctx_->materialize_current_logits_block_batch(r, blk, softcap_, &bl, &nv);
+                nxt[r] = sample_block_logits((uint32_t)(blk * 256), bl, nv, req.temperature, &rng[r]);   // :613
+            }
+        } else {                                                                   // :626-638
+            const float *lg = ctx_->decode_next_logits_batch(cur.data(), softcap_);
+            for (size_t r = 0; r < R; ++r)
+                nxt[r] = sample_next(lg + r * cfg_.vocab, cfg_.vocab, req.temperature, req.top_k, &rng[r], &sampler_scratch_);
+        }
+        for (size_t r = 0; r < R; ++r) {
+            cur[r] = nxt[r];
+            res[r].generated.push_back(cur[r]);
+            res[r].sampled.push_back(cur[r]);
+        }
+    }
+    ctx_->batch_end();
+    const double elapsed = now_s() - t0;
+    for (size_t r = 0; r < R; ++r) res[r].decode_elapsed = elapsed / (double)R;   // the samples shared every step
+    *out = std::move(res);
+    *done = true;
     return true;
 }
 

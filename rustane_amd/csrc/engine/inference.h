@@ -83,6 +83,10 @@ struct SessionOptions {
     KvDtype kv_dtype = KvDtype::F32;
     int device = 0;
     uint32_t flags = 0;
+    // samples > 1 on the KV-cache path advance together, one weight pass per step for all of them
+    // (the reference runs them one after the other, inference.rs:247-262; results per sample are
+    // the same).  false restores the sequential loop.
+    bool batch_samples = true;
 };
 
 // inference.rs:107-452.  Errors the reference returns as Err(String) come back through `err`
@@ -114,6 +118,10 @@ private:
     bool run_naive_sample(const std::vector<uint32_t> &prompt, const std::vector<float> &prompt_logits,
                           const GenerationRequest &req, uint64_t seed, const StreamCallback *cb, SampleResult *out,
                           std::string *err);
+    // all samples of a request at once; *done = false when the backend has no multi-row path
+    bool run_cached_batch(const std::vector<uint32_t> &prompt, const std::vector<float> &prompt_logits,
+                          const std::vector<uint32_t> &suffix, const GenerationRequest &req,
+                          std::vector<SampleResult> *out, bool *done, std::string *err);
     std::vector<float> window_logits(const std::vector<uint32_t> &ids);   // naive: whole window from position 0
     void restore_prompt_cache();                                          // device KV holds the base prompt again
 
@@ -126,6 +134,7 @@ private:
     std::vector<float> prompt_logits_;
     std::vector<size_t> sampler_scratch_;
     bool prompt_cache_valid_ = false;
+    bool batch_samples_ = true;
 };
 
 }  // namespace rustane

@@ -147,3 +147,40 @@ def test_session_errors():
         s.generate(E.GenerationRequest(samples=0))
     with pytest.raises(E.SessionError, match="prompt suffix token id 5000"):
         s.generate_with_suffix(E.GenerationRequest(), [5000])
+
+
+@pytest.mark.parametrize("T,k,softcap", [(0.0, 0, 0.0), (0.8, 8, 0.0), (0.8, 4, 3.0), (1.0, 0, 2.5), (0.9, 40, 0.0)])
+def test_samples_stepped_together_equal_sequential_samples(T, k, softcap):
+    # The reference draws its samples one after the other (inference.rs:247-262); with bf16 weights
+    # this backend advances them together.  Both orders, and the oracle's loop, must give each
+    # sample the same stream.
+    cfg = tiny_cfg(vocab=1000)
+    prompt = [5, 6, 7, 8, 9, 10, 11, 12, 13]
+    w = synth.make_weights(cfg, seed=31, std=0.08, round_bf16=True)
+    req = E.GenerationRequest(E.DecodeBackendRequest.HIP, steps=10, temperature=T, top_k=k, samples=3, seed=21)
+    together = E.InferenceSession(cfg, w, prompt, softcap=softcap, weight_dtype=1).generate(req)
+    one_by_one = E.InferenceSession(cfg, w, prompt, softcap=softcap, weight_dtype=1, flags=0x100).generate(req)
+    want = oracle_streams(cfg, w, prompt, req, softcap)
+    assert len(together.results) == len(one_by_one.results) == 3
+    for a, b, (sampled, gen) in zip(together.results, one_by_one.results, want):
+        np.testing.assert_array_equal(a.sampled, b.sampled)
+        np.testing.assert_array_equal(a.sampled, sampled)
+        np.testing.assert_array_equal(a.generated, gen)
+        assert a.seed == b.seed
+    assert together.total_decode_elapsed > 0
+
+
+def test_samples_stepped_together_after_a_suffix():
+    cfg = tiny_cfg()
+    w = synth.make_weights(cfg, seed=31, std=0.08, round_bf16=True)
+    base, suffix = [1, 2, 3, 4, 5, 6, 7, 8], [9, 10]
+    req = E.GenerationRequest(E.DecodeBackendRequest.HIP, steps=6, temperature=0.8, top_k=4, samples=4, seed=17)
+    s = E.InferenceSession(cfg, w, base, weight_dtype=1)
+    extended = s.generate_with_suffix(req, suffix)
+    fresh = E.InferenceSession(cfg, w, base + suffix, weight_dtype=1, flags=0x100).generate(req)
+    for a, b in zip(extended.results, fresh.results):
+        np.testing.assert_array_equal(a.generated, b.generated)
+    # the session's prompt cache survives the batch: a second request gives the same streams
+    again = s.generate_with_suffix(req, suffix)
+    for a, b in zip(extended.results, again.results):
+        np.testing.assert_array_equal(a.sampled, b.sampled)
