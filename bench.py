@@ -33,7 +33,54 @@ WORKLOADS = {
     "c4_5b_bf16_bs1": ("config_5b", "BF16", "BF16", 1024, 128),
     "c5_5b_fp8_bs1": ("config_5b", "FP8_E4M3", "BF16", 512, 256),
     "c5_5b_int4_bs1": ("config_5b", "INT4_G128", "BF16", 512, 256),
+    # 8 samples over one shared 512-token prompt, temperature 0.8, top-k 8, stepped together
+    "c3_600m_bf16_8samples": ("config_600m", "BF16", "BF16", 512, 256),
 }
+C3_SAMPLES, C3_TEMPERATURE, C3_TOP_K = 8, 0.8, 8
+
+
+def run_c3(args, cfg, weights, n_prompt):
+    """Multi-sample workload through the session layer: a step is one pass of the weights that
+    advances all 8 samples by one token (top-k candidates on the device, the reference's sampler on
+    the host); value = sampled tokens per second over all samples."""
+    from rustane_amd import engine as E
+    from rustane_amd import synth
+    prompt = synth.make_prompt(7, cfg.vocab, n_prompt)
+    s = E.InferenceSession(cfg, weights, prompt, weight_dtype=1, kv_dtype=1)
+    K, W = args.steps, args.warmup
+    room = cfg.seq - n_prompt - 1
+    K = min(K, room)
+
+    def request(steps, seed):
+        return E.GenerationRequest(E.DecodeBackendRequest.HIP, steps=steps + 1, temperature=C3_TEMPERATURE,
+                                   top_k=C3_TOP_K, samples=C3_SAMPLES, seed=seed)
+    if W > 0:
+        s.generate(request(min(W, room), args.seed))
+    t0 = time.perf_counter()
+    got = s.generate(request(K, args.seed))
+    wall = time.perf_counter() - t0
+    dev_ms = s.batch_device_ms()
+    decode_s = got.total_decode_elapsed
+    mean_kv = n_prompt + (K + 1) // 2
+    w_bytes = s.bytes_per_token(0)
+    bytes_per_step = w_bytes + C3_SAMPLES * (s.bytes_per_token(mean_kv) - w_bytes)
+    achieved = bytes_per_step * K / (dev_ms * 1e-3) / 1e9
+    flops_per_step = 2.0 * C3_SAMPLES * cfg.param_count()              # every weight multiplies every row once
+    return {
+        "metric": "decode tok/s @600M bf16 bs1; % of HBM peak GB/s; prefill ms",
+        "value": C3_SAMPLES * K / decode_s, "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": decode_s * 1e3 / K, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "prompt_tokens": n_prompt, "batch": C3_SAMPLES, "kv_dtype": "bf16",
+                   "temperature": C3_TEMPERATURE, "top_k": C3_TOP_K, "params": cfg.param_count(), "mean_kv_len": mean_kv},
+        "prefill_ms": s.prefill_elapsed() * 1e3, "request_wall_ms": wall * 1e3,
+        "device_ms_per_step": dev_ms / K,
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "bytes_per_step": bytes_per_step},
+        "mfma_roofline": {"bound": "mfma", "achieved": flops_per_step * K / (dev_ms * 1e-3) / 1e12, "peak": 2500.0,
+                          "unit": "TFLOP/s", "frac": flops_per_step * K / (dev_ms * 1e-3) / 2.5e15},
+        "sampled_head": [int(r.sampled[1]) for r in got.results],
+    }
 
 
 def cpu_baseline(cfg, weights, kv_bf16, budget_s=20.0, max_steps=64):
@@ -79,6 +126,9 @@ def main():
     cfg = getattr(synth, cfg_name)()
     wdt, kvdt = WeightDtype[wdt], KvDtype[kvdt]
     weights = synth.make_weights(cfg, seed=args.seed, std=0.02, round_bf16=(wdt != WeightDtype.F32))
+    if args.workload == "c3_600m_bf16_8samples":
+        print(json.dumps(run_c3(args, cfg, weights, n_prompt)))
+        return
     dev = HipDecodeModel(cfg, weights, weight_dtype=wdt, kv_dtype=kvdt)
     prompt = synth.make_prompt(7, cfg.vocab, n_prompt)
 

@@ -125,6 +125,8 @@ int rs_session_generate(rs_session *s, const rs_request *r, const uint32_t *suff
     info->n_results = b.results.size();
     return 0;
 }
+double rs_session_batch_device_ms(const rs_session *s) { return s->s->batch_device_ms(); }
+uint64_t rs_session_bytes_per_token(rs_session *s, size_t kv_len) { return s->s->context()->bytes_per_token(kv_len); }
 uint64_t rs_session_stream_count(const rs_session *s) { return s->stream_count; }
 uint64_t rs_session_result_len(const rs_session *s, size_t i, int which) {
     const SampleResult &r = s->last.results[i];

@@ -394,17 +394,21 @@ bool InferenceSession::run_cached_batch(const std::vector<uint32_t> &prompt, con
         res[r].generated.push_back(cur[r]);
         res[r].sampled.push_back(cur[r]);
     }
+    batch_device_ms_ = 0.0;
     for (size_t i = 1; i < req.steps; ++i) {
         if (req.temperature <= 0.0f || req.top_k == 1) {                           // :576-585
             ctx_->decode_next_greedy_tokens(cur.data(), nxt.data());
+            batch_device_ms_ += ctx_->last_device_ms();
         } else if (req.top_k > 0 && req.top_k <= MAX_GPU_TOPK) {                   // :586-599
             const uint32_t *idxs; const float *lg; const size_t *n;
             ctx_->decode_next_topk_candidates_batch(cur.data(), req.top_k, softcap_, &idxs, &lg, &n);
+            batch_device_ms_ += ctx_->last_device_ms();
             for (size_t r = 0; r < R; ++r)
                 nxt[r] = sample_topk_candidates(idxs + r * MAX_GPU_TOPK, lg + r * MAX_GPU_TOPK, n[r], req.temperature, &rng[r]);
         } else if (req.top_k == 0) {                                               // :600-625
             const float *mx, *sm; size_t nb;
             ctx_->decode_next_fullvocab_block_stats_batch(cur.data(), req.temperature, softcap_, &mx, &sm, &nb);
+            batch_device_ms_ += ctx_->last_device_ms();
             for (size_t r = 0; r < R; ++r) {
                 const size_t blk = sample_block_from_stats(mx + r * nb, sm + r * nb, nb, &rng[r]);
                 const float *bl; size_t nv;
@@ -413,6 +417,7 @@ bool InferenceSession::run_cached_batch(const std::vector<uint32_t> &prompt, con
             }
         } else {                                                                   // :626-638
             const float *lg = ctx_->decode_next_logits_batch(cur.data(), softcap_);
+            batch_device_ms_ += ctx_->last_device_ms();
             for (size_t r = 0; r < R; ++r)
                 nxt[r] = sample_next(lg + r * cfg_.vocab, cfg_.vocab, req.temperature, req.top_k, &rng[r], &sampler_scratch_);
         }

@@ -102,6 +102,8 @@ public:
     float softcap() const { return softcap_; }
     const std::vector<float> &prompt_logits() const { return prompt_logits_; }
     DecodeContext *context() { return ctx_.get(); }
+    // device time (HIP events) summed over the steps of the last request whose samples advanced together
+    double batch_device_ms() const { return batch_device_ms_; }
 
     bool generate(const GenerationRequest &req, GenerationBatch *out, std::string *err);
     bool generate_with_suffix(const GenerationRequest &req, const std::vector<uint32_t> &suffix, GenerationBatch *out,
@@ -135,6 +137,7 @@ private:
     std::vector<size_t> sampler_scratch_;
     bool prompt_cache_valid_ = false;
     bool batch_samples_ = true;
+    double batch_device_ms_ = 0.0;
 };
 
 }  // namespace rustane

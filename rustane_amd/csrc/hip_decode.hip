@@ -33,6 +33,7 @@ struct PrefillWork {
     float *x = nullptr, *x2 = nullptr, *q = nullptr;
     uint16_t *xn_hi = nullptr, *xn_lo = nullptr, *att_hi = nullptr, *att_lo = nullptr, *gate_hi = nullptr,
              *gate_lo = nullptr;
+    float *ssq = nullptr;                // [rows][chunks] sums of squares of the residual rows
     float *P = nullptr;                  // split-K partial planes
     size_t P_floats = 0;
     uint32_t *h_ids = nullptr;           // pinned
@@ -398,9 +399,18 @@ bool prefill_batched_ok(const hipdec_model *m, size_t n) {
 }
 
 struct PfSplit { int splits, steps_per_split; };
+constexpr int kSkinnyRows = 32;          // at most this many rows: the streaming GEMM without LDS tiles
 PfSplit pf_split_k(const hipdec_model *m, int T, int N, int K) {
-    const int tiles = ((N + PF_BN - 1) / PF_BN) * ((T + PF_BM - 1) / PF_BM);
     const int nsteps = K / PF_BK;
+    if (T <= kSkinnyRows) {
+        // 4 waves per workgroup share a K range; aim at ~8 waves per CU over the whole grid
+        const int tiles = (N + 31) / 32;
+        int s = std::max(1, (2 * m->num_cu) / tiles);
+        s = std::min(s, std::max(1, nsteps / 8));
+        const int sps = (nsteps + s - 1) / s;
+        return PfSplit{(nsteps + sps - 1) / sps, sps};
+    }
+    const int tiles = ((N + PF_BN - 1) / PF_BN) * ((T + PF_BM - 1) / PF_BM);
     int s = (2 * m->num_cu + tiles - 1) / tiles;
     s = std::min(s, 8);
     s = std::min(s, std::max(1, nsteps / 8));
@@ -426,6 +436,7 @@ int pf_ensure(hipdec_model *m, int T, bool with_head = false) {
         if ((rc = dalloc(m, &w.att_lo, R * Q * 2))) return rc;
         if ((rc = dalloc(m, &w.gate_hi, R * H * 2))) return rc;
         if ((rc = dalloc(m, &w.gate_lo, R * H * 2))) return rc;
+        if ((rc = dalloc(m, &w.ssq, R * ((D + PF_CHUNK - 1) / PF_CHUNK) * 4))) return rc;
         if (!w.h_ids) HCHK(hipHostMalloc((void **)&w.h_ids, R * 4));
         w.rows = (int)R;
     }
@@ -444,10 +455,46 @@ int pf_ensure(hipdec_model *m, int T, bool with_head = false) {
 int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, const void *W, int T, int N, int K) {
     const PfSplit sp = pf_split_k(m, T, N, K);
     PfGemm g{Ahi, Alo, W, m->pf.P, T, N, K, sp.steps_per_split};
+    if (T <= kSkinnyRows) {
+        dim3 grid((N + 31) / 32, sp.splits), block(256);
+        if (wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_BF16>, grid, block, 0, m->stream, g);
+        else hipLaunchKernelGGL(k_pf_gemm_skinny<WT_FP8>, grid, block, 0, m->stream, g);
+        return sp.splits;
+    }
     dim3 grid((N + PF_BN - 1) / PF_BN, (T + PF_BM - 1) / PF_BM, sp.splits), block(256);
     if (wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm<WT_BF16>, grid, block, 0, m->stream, g);
     else hipLaunchKernelGGL(k_pf_gemm<WT_FP8>, grid, block, 0, m->stream, g);
     return sp.splits;
+}
+
+// launches shared by the prompt prefill and the multi-sample step
+void pf_launch_embed(hipdec_model *m, int T) {
+    PrefillWork &w = m->pf;
+    const int D = (int)m->cfg.dim;
+    dim3 grid((D + PF_CHUNK - 1) / PF_CHUNK, T), block(PF_CHUNK);
+    if (m->embed_wt == WT_F32)
+        hipLaunchKernelGGL(k_pf_embed<WT_F32>, grid, block, 0, m->stream, m->embed, w.ids, w.x, m->layers[0].g1, w.xn_hi,
+                           w.xn_lo, w.ssq, D);
+    else
+        hipLaunchKernelGGL(k_pf_embed<WT_BF16>, grid, block, 0, m->stream, m->embed, w.ids, w.x, m->layers[0].g1, w.xn_hi,
+                           w.xn_lo, w.ssq, D);
+}
+void pf_launch_resid(hipdec_model *m, int T, int splits, const void *wscale, const float *resid, float *out,
+                     const float *gamma) {
+    PrefillWork &w = m->pf;
+    const int D = (int)m->cfg.dim;
+    dim3 grid((D + PF_CHUNK - 1) / PF_CHUNK, T), block(PF_CHUNK);
+    hipLaunchKernelGGL(k_pf_resid, grid, block, 0, m->stream, w.P, splits, (size_t)T * D,
+                       m->wt == WT_FP8 ? (const float *)wscale : nullptr, resid, m->alpha, out, gamma, w.xn_hi, w.xn_lo,
+                       w.ssq, D);
+}
+void pf_launch_gate(hipdec_model *m, int T, int splits, const void *wscale) {
+    PrefillWork &w = m->pf;
+    const int D = (int)m->cfg.dim, H = (int)m->cfg.hidden;
+    const size_t items = (size_t)T * H;
+    hipLaunchKernelGGL(k_pf_gate_epi, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, m->stream, w.P, splits,
+                       (size_t)T * 2 * H, m->wt == WT_FP8 ? (const float *)wscale : nullptr, w.gate_hi, w.gate_lo, w.ssq,
+                       (D + PF_CHUNK - 1) / PF_CHUNK, D, T, H, (int)m->opt.ffn_activation);
 }
 
 // Runs prompt rows ids[0..n) at positions len .. len+n-1 through every layer, chunk by chunk; on
@@ -468,12 +515,8 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
         HCHK(hipStreamSynchronize(m->stream));                  // the pinned id buffer is free again
         memcpy(w.h_ids, ids + done, (size_t)T * 4);
         HCHK(hipMemcpyAsync(w.ids, w.h_ids, (size_t)T * 4, hipMemcpyHostToDevice, m->stream));
-        if (m->embed_wt == WT_F32)
-            hipLaunchKernelGGL(k_pf_embed_norm<WT_F32>, dim3(T), dim3(256), 0, m->stream, m->embed, w.ids, w.x,
-                               m->layers[0].g1, w.xn_hi, w.xn_lo, D);
-        else
-            hipLaunchKernelGGL(k_pf_embed_norm<WT_BF16>, dim3(T), dim3(256), 0, m->stream, m->embed, w.ids, w.x,
-                               m->layers[0].g1, w.xn_hi, w.xn_lo, D);
+        pf_launch_embed(m, T);
+        const int nch = (D + PF_CHUNK - 1) / PF_CHUNK;
         for (uint32_t l = 0; l < c.nlayers; ++l) {
             const DevLayer &L = m->layers[l];
             const bool fp8 = m->wt == WT_FP8;
@@ -486,11 +529,11 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
                 if (m->kvbf16)
                     hipLaunchKernelGGL(k_pf_qkv_epi<1>, grid, block, 0, m->stream, w.P, sp, (size_t)T * N,
                                        fp8 ? (const float *)L.s_qkv : nullptr, w.q, L.kc, L.vc, m->rope_cos, m->rope_sin,
-                                       T, Q, KV, (int)c.hd, pos0);
+                                       w.ssq, nch, D, T, Q, KV, (int)c.hd, pos0);
                 else
                     hipLaunchKernelGGL(k_pf_qkv_epi<0>, grid, block, 0, m->stream, w.P, sp, (size_t)T * N,
                                        fp8 ? (const float *)L.s_qkv : nullptr, w.q, L.kc, L.vc, m->rope_cos, m->rope_sin,
-                                       T, Q, KV, (int)c.hd, pos0);
+                                       w.ssq, nch, D, T, Q, KV, (int)c.hd, pos0);
             }
             // causal attention of the chunk's rows over positions 0 .. pos0 + t
             {
@@ -504,21 +547,13 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
             }
             // output projection, residual, second norm
             sp = pf_gemm(m, m->wt, w.att_hi, w.att_lo, L.wo, T, D, Q);
-            hipLaunchKernelGGL(k_pf_resid_norm, dim3(T), dim3(256), 0, m->stream, w.P, sp, (size_t)T * D,
-                               fp8 ? (const float *)L.s_wo : nullptr, w.x, m->alpha, w.x2, L.g2, w.xn_hi, w.xn_lo, D);
+            pf_launch_resid(m, T, sp, L.s_wo, w.x, w.x2, L.g2);
             // gate/up, activation
             sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.w13, T, 2 * H, D);
-            {
-                const size_t items = (size_t)T * H;
-                hipLaunchKernelGGL(k_pf_gate_epi, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, m->stream, w.P, sp,
-                                   (size_t)T * 2 * H, fp8 ? (const float *)L.s_w13 : nullptr, w.gate_hi, w.gate_lo, T, H,
-                                   (int)m->opt.ffn_activation);
-            }
+            pf_launch_gate(m, T, sp, L.s_w13);
             // down projection, residual, next layer's first norm
             sp = pf_gemm(m, m->wt, w.gate_hi, w.gate_lo, L.w2, T, D, H);
-            const float *gnext = l + 1 < c.nlayers ? m->layers[l + 1].g1 : nullptr;
-            hipLaunchKernelGGL(k_pf_resid_norm, dim3(T), dim3(256), 0, m->stream, w.P, sp, (size_t)T * D,
-                               fp8 ? (const float *)L.s_w2 : nullptr, w.x2, m->alpha, w.x, gnext, w.xn_hi, w.xn_lo, D);
+            pf_launch_resid(m, T, sp, L.s_w2, w.x2, w.x, l + 1 < c.nlayers ? m->layers[l + 1].g1 : nullptr);
         }
         HCHK(hipGetLastError());
         *x_last = w.x + (size_t)(T - 1) * D;
@@ -581,12 +616,8 @@ int batch_step(hipdec_model *m, const uint32_t *tokens, int variant, uint32_t to
     HCHK(hipMemcpyAsync(w.ids, w.h_ids, (size_t)R * 4, hipMemcpyHostToDevice, m->stream));
     HCHK(hipMemcpyAsync(b.d_bp, b.h_bp, sizeof(BatchParams), hipMemcpyHostToDevice, m->stream));
     HCHK(hipEventRecord(m->ev0, m->stream));
-    if (m->embed_wt == WT_F32)
-        hipLaunchKernelGGL(k_pf_embed_norm<WT_F32>, dim3(R), dim3(256), 0, m->stream, m->embed, w.ids, w.x,
-                           m->layers[0].g1, w.xn_hi, w.xn_lo, D);
-    else
-        hipLaunchKernelGGL(k_pf_embed_norm<WT_BF16>, dim3(R), dim3(256), 0, m->stream, m->embed, w.ids, w.x,
-                           m->layers[0].g1, w.xn_hi, w.xn_lo, D);
+    pf_launch_embed(m, R);
+    const int nch = (D + PF_CHUNK - 1) / PF_CHUNK;
     const bool fp8 = m->wt == WT_FP8;
     for (uint32_t l = 0; l < c.nlayers; ++l) {
         const DevLayer &L = m->layers[l];
@@ -598,11 +629,11 @@ int batch_step(hipdec_model *m, const uint32_t *tokens, int variant, uint32_t to
             if (m->kvbf16)
                 hipLaunchKernelGGL(k_bd_qkv_epi<1>, grid, block, 0, m->stream, w.P, sp, (size_t)R * N,
                                    fp8 ? (const float *)L.s_qkv : nullptr, w.q, b.kc_suf[l], b.vc_suf[l], b.suf_rows,
-                                   m->rope_cos, m->rope_sin, b.d_bp, R, Q, KV, (int)c.hd);
+                                   m->rope_cos, m->rope_sin, b.d_bp, w.ssq, nch, D, R, Q, KV, (int)c.hd);
             else
                 hipLaunchKernelGGL(k_bd_qkv_epi<0>, grid, block, 0, m->stream, w.P, sp, (size_t)R * N,
                                    fp8 ? (const float *)L.s_qkv : nullptr, w.q, b.kc_suf[l], b.vc_suf[l], b.suf_rows,
-                                   m->rope_cos, m->rope_sin, b.d_bp, R, Q, KV, (int)c.hd);
+                                   m->rope_cos, m->rope_sin, b.d_bp, w.ssq, nch, D, R, Q, KV, (int)c.hd);
         }
         {
             dim3 grid(c.heads, R), block(256);
@@ -614,27 +645,19 @@ int batch_step(hipdec_model *m, const uint32_t *tokens, int variant, uint32_t to
 #undef BDATT
         }
         sp = pf_gemm(m, m->wt, w.att_hi, w.att_lo, L.wo, R, D, Q);
-        hipLaunchKernelGGL(k_pf_resid_norm, dim3(R), dim3(256), 0, m->stream, w.P, sp, (size_t)R * D,
-                           fp8 ? (const float *)L.s_wo : nullptr, w.x, m->alpha, w.x2, L.g2, w.xn_hi, w.xn_lo, D);
+        pf_launch_resid(m, R, sp, L.s_wo, w.x, w.x2, L.g2);
         sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.w13, R, 2 * H, D);
-        {
-            const size_t items = (size_t)R * H;
-            hipLaunchKernelGGL(k_pf_gate_epi, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, m->stream, w.P, sp,
-                               (size_t)R * 2 * H, fp8 ? (const float *)L.s_w13 : nullptr, w.gate_hi, w.gate_lo, R, H,
-                               (int)m->opt.ffn_activation);
-        }
+        pf_launch_gate(m, R, sp, L.s_w13);
         sp = pf_gemm(m, m->wt, w.gate_hi, w.gate_lo, L.w2, R, D, H);
-        // the last layer's residual kernel applies the final norm instead of the next layer's first one
-        const float *gnext = l + 1 < c.nlayers ? m->layers[l + 1].g1 : m->gfinal;
-        hipLaunchKernelGGL(k_pf_resid_norm, dim3(R), dim3(256), 0, m->stream, w.P, sp, (size_t)R * D,
-                           fp8 ? (const float *)L.s_w2 : nullptr, w.x2, m->alpha, w.x, gnext, w.xn_hi, w.xn_lo, D);
+        // the last layer's residual kernel prepares the final norm instead of the next layer's first one
+        pf_launch_resid(m, R, sp, L.s_w2, w.x2, w.x, l + 1 < c.nlayers ? m->layers[l + 1].g1 : m->gfinal);
     }
     // tied LM head for every row (full_model.rs:419-428), then the per-row head kernel
     {
         const int sp = pf_gemm(m, m->embed_wt, w.xn_hi, w.xn_lo, m->embed, R, V, D);
         const size_t n = (size_t)R * V;
         hipLaunchKernelGGL(k_bd_sum_planes, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, m->stream, w.P, sp, n,
-                           b.logits, n);
+                           b.logits, n, w.ssq, nch, D, V);
     }
     if (variant == B_ARGMAX)
         hipLaunchKernelGGL(k_bd_argmax, dim3(R), dim3(1024), 0, m->stream, b.logits, V, b.d_tok);

@@ -26,7 +26,8 @@ __global__ __launch_bounds__(256) void k_bd_qkv_epi(const float *__restrict__ P,
                                                     const float *__restrict__ wscale, float *__restrict__ q,
                                                     void *__restrict__ kc_suf, void *__restrict__ vc_suf, size_t suf_rows,
                                                     const float *__restrict__ rope_cos, const float *__restrict__ rope_sin,
-                                                    const BatchParams *__restrict__ bp, int R, int Q, int KV, int hd) {
+                                                    const BatchParams *__restrict__ bp, const float *__restrict__ ssq,
+                                                    int nch, int D, int R, int Q, int KV, int hd) {
     const int N = Q + 2 * KV, npairs = N >> 1;
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= (size_t)R * npairs) return;
@@ -37,6 +38,8 @@ __global__ __launch_bounds__(256) void k_bd_qkv_epi(const float *__restrict__ P,
         s0 += v.x; s1 += v.y;
     }
     if (wscale) { s0 *= wscale[row0]; s1 *= wscale[row0 + 1]; }
+    const float inv = pf_row_inv(ssq, t, nch, D);
+    s0 *= inv; s1 *= inv;
     const int pos = bp->pos;
     if (row0 < Q + KV) {
         const int rr = row0 < Q ? row0 : row0 - Q;
@@ -139,14 +142,15 @@ __global__ __launch_bounds__(256) void k_bd_attn(const float *__restrict__ q, co
     }
 }
 
-// logits[r][v] = sum_z P[z][r][v]
+// logits[r][v] = inv_rms[r] * sum_z P[z][r][v]   (the final RMSNorm's row factor, applied after the product)
 __global__ __launch_bounds__(256) void k_bd_sum_planes(const float *__restrict__ P, int splits, size_t plane,
-                                                       float *__restrict__ out, size_t n) {
+                                                       float *__restrict__ out, size_t n, const float *__restrict__ ssq,
+                                                       int nch, int D, int V) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     float s = 0.0f;
     for (int z = 0; z < splits; ++z) s += P[z * plane + i];
-    out[i] = s;
+    out[i] = s * pf_row_inv(ssq, (int)(i / V), nch, D);
 }
 
 // ---- head kernels, one grid row per sequence (same selection rules as the single-row kernels)

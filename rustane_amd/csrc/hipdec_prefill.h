@@ -42,53 +42,57 @@ __device__ __forceinline__ float pf_block_sum(float v, float *red) {
     return t;
 }
 
-// x[t] = embed[ids[t]] (cpu/embedding.rs:8-16), then RMSNorm with the first layer's gamma1
-// (cpu/rmsnorm.rs:149-183) into the hi/lo activation pair.  One workgroup per prompt row.
-template <int EWT>
-__global__ __launch_bounds__(256) void k_pf_embed_norm(const void *__restrict__ embed, const uint32_t *__restrict__ ids,
-                                                       float *__restrict__ x, const float *__restrict__ gamma,
-                                                       uint16_t *__restrict__ hi, uint16_t *__restrict__ lo, int D) {
-    __shared__ float red[8];
-    const int t = blockIdx.x;
-    const size_t tok = ids[t];
-    float ss = 0.0f;
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        float v = EWT == WT_F32 ? ((const float *)embed)[tok * D + d] : bf16_to_f32(((const uint16_t *)embed)[tok * D + d]);
-        x[(size_t)t * D + d] = v;
-        ss += v * v;
-    }
-    ss = pf_block_sum(ss, red);
-    const float inv = 1.0f / sqrtf(ss * (1.0f / (float)D) + 1e-5f);
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        const float v = x[(size_t)t * D + d] * inv * gamma[d];
-        pf_split(v, hi[(size_t)t * D + d], lo[(size_t)t * D + d]);
-    }
+// RMSNorm (cpu/rmsnorm.rs:149-183) is split so that no kernel has to wait for a whole row: the
+// kernel that produces a residual row writes x * gamma as the hi/lo pair and, per 256-element
+// chunk, the sum of squares; the kernel that consumes the following GEMM multiplies its sums by
+// inv[t] = 1 / sqrt(sum_chunks / D + eps), which commutes with the product.
+#define PF_CHUNK 256
+__device__ __forceinline__ float pf_row_inv(const float *__restrict__ ssq, int t, int nch, int D) {
+    float s = 0.0f;
+    for (int c = 0; c < nch; ++c) s += ssq[t * nch + c];
+    return 1.0f / sqrtf(s * (1.0f / (float)D) + 1e-5f);
 }
 
-// out[t][d] = resid[t][d] + alpha * scale[d] * sum_z P[z][t][d]   (layer.rs:1397-1405, :1300), then
-// RMSNorm(out[t]) * gamma into the hi/lo pair for the next GEMM (gamma == nullptr: no norm output).
-__global__ __launch_bounds__(256) void k_pf_resid_norm(const float *__restrict__ P, int splits, size_t plane,
+// x[t] = embed[ids[t]] (cpu/embedding.rs:8-16); hi/lo = x * gamma1 of the first layer; chunk sums of squares.
+// grid (chunks, rows)
+template <int EWT>
+__global__ __launch_bounds__(PF_CHUNK) void k_pf_embed(const void *__restrict__ embed, const uint32_t *__restrict__ ids,
+                                                       float *__restrict__ x, const float *__restrict__ gamma,
+                                                       uint16_t *__restrict__ hi, uint16_t *__restrict__ lo,
+                                                       float *__restrict__ ssq, int D) {
+    __shared__ float red[8];
+    const int t = blockIdx.y, d = blockIdx.x * PF_CHUNK + threadIdx.x;
+    float v = 0.0f;
+    if (d < D) {
+        const size_t tok = ids[t];
+        v = EWT == WT_F32 ? ((const float *)embed)[tok * D + d] : bf16_to_f32(((const uint16_t *)embed)[tok * D + d]);
+        x[(size_t)t * D + d] = v;
+        pf_split(v * gamma[d], hi[(size_t)t * D + d], lo[(size_t)t * D + d]);
+    }
+    const float ss = pf_block_sum(v * v, red);
+    if (threadIdx.x == 0) ssq[t * gridDim.x + blockIdx.x] = ss;
+}
+
+// out[t][d] = resid[t][d] + alpha * scale[d] * sum_z P[z][t][d]   (layer.rs:1397-1405, :1300);
+// hi/lo = out * gamma for the next GEMM (gamma == nullptr: none); chunk sums of squares.  grid (chunks, rows)
+__global__ __launch_bounds__(PF_CHUNK) void k_pf_resid(const float *__restrict__ P, int splits, size_t plane,
                                                        const float *__restrict__ wscale, const float *__restrict__ resid,
                                                        float alpha, float *__restrict__ out, const float *__restrict__ gamma,
-                                                       uint16_t *__restrict__ hi, uint16_t *__restrict__ lo, int D) {
+                                                       uint16_t *__restrict__ hi, uint16_t *__restrict__ lo,
+                                                       float *__restrict__ ssq, int D) {
     __shared__ float red[8];
-    const int t = blockIdx.x;
-    float ss = 0.0f;
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    const int t = blockIdx.y, d = blockIdx.x * PF_CHUNK + threadIdx.x;
+    float v = 0.0f;
+    if (d < D) {
         float s = 0.0f;
         for (int z = 0; z < splits; ++z) s += P[z * plane + (size_t)t * D + d];
         if (wscale) s *= wscale[d];
-        const float v = resid[(size_t)t * D + d] + alpha * s;
+        v = resid[(size_t)t * D + d] + alpha * s;
         out[(size_t)t * D + d] = v;
-        ss += v * v;
+        if (gamma) pf_split(v * gamma[d], hi[(size_t)t * D + d], lo[(size_t)t * D + d]);
     }
-    if (!gamma) return;
-    ss = pf_block_sum(ss, red);
-    const float inv = 1.0f / sqrtf(ss * (1.0f / (float)D) + 1e-5f);
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        const float v = out[(size_t)t * D + d] * inv * gamma[d];
-        pf_split(v, hi[(size_t)t * D + d], lo[(size_t)t * D + d]);
-    }
+    const float ss = pf_block_sum(v * v, red);
+    if (threadIdx.x == 0) ssq[t * gridDim.x + blockIdx.x] = ss;
 }
 
 // q/k/v rows of the chunk: sum the split planes, scale (8-bit weights), RoPE on interleaved pairs
@@ -99,6 +103,7 @@ __global__ __launch_bounds__(256) void k_pf_qkv_epi(const float *__restrict__ P,
                                                     const float *__restrict__ wscale, float *__restrict__ q,
                                                     void *__restrict__ kc, void *__restrict__ vc,
                                                     const float *__restrict__ rope_cos, const float *__restrict__ rope_sin,
+                                                    const float *__restrict__ ssq, int nch, int D,
                                                     int T, int Q, int KV, int hd, int pos0) {
     const int N = Q + 2 * KV, npairs = N >> 1;
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -110,6 +115,8 @@ __global__ __launch_bounds__(256) void k_pf_qkv_epi(const float *__restrict__ P,
         s0 += v.x; s1 += v.y;
     }
     if (wscale) { s0 *= wscale[row0]; s1 *= wscale[row0 + 1]; }
+    const float inv = pf_row_inv(ssq, t, nch, D);
+    s0 *= inv; s1 *= inv;
     const int pos = pos0 + t;
     if (row0 < Q + KV) {
         const int rr = row0 < Q ? row0 : row0 - Q;
@@ -138,7 +145,8 @@ __global__ __launch_bounds__(256) void k_pf_qkv_epi(const float *__restrict__ P,
 // (kernels/ffn_fused.rs:114-150), written as the hi/lo pair the down projection reads.
 __global__ __launch_bounds__(256) void k_pf_gate_epi(const float *__restrict__ P, int splits, size_t plane,
                                                      const float *__restrict__ wscale, uint16_t *__restrict__ hi,
-                                                     uint16_t *__restrict__ lo, int T, int H, int act) {
+                                                     uint16_t *__restrict__ lo, const float *__restrict__ ssq, int nch,
+                                                     int D, int T, int H, int act) {
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= (size_t)T * H) return;
     const int t = (int)(gid / H), j = (int)(gid - (size_t)t * H);
@@ -148,6 +156,8 @@ __global__ __launch_bounds__(256) void k_pf_gate_epi(const float *__restrict__ P
         h1 += v.x; h3 += v.y;
     }
     if (wscale) { h1 *= wscale[2 * j]; h3 *= wscale[2 * j + 1]; }
+    const float inv = pf_row_inv(ssq, t, nch, D);
+    h1 *= inv; h3 *= inv;
     float g;
     if (act == 1) { const float lr = h1 > 0.0f ? h1 : 0.5f * h1; g = lr * lr * h3; }
     else { const float sig = 1.0f / (1.0f + expf(-h1)); g = h1 * sig * h3; }
@@ -281,6 +291,85 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
                 if (t < g.T && n < g.N) Pz[(size_t)t * g.N + n] = acc[mt][nt][i];
             }
         }
+}
+
+// GEMM for at most 32 activation rows (multi-sample decode, short prompts): weight streaming, not
+// matrix throughput, bounds it, so there is no LDS tile and no barrier in the loop.  A workgroup
+// owns 32 weight rows; its four waves split the workgroup's K range and each lane streams its own
+// weight row straight into MFMA operand registers, several steps of loads in flight.  The few
+// activation rows (hi and lo parts) are re-read from cache by every wave; rows past T re-read row
+// T-1 and are not stored.  The four partial tiles are summed through LDS in wave order.
+#define PF_SK_UNROLL 2      // 32-element steps whose loads are issued together
+template <int WT>
+__global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
+    __shared__ float red[4][16][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, gq = lane >> 5;
+    const int n0 = blockIdx.x * 32, z = blockIdx.y;
+    const int nsteps = g.K / PF_BK;
+    const int zb = z * g.steps_per_split, ze = min(nsteps, zb + g.steps_per_split);
+    const int per_wave = (ze - zb + 3) / 4;
+    const int s_begin = min(ze, zb + wave * per_wave), s_end = min(ze, s_begin + per_wave);
+    const size_t na = (size_t)min(n0 + r, g.N - 1), ta = (size_t)min(r, g.T - 1);
+    const uint16_t *ah = g.Ahi + ta * g.K + 16 * gq, *al = g.Alo + ta * g.K + 16 * gq;
+    const char *wp = (const char *)g.W + na * (WT == WT_BF16 ? (size_t)g.K * 2 : (size_t)g.K) + (WT == WT_BF16 ? 32 : 16) * gq;
+
+    pf_f32x16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    for (int s0 = s_begin; s0 < s_end; s0 += PF_SK_UNROLL) {
+        uint4 w[PF_SK_UNROLL][2], xh[PF_SK_UNROLL][2], xl[PF_SK_UNROLL][2];
+#pragma unroll
+        for (int u = 0; u < PF_SK_UNROLL; ++u) {
+            const int s = min(s0 + u, s_end - 1);             // a padded step re-reads the last one (and is skipped below)
+            const size_t k0 = (size_t)s * PF_BK;
+            if (WT == WT_BF16) {
+                w[u][0] = *(const uint4 *)(wp + k0 * 2);
+                w[u][1] = *(const uint4 *)(wp + k0 * 2 + 16);
+            } else {
+                w[u][0] = *(const uint4 *)(wp + k0);
+            }
+            xh[u][0] = *(const uint4 *)(ah + k0); xh[u][1] = *(const uint4 *)(ah + k0 + 8);
+            xl[u][0] = *(const uint4 *)(al + k0); xl[u][1] = *(const uint4 *)(al + k0 + 8);
+        }
+#pragma unroll
+        for (int u = 0; u < PF_SK_UNROLL; ++u) {
+            if (s0 + u < s_end) {
+                uint4 b0, b1;
+                if (WT == WT_BF16) { b0 = w[u][0]; b1 = w[u][1]; }
+                else {
+                    const uint32_t q[4] = {w[u][0].x, w[u][0].y, w[u][0].z, w[u][0].w};
+                    uint32_t o[8];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        auto lo2 = __builtin_amdgcn_cvt_pk_f32_fp8(q[i], false);
+                        auto hi2 = __builtin_amdgcn_cvt_pk_f32_fp8(q[i], true);
+                        o[2 * i] = (__float_as_uint(lo2[0]) >> 16) | (__float_as_uint(lo2[1]) & 0xffff0000u);
+                        o[2 * i + 1] = (__float_as_uint(hi2[0]) >> 16) | (__float_as_uint(hi2[1]) & 0xffff0000u);
+                    }
+                    b0 = make_uint4(o[0], o[1], o[2], o[3]); b1 = make_uint4(o[4], o[5], o[6], o[7]);
+                }
+                const pf_bf16x8 B0 = __builtin_bit_cast(pf_bf16x8, b0), B1 = __builtin_bit_cast(pf_bf16x8, b1);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xh[u][0]), B0, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xl[u][0]), B0, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xh[u][1]), B1, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xl[u][1]), B1, acc, 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) red[wave][i][lane] = acc[i];
+    __syncthreads();
+    // wave w finishes result registers 4w .. 4w+3 (rows 8w + 4*gq + 0..3)
+    float *Pz = g.P + (size_t)z * g.T * g.N;
+    const int n = n0 + r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int i = 4 * wave + j;
+        const float v = ((red[0][i][lane] + red[1][i][lane]) + red[2][i][lane]) + red[3][i][lane];
+        const int t = 8 * wave + 4 * gq + j;
+        if (t < g.T && n < g.N) Pz[(size_t)t * g.N + n] = v;
+    }
 }
 
 // ---------------------------------------------------------------- causal attention over the chunk

@@ -75,6 +75,10 @@ def lib():
         L.rs_session_prompt_logits.argtypes = [C.c_void_p, fp]
         L.rs_session_generate.argtypes = [C.c_void_p, C.POINTER(RsRequest), u32p, C.c_size_t, C.c_int, C.c_uint64,
                                           C.POINTER(RsBatchInfo), C.c_char_p, C.c_size_t]
+        L.rs_session_batch_device_ms.restype = C.c_double
+        L.rs_session_batch_device_ms.argtypes = [C.c_void_p]
+        L.rs_session_bytes_per_token.restype = C.c_uint64
+        L.rs_session_bytes_per_token.argtypes = [C.c_void_p, C.c_size_t]
         L.rs_session_stream_count.restype = C.c_uint64
         L.rs_session_stream_count.argtypes = [C.c_void_p]
         L.rs_session_result_len.restype = C.c_uint64
@@ -249,6 +253,14 @@ class InferenceSession:
         """Streams through a callback inside the engine; it fails the generation once it has seen
         `abort_after` tokens (0 = never).  stream_count() tells how many tokens it was handed."""
         return self._run(req, prompt_suffix, True, abort_after)
+
+    def batch_device_ms(self):
+        """Device time (HIP events) summed over the steps of the last request whose samples advanced together."""
+        return self._L.rs_session_batch_device_ms(self._s)
+
+    def bytes_per_token(self, kv_len):
+        """Bytes one single-row decode step streams at the given live KV length (hipdec_bytes_per_token)."""
+        return int(self._L.rs_session_bytes_per_token(self._s, kv_len))
 
     def stream_count(self):
         return int(self._L.rs_session_stream_count(self._s))
