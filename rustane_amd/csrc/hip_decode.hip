@@ -399,7 +399,8 @@ bool prefill_batched_ok(const hipdec_model *m, size_t n) {
 }
 
 struct PfSplit { int splits, steps_per_split; };
-constexpr int kSkinnyRows = 32;          // at most this many rows: the streaming GEMM without LDS tiles
+constexpr int kSkinnyRows = 32;          // at most this many rows: the streaming GEMM without LDS weight tiles
+constexpr int kSkinnyLdsBytes = 40 * 1024;   // dynamic LDS for the staged activation slice
 PfSplit pf_split_k(const hipdec_model *m, int T, int N, int K) {
     const int nsteps = K / PF_BK;
     if (T <= kSkinnyRows) {
@@ -407,6 +408,9 @@ PfSplit pf_split_k(const hipdec_model *m, int T, int N, int K) {
         const int tiles = (N + 31) / 32;
         int s = std::max(1, (2 * m->num_cu) / tiles);
         s = std::min(s, std::max(1, nsteps / 8));
+        // the workgroup's slice of the activation rows (hi + lo) has to fit its LDS budget
+        const int max_steps = std::max(1, ((kSkinnyLdsBytes / (4 * T)) - PF_SK_PAD) / PF_BK);
+        s = std::max(s, (nsteps + max_steps - 1) / max_steps);
         const int sps = (nsteps + s - 1) / s;
         return PfSplit{(nsteps + sps - 1) / sps, sps};
     }
@@ -457,8 +461,9 @@ int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, c
     PfGemm g{Ahi, Alo, W, m->pf.P, T, N, K, sp.steps_per_split};
     if (T <= kSkinnyRows) {
         dim3 grid((N + 31) / 32, sp.splits), block(256);
-        if (wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_BF16>, grid, block, 0, m->stream, g);
-        else hipLaunchKernelGGL(k_pf_gemm_skinny<WT_FP8>, grid, block, 0, m->stream, g);
+        const size_t lds = (size_t)2 * T * (sp.steps_per_split * PF_BK + PF_SK_PAD) * 2;
+        if (wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_BF16>, grid, block, lds, m->stream, g);
+        else hipLaunchKernelGGL(k_pf_gemm_skinny<WT_FP8>, grid, block, lds, m->stream, g);
         return sp.splits;
     }
     dim3 grid((N + PF_BN - 1) / PF_BN, (T + PF_BM - 1) / PF_BM, sp.splits), block(256);
@@ -636,7 +641,7 @@ int batch_step(hipdec_model *m, const uint32_t *tokens, int variant, uint32_t to
                                    m->rope_cos, m->rope_sin, b.d_bp, w.ssq, nch, D, R, Q, KV, (int)c.hd);
         }
         {
-            dim3 grid(c.heads, R), block(256);
+            dim3 grid(c.heads, R), block(BD_ATT_THREADS);
 #define BDATT(KVB, HD)                                                                                             \
     hipLaunchKernelGGL((k_bd_attn<KVB, HD>), grid, block, 0, m->stream, w.q, L.kc, L.vc, b.kc_suf[l], b.vc_suf[l], \
                        b.suf_rows, b.d_bp, w.att_hi, w.att_lo, Q, KV, gqa, scale)

@@ -68,8 +68,9 @@ __global__ __launch_bounds__(256) void k_bd_qkv_epi(const float *__restrict__ P,
 // One workgroup per (head, row): online softmax over the shared prefix rows and then the row's own
 // suffix rows (same arithmetic as the single-row decode attention; crates/metal-decode/src/lib.rs:1426-1489),
 // result as the hi/lo pair the output projection reads.
+#define BD_ATT_THREADS 1024
 template <int KVBF16, int HD>
-__global__ __launch_bounds__(256) void k_bd_attn(const float *__restrict__ q, const void *__restrict__ kc,
+__global__ __launch_bounds__(BD_ATT_THREADS) void k_bd_attn(const float *__restrict__ q, const void *__restrict__ kc,
                                                  const void *__restrict__ vc, const void *__restrict__ kc_suf,
                                                  const void *__restrict__ vc_suf, size_t suf_rows,
                                                  const BatchParams *__restrict__ bp, uint16_t *__restrict__ ohi,
@@ -78,7 +79,8 @@ __global__ __launch_bounds__(256) void k_bd_attn(const float *__restrict__ q, co
     constexpr int EPL = 16 / ESZ;          // elements per 16-byte load
     constexpr int LPR = HD / EPL;          // lanes per cache row
     constexpr int RPI = 64 / LPR;          // rows per wave instruction
-    constexpr int SLOTS = 4 * RPI;
+    constexpr int SLOTS = (BD_ATT_THREADS / 64) * RPI;
+    constexpr int UNR = 4;                 // cache rows in flight per thread
     __shared__ float sm[SLOTS][HD + 2];
     const int h = blockIdx.x, row = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -97,25 +99,39 @@ __global__ __launch_bounds__(256) void k_bd_attn(const float *__restrict__ q, co
     const char *kb = (const char *)kc + hoff, *vb = (const char *)vc + hoff;
     const char *ksb = (const char *)kc_suf + (size_t)row * suf_rows * rowb + hoff;
     const char *vsb = (const char *)vc_suf + (size_t)row * suf_rows * rowb + hoff;
-    for (int t = wave * RPI + r; t < n; t += SLOTS) {
-        const bool shared = t < prefix;
-        const size_t at = (size_t)(shared ? t : t - prefix) * rowb;
-        const uint4 kw = *(const uint4 *)((shared ? kb : ksb) + at);
-        const uint4 vw = *(const uint4 *)((shared ? vb : vsb) + at);
-        float kf[EPL], vf[EPL];
-        WS<KVBF16 ? WT_BF16 : WT_F32>::decode(kw, kf);
-        WS<KVBF16 ? WT_BF16 : WT_F32>::decode(vw, vf);
-        float d = 0.0f;
+    for (int tb = wave * RPI + r; tb < n; tb += SLOTS * UNR) {
+        uint4 kw[UNR], vw[UNR];
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) d = fmaf(qv[e], kf[e], d);
+        for (int u = 0; u < UNR; ++u) {
+            const int t = tb + u * SLOTS;
+            if (t < n) {
+                const bool shared = t < prefix;
+                const size_t at = (size_t)(shared ? t : t - prefix) * rowb;
+                kw[u] = *(const uint4 *)((shared ? kb : ksb) + at);
+                vw[u] = *(const uint4 *)((shared ? vb : vsb) + at);
+            }
+        }
 #pragma unroll
-        for (int o = LPR >> 1; o > 0; o >>= 1) d += __shfl_xor(d, o, WAVE);
-        const float mn = fmaxf(m, d);
-        const float corr = __expf(m - mn), p = __expf(d - mn);
-        l = l * corr + p;
+        for (int u = 0; u < UNR; ++u) {
+            // the rows of one lane group are either all present or all past the end, so the
+            // reduction below stays inside converged lanes
+            if (tb + u * SLOTS < n) {
+                float kf[EPL], vf[EPL];
+                WS<KVBF16 ? WT_BF16 : WT_F32>::decode(kw[u], kf);
+                WS<KVBF16 ? WT_BF16 : WT_F32>::decode(vw[u], vf);
+                float d = 0.0f;
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) acc[e] = acc[e] * corr + p * vf[e];
-        m = mn;
+                for (int e = 0; e < EPL; ++e) d = fmaf(qv[e], kf[e], d);
+#pragma unroll
+                for (int o = LPR >> 1; o > 0; o >>= 1) d += __shfl_xor(d, o, WAVE);
+                const float mn = fmaxf(m, d);
+                const float corr = __expf(m - mn), p = __expf(d - mn);
+                l = l * corr + p;
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) acc[e] = acc[e] * corr + p * vf[e];
+                m = mn;
+            }
+        }
     }
     {
         const int slot = wave * RPI + r;

@@ -296,13 +296,16 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
 // GEMM for at most 32 activation rows (multi-sample decode, short prompts): weight streaming, not
 // matrix throughput, bounds it, so there is no LDS tile and no barrier in the loop.  A workgroup
 // owns 32 weight rows; its four waves split the workgroup's K range and each lane streams its own
-// weight row straight into MFMA operand registers, several steps of loads in flight.  The few
-// activation rows (hi and lo parts) are re-read from cache by every wave; rows past T re-read row
-// T-1 and are not stored.  The four partial tiles are summed through LDS in wave order.
-#define PF_SK_UNROLL 2      // 32-element steps whose loads are issued together
+// weight row straight into MFMA operand registers, several steps of loads in flight.  The
+// workgroup's slice of the few activation rows (hi and lo parts) is staged once in LDS while the
+// first weight loads are in flight; rows past T read row T-1 and are not stored.  The four partial
+// tiles are summed through LDS in wave order.
+#define PF_SK_UNROLL 4     // 32-element steps whose loads are issued together
+#define PF_SK_PAD 8        // bf16 elements of padding per staged activation row
 template <int WT>
 __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
     __shared__ float red[4][16][64];
+    extern __shared__ __align__(16) uint16_t s_act[];      // [2][T][krange + PF_SK_PAD]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, gq = lane >> 5;
     const int n0 = blockIdx.x * 32, z = blockIdx.y;
@@ -310,15 +313,14 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
     const int zb = z * g.steps_per_split, ze = min(nsteps, zb + g.steps_per_split);
     const int per_wave = (ze - zb + 3) / 4;
     const int s_begin = min(ze, zb + wave * per_wave), s_end = min(ze, s_begin + per_wave);
-    const size_t na = (size_t)min(n0 + r, g.N - 1), ta = (size_t)min(r, g.T - 1);
-    const uint16_t *ah = g.Ahi + ta * g.K + 16 * gq, *al = g.Alo + ta * g.K + 16 * gq;
+    const size_t na = (size_t)min(n0 + r, g.N - 1);
+    const int krange = (ze - zb) * PF_BK, astride = g.steps_per_split * PF_BK + PF_SK_PAD;
+    const uint16_t *ah = s_act + min(r, g.T - 1) * astride + 16 * gq;
+    const uint16_t *al = ah + g.T * astride;
     const char *wp = (const char *)g.W + na * (WT == WT_BF16 ? (size_t)g.K * 2 : (size_t)g.K) + (WT == WT_BF16 ? 32 : 16) * gq;
 
-    pf_f32x16 acc;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
-    for (int s0 = s_begin; s0 < s_end; s0 += PF_SK_UNROLL) {
-        uint4 w[PF_SK_UNROLL][2], xh[PF_SK_UNROLL][2], xl[PF_SK_UNROLL][2];
+    uint4 w[PF_SK_UNROLL][2];
+    auto wload = [&](int s0) {
 #pragma unroll
         for (int u = 0; u < PF_SK_UNROLL; ++u) {
             const int s = min(s0 + u, s_end - 1);             // a padded step re-reads the last one (and is skipped below)
@@ -329,6 +331,32 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
             } else {
                 w[u][0] = *(const uint4 *)(wp + k0);
             }
+        }
+    };
+    if (s_begin < s_end) wload(s_begin);
+    // stage activation rows [0, T) x this workgroup's K range
+    {
+        const int cpr = krange / 8;                           // 16-byte chunks per row
+        for (int c = tid; c < g.T * cpr; c += 256) {
+            const int t = c / cpr, kc = c - t * cpr;
+            const size_t src = (size_t)t * g.K + (size_t)zb * PF_BK + kc * 8;
+            *(uint4 *)(s_act + t * astride + kc * 8) = *(const uint4 *)(g.Ahi + src);
+            *(uint4 *)(s_act + (g.T + t) * astride + kc * 8) = *(const uint4 *)(g.Alo + src);
+        }
+    }
+    __syncthreads();
+
+    pf_f32x16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    for (int s0 = s_begin; s0 < s_end; s0 += PF_SK_UNROLL) {
+        uint4 wc[PF_SK_UNROLL][2], xh[PF_SK_UNROLL][2], xl[PF_SK_UNROLL][2];
+#pragma unroll
+        for (int u = 0; u < PF_SK_UNROLL; ++u) { wc[u][0] = w[u][0]; wc[u][1] = w[u][1]; }
+        if (s0 + PF_SK_UNROLL < s_end) wload(s0 + PF_SK_UNROLL);   // next group in flight while this one multiplies
+#pragma unroll
+        for (int u = 0; u < PF_SK_UNROLL; ++u) {
+            const int k0 = (min(s0 + u, s_end - 1) - zb) * PF_BK;
             xh[u][0] = *(const uint4 *)(ah + k0); xh[u][1] = *(const uint4 *)(ah + k0 + 8);
             xl[u][0] = *(const uint4 *)(al + k0); xl[u][1] = *(const uint4 *)(al + k0 + 8);
         }
@@ -336,9 +364,9 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
         for (int u = 0; u < PF_SK_UNROLL; ++u) {
             if (s0 + u < s_end) {
                 uint4 b0, b1;
-                if (WT == WT_BF16) { b0 = w[u][0]; b1 = w[u][1]; }
+                if (WT == WT_BF16) { b0 = wc[u][0]; b1 = wc[u][1]; }
                 else {
-                    const uint32_t q[4] = {w[u][0].x, w[u][0].y, w[u][0].z, w[u][0].w};
+                    const uint32_t q[4] = {wc[u][0].x, wc[u][0].y, wc[u][0].z, wc[u][0].w};
                     uint32_t o[8];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
