@@ -1,0 +1,70 @@
+"""Full-size known answers (tests/golden/*.json, written by tests/golden/make_fullsize_vectors.py):
+the CPU oracle must keep reproducing them (CPU suite), and the HIP backend must match them on the
+600M-class benchmark model through the C ABI (GPU suite) -- chunked matrix-core prefill, then the
+persistent decode kernel, greedy stream identical and prompt logits within 1e-4 of the largest
+logit with an fp32 cache, 2e-3 with a bf16 cache (a 1-ulp difference can flip a cached value's bf16
+rounding)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from rustane_amd import synth
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+CASES = ["c2_600m_bf16_std002", "c2_600m_bf16_std005_kvf32"]
+
+
+def load(name):
+    with open(os.path.join(GOLDEN, name + ".json")) as f:
+        return json.load(f)
+
+
+def model_inputs(g):
+    cfg = getattr(synth, g["config"])()
+    w = synth.make_weights(cfg, seed=g["weight_seed"], std=g["weight_std"], round_bf16=True)
+    ids = synth.make_prompt(g["prompt_seed"], cfg.vocab, g["prompt_tokens"])
+    assert [int(x) for x in ids[:8]] == g["prompt_head"]
+    return cfg, w, ids
+
+
+def check_logits(g, lg, tol):
+    scale = g["logit_abs_max"]
+    top_i = np.array(g["top_logit_indices"])
+    top_v = np.array(g["top_logit_values"])
+    assert np.abs(lg[top_i] - top_v).max() <= tol * scale
+    # nothing outside the recorded set may beat its smallest member by more than the tolerance
+    rest = np.delete(lg, top_i)
+    assert rest.max() <= top_v.min() + tol * scale
+    assert abs(float(np.abs(lg.astype(np.float64)).sum()) - g["logit_abs_sum"]) <= tol * g["logit_abs_sum"]
+
+
+def test_oracle_reproduces_the_fullsize_vector():
+    g = load("c2_600m_bf16_std005_kvf32")
+    cfg, w, ids = model_inputs(g)
+    orc = O.Oracle(cfg, w, kv_round_bf16=(g["kv_cache"] == "bf16"))
+    lg, _, _ = orc.forward_window(ids)
+    check_logits(g, lg[0], 1e-5)
+    sampled, _ = orc.run_cached_sample(ids, lg[0], len(g["greedy_stream"]))
+    assert [int(t) for t in sampled] == g["greedy_stream"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", CASES)
+@pytest.mark.parametrize("prefill_steps", [False, True])
+def test_hip_backend_matches_the_fullsize_vector(name, prefill_steps):
+    from rustane_amd.hipdec import HipDecodeModel, KvDtype, WeightDtype
+    g = load(name)
+    cfg, w, ids = model_inputs(g)
+    bf16_cache = g["kv_cache"] == "bf16"
+    dev = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.BF16 if bf16_cache else KvDtype.F32,
+                         flags=4 if prefill_steps else 0)
+    lg = dev.prefill(ids)
+    check_logits(g, lg, 2e-3 if bf16_cache else 1e-4)
+    want = g["greedy_stream"]
+    first = int(np.argmax(lg))
+    assert first == want[0]
+    got = dev.decode_greedy_run(first, len(want) - 1)
+    assert [int(t) for t in got] == want[1:]
