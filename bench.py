@@ -38,6 +38,11 @@ WORKLOADS = {
 }
 C3_SAMPLES, C3_TEMPERATURE, C3_TOP_K = 8, 0.8, 8
 
+# HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, each
+# scaled by what the same counter reads for a plain copy of known size): measured separately with
+# rocprofv3 --pmc and recorded in profiles/k_mega_c2_600m_bf16_bs1.md; a benchmark run cannot collect it itself.
+MEASURED_TRAFFIC_BYTES = {"c2_600m_bf16_bs1": 1.514e9}
+
 
 def run_c3(args, cfg, weights, n_prompt):
     """Multi-sample workload through the session layer: a step is one pass of the weights that
@@ -193,7 +198,7 @@ def main():
                              "frac": prefill_flops / (prefill_dev_ms * 1e-3) / mfma_peak},
         "device_ms_per_step": dev_ms / K,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "bytes_per_step": bytes_per_step},
     }
     if not args.no_cpu_baseline:
