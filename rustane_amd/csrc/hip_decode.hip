@@ -54,6 +54,8 @@ struct BatchState {
     float *h_stage = nullptr;            // pinned, cap_rows * max(vocab, 2 * blocks * 32) floats
     size_t h_stage_floats = 0;
     bool have_logits = false;            // a step has run since hipdec_batch_begin
+    hipGraphExec_t graphs[4] = {};       // one captured step per head variant, for graph_rows rows
+    int graph_rows = 0;
 };
 
 }  // namespace
@@ -599,6 +601,8 @@ int batch_alloc(hipdec_model *m, int rows) {
     return HIPDEC_OK;
 }
 
+void batch_enqueue(hipdec_model *m, int variant);
+
 // one step of every open row: tokens[r] at position prefix + slot
 int batch_step(hipdec_model *m, const uint32_t *tokens, int variant, uint32_t top_k, float inv_t, float softcap) {
     const hipdec_config &c = m->cfg;
@@ -609,9 +613,6 @@ int batch_step(hipdec_model *m, const uint32_t *tokens, int variant, uint32_t to
     const int R = b.rows;
     for (int r = 0; r < R; ++r)
         if (tokens[r] >= c.vocab) return fail(m, HIPDEC_ERR_ARG, "token id must fit vocab");
-    const int D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden, V = c.vocab;
-    const int gqa = c.gqa_ratio ? c.gqa_ratio : 1;
-    const float scale = 1.0f / sqrtf((float)c.hd);
     int rc = pf_ensure(m, R, true);
     if (rc) return rc;
     PrefillWork &w = m->pf;
@@ -621,6 +622,43 @@ int batch_step(hipdec_model *m, const uint32_t *tokens, int variant, uint32_t to
     HCHK(hipMemcpyAsync(w.ids, w.h_ids, (size_t)R * 4, hipMemcpyHostToDevice, m->stream));
     HCHK(hipMemcpyAsync(b.d_bp, b.h_bp, sizeof(BatchParams), hipMemcpyHostToDevice, m->stream));
     HCHK(hipEventRecord(m->ev0, m->stream));
+    // Everything that changes from step to step (tokens, position, sampler parameters) was just
+    // written to device memory, so the ~210 launches of a step are captured once per (rows, head
+    // variant) and replayed.
+    if (m->opt.flags & HIPDEC_FLAG_NO_GRAPH) {
+        batch_enqueue(m, variant);
+        HCHK(hipGetLastError());
+    } else {
+        if (b.graph_rows != R) {
+            for (auto &g : b.graphs) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
+            b.graph_rows = R;
+        }
+        if (!b.graphs[variant]) {
+            hipGraph_t g = nullptr;
+            HCHK(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
+            batch_enqueue(m, variant);
+            hipError_t e = hipStreamEndCapture(m->stream, &g);
+            if (e != hipSuccess || !g) { m->err = std::string("graph capture failed: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+            HCHK(hipGraphInstantiate(&b.graphs[variant], g, nullptr, nullptr, 0));
+            HCHK(hipGraphDestroy(g));
+        }
+        HCHK(hipGraphLaunch(b.graphs[variant], m->stream));
+    }
+    HCHK(hipEventRecord(m->ev1, m->stream));
+    b.slot += 1;
+    b.have_logits = true;
+    return HIPDEC_OK;
+}
+
+// the kernels of one multi-row step (no host-side state changes: safe to capture)
+void batch_enqueue(hipdec_model *m, int variant) {
+    const hipdec_config &c = m->cfg;
+    BatchState &b = m->bt;
+    PrefillWork &w = m->pf;
+    const int R = b.rows;
+    const int D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden, V = c.vocab;
+    const int gqa = c.gqa_ratio ? c.gqa_ratio : 1;
+    const float scale = 1.0f / sqrtf((float)c.hd);
     pf_launch_embed(m, R);
     const int nch = (D + PF_CHUNK - 1) / PF_CHUNK;
     const bool fp8 = m->wt == WT_FP8;
@@ -671,11 +709,6 @@ int batch_step(hipdec_model *m, const uint32_t *tokens, int variant, uint32_t to
     else if (variant == B_STATS)
         hipLaunchKernelGGL(k_bd_block_stats, dim3(m->blocks, R), dim3(256), 0, m->stream, b.logits, V, b.d_bp, b.d_bmax,
                            b.d_bsum);
-    HCHK(hipGetLastError());
-    HCHK(hipEventRecord(m->ev1, m->stream));
-    b.slot += 1;
-    b.have_logits = true;
-    return HIPDEC_OK;
 }
 
 // copies `floats` values from device memory to the caller through the pinned staging buffer
@@ -699,6 +732,7 @@ void hipdec_destroy(hipdec_model *m) {
     if (!m) return;
     if (m->stream) (void)hipStreamSynchronize(m->stream);
     for (auto &g : m->graphs) if (g) (void)hipGraphExecDestroy(g);
+    for (auto &g : m->bt.graphs) if (g) (void)hipGraphExecDestroy(g);
     for (void *p : m->allocs) (void)hipFree(p);
     if (m->h_sp) (void)hipHostFree(m->h_sp);
     if (m->h_out) (void)hipHostFree(m->h_out);
