@@ -417,12 +417,13 @@ PfSplit pf_split_k(const hipdec_model *m, int T, int N, int K) {
         return PfSplit{(nsteps + sps - 1) / sps, sps};
     }
     const int tiles = ((N + PF_BN - 1) / PF_BN) * ((T + PF_BM - 1) / PF_BM);
+    const int lsteps = (K + PF_BKL - 1) / PF_BKL;
     int s = (2 * m->num_cu + tiles - 1) / tiles;
     s = std::min(s, 8);
-    s = std::min(s, std::max(1, nsteps / 8));
+    s = std::min(s, std::max(1, lsteps / 4));
     s = std::max(s, 1);
-    const int sps = (nsteps + s - 1) / s;
-    return PfSplit{(nsteps + sps - 1) / sps, sps};
+    const int sps = (lsteps + s - 1) / s;
+    return PfSplit{(lsteps + sps - 1) / sps, sps};
 }
 
 int pf_ensure(hipdec_model *m, int T, bool with_head = false) {

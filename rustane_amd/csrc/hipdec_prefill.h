@@ -23,8 +23,10 @@ typedef float pf_f32x16 __attribute__((ext_vector_type(16)));
 
 #define PF_BM 128           // prompt rows per GEMM workgroup tile
 #define PF_BN 128           // weight rows (output channels) per GEMM workgroup tile
-#define PF_BK 32            // reduction elements per step
-#define PF_LDS_STRIDE 40    // bf16 elements per LDS tile row (80 bytes: 16-byte aligned, spreads rows over banks)
+#define PF_BK 32            // reduction elements per step of the streaming (few-row) GEMM; K must be a multiple
+#define PF_BKL 64           // reduction elements per step of the tiled GEMM
+#define PF_LDS_STRIDE 72    // bf16 elements per LDS tile row (144 bytes: 16-byte aligned; 16 consecutive rows
+                            // start 36 banks apart, so a 128-bit operand read by 16 lanes touches every bank once)
 
 __device__ __forceinline__ void pf_split(float v, uint16_t &hi, uint16_t &lo) {
     hi = f32_to_bf16_rne(v);
@@ -170,7 +172,7 @@ struct PfGemm {
     const void *W;               // weights [N][K], bf16 or e4m3
     float *P;                    // partial planes [splits][T][N]
     int T, N, K;
-    int steps_per_split;         // PF_BK-steps of the reduction each blockIdx.z covers
+    int steps_per_split;         // reduction steps (PF_BKL tiled, PF_BK streaming) each K split covers
 };
 
 __device__ __forceinline__ pf_bf16x8 pf_frag(const uint16_t *p) {
@@ -190,7 +192,7 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int n0 = blockIdx.x * PF_BN, t0 = blockIdx.y * PF_BM, z = blockIdx.z;
-    const int nsteps = g.K / PF_BK;
+    const int nsteps = (g.K + PF_BKL - 1) / PF_BKL;
     const int s_begin = z * g.steps_per_split, s_end = min(nsteps, s_begin + g.steps_per_split);
 
     pf_f32x16 acc[2][2];
@@ -201,65 +203,69 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.0f;
 
-    // global -> register staging of the next tiles.  Activation tiles: 128 rows x 4 chunks of 8
-    // elements, two chunks per thread for hi and for lo.  Weight tile: bf16 the same; e4m3 128 rows
-    // x 2 chunks of 16 elements, one per thread.  Rows past the end re-read the last valid row;
-    // their results are not stored.
-    uint4 rah[2], ral[2], rw[2];
-    auto gload = [&](int step) {
-        const int k0 = step * PF_BK;
+    // global -> register staging, two steps ahead of the multiply.  Activation tiles: 128 rows x 8
+    // chunks of 8 elements, four chunks per thread for hi and for lo.  Weight tile: bf16 the same;
+    // e4m3 128 rows x 4 chunks of 16 elements, two per thread.  Rows past the end re-read the last
+    // valid row (their results are not stored); chunks past K are zero.
+    struct Stage { uint4 ah[4], al[4], w[4]; };
+    const uint4 zero4 = make_uint4(0, 0, 0, 0);
+    auto gload = [&](Stage &s, int step) {
+        const int k0 = step * PF_BKL;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int c = tid + 256 * j, row = c >> 2, kc = c & 3;
+        for (int j = 0; j < 4; ++j) {
+            const int c = tid + 256 * j, row = c >> 3, k = k0 + (c & 7) * 8;
             const size_t ta = (size_t)min(t0 + row, g.T - 1);
-            rah[j] = *(const uint4 *)(g.Ahi + ta * g.K + k0 + kc * 8);
-            ral[j] = *(const uint4 *)(g.Alo + ta * g.K + k0 + kc * 8);
-            if (WT == WT_BF16) {
+            s.ah[j] = zero4; s.al[j] = zero4; s.w[j] = zero4;
+            if (k < g.K) {
+                s.ah[j] = *(const uint4 *)(g.Ahi + ta * g.K + k);
+                s.al[j] = *(const uint4 *)(g.Alo + ta * g.K + k);
+                if (WT == WT_BF16) {
+                    const size_t na = (size_t)min(n0 + row, g.N - 1);
+                    s.w[j] = *(const uint4 *)((const uint16_t *)g.W + na * g.K + k);
+                }
+            }
+        }
+        if (WT == WT_FP8) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int c = tid + 256 * j, row = c >> 2, k = k0 + (c & 3) * 16;
                 const size_t na = (size_t)min(n0 + row, g.N - 1);
-                rw[j] = *(const uint4 *)((const uint16_t *)g.W + na * g.K + k0 + kc * 8);
+                if (k < g.K) s.w[j] = *(const uint4 *)((const uint8_t *)g.W + na * g.K + k);
             }
         }
-        if (WT == WT_FP8) {
-            const int row = tid >> 1, half = tid & 1;
-            const size_t na = (size_t)min(n0 + row, g.N - 1);
-            rw[0] = *(const uint4 *)((const uint8_t *)g.W + na * g.K + k0 + half * 16);
-        }
     };
-    auto lstore = [&]() {
+    auto lstore = [&](const Stage &s) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int c = tid + 256 * j, row = c >> 2, kc = c & 3;
-            *(uint4 *)(sAh + row * PF_LDS_STRIDE + kc * 8) = rah[j];
-            *(uint4 *)(sAl + row * PF_LDS_STRIDE + kc * 8) = ral[j];
-            if (WT == WT_BF16) *(uint4 *)(sW + row * PF_LDS_STRIDE + kc * 8) = rw[j];
+        for (int j = 0; j < 4; ++j) {
+            const int c = tid + 256 * j, row = c >> 3, kc = c & 7;
+            *(uint4 *)(sAh + row * PF_LDS_STRIDE + kc * 8) = s.ah[j];
+            *(uint4 *)(sAl + row * PF_LDS_STRIDE + kc * 8) = s.al[j];
+            if (WT == WT_BF16) *(uint4 *)(sW + row * PF_LDS_STRIDE + kc * 8) = s.w[j];
         }
         if (WT == WT_FP8) {
-            const int row = tid >> 1, half = tid & 1;
-            const uint32_t u[4] = {rw[0].x, rw[0].y, rw[0].z, rw[0].w};
-            uint32_t o[8];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                auto lo2 = __builtin_amdgcn_cvt_pk_f32_fp8(u[i], false);
-                auto hi2 = __builtin_amdgcn_cvt_pk_f32_fp8(u[i], true);
-                // e4m3 values are exact in bf16: keep the upper halves of the fp32 patterns
-                o[2 * i] = (__float_as_uint(lo2[0]) >> 16) | (__float_as_uint(lo2[1]) & 0xffff0000u);
-                o[2 * i + 1] = (__float_as_uint(hi2[0]) >> 16) | (__float_as_uint(hi2[1]) & 0xffff0000u);
+            for (int j = 0; j < 2; ++j) {
+                const int c = tid + 256 * j, row = c >> 2, q = c & 3;
+                const uint32_t u[4] = {s.w[j].x, s.w[j].y, s.w[j].z, s.w[j].w};
+                uint32_t o[8];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    auto lo2 = __builtin_amdgcn_cvt_pk_f32_fp8(u[i], false);
+                    auto hi2 = __builtin_amdgcn_cvt_pk_f32_fp8(u[i], true);
+                    // e4m3 values are exact in bf16: keep the upper halves of the fp32 patterns
+                    o[2 * i] = (__float_as_uint(lo2[0]) >> 16) | (__float_as_uint(lo2[1]) & 0xffff0000u);
+                    o[2 * i + 1] = (__float_as_uint(hi2[0]) >> 16) | (__float_as_uint(hi2[1]) & 0xffff0000u);
+                }
+                uint16_t *dst = sW + row * PF_LDS_STRIDE + q * 16;
+                *(uint4 *)dst = make_uint4(o[0], o[1], o[2], o[3]);
+                *(uint4 *)(dst + 8) = make_uint4(o[4], o[5], o[6], o[7]);
             }
-            uint16_t *dst = sW + row * PF_LDS_STRIDE + half * 16;
-            *(uint4 *)dst = make_uint4(o[0], o[1], o[2], o[3]);
-            *(uint4 *)(dst + 8) = make_uint4(o[4], o[5], o[6], o[7]);
         }
     };
-
-    if (s_begin < s_end) gload(s_begin);
-    for (int step = s_begin; step < s_end; ++step) {
-        __syncthreads();                       // the previous step's operand reads are done
-        lstore();
-        __syncthreads();
-        if (step + 1 < s_end) gload(step + 1); // in flight while this step multiplies
+    auto multiply = [&]() {
         const int r = lane & 31, kq = 8 * (lane >> 5);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < PF_BKL / 16; ++j) {
             pf_bf16x8 b[2], ah[2], al[2];
 #pragma unroll
             for (int nt = 0; nt < 2; ++nt) b[nt] = pf_frag(sW + (64 * wn + 32 * nt + r) * PF_LDS_STRIDE + 16 * j + kq);
@@ -275,6 +281,25 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
                     acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mt], b[nt], acc[mt][nt], 0, 0, 0);
                     acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], b[nt], acc[mt][nt], 0, 0, 0);
                 }
+        }
+    };
+
+    Stage S0, S1;
+    const int n = s_end - s_begin;
+    if (n > 0) gload(S0, s_begin);
+    if (n > 1) gload(S1, s_begin + 1);
+    for (int i = 0; i < n; i += 2) {
+        __syncthreads();                       // the previous step's operand reads are done
+        lstore(S0);
+        __syncthreads();
+        if (i + 2 < n) gload(S0, s_begin + i + 2);   // two steps in flight while this one multiplies
+        multiply();
+        if (i + 1 < n) {
+            __syncthreads();
+            lstore(S1);
+            __syncthreads();
+            if (i + 3 < n) gload(S1, s_begin + i + 3);
+            multiply();
         }
     }
 
