@@ -88,24 +88,90 @@ def run_c3(args, cfg, weights, n_prompt):
     }
 
 
-def cpu_baseline(cfg, weights, kv_bf16, budget_s=20.0, max_steps=64):
-    """Times the oracle's KV-cached token loop (the CPU restatement of the reference's arithmetic)
-    from an empty cache; the weight stream dominates its cost, so the rate barely depends on the
-    position.  Returns the cpu_baseline object."""
+def cpu_baseline(cfg, weights, kv_bf16, prompt=None, gpu_stream=None, budget_s=20.0, max_steps=64):
+    """Times the oracle's KV-cached greedy loop (the CPU restatement of the reference's arithmetic) on
+    this box's host cores.  With a prompt (the small workloads) the oracle replays the workload itself
+    -- window forward over the prompt, then greedy steps -- and its tokens are compared with the
+    GPU's stream; otherwise it steps from an empty cache (the weight stream dominates the cost, so the
+    rate barely depends on the position).  Returns the cpu_baseline object."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle_lib as O
     orc = O.Oracle(cfg, weights, kv_round_bf16=kv_bf16)
-    tok, n, t0 = 1, 0, time.perf_counter()
-    while n < max_steps and n < cfg.seq:
+    extra, tok = {}, 1
+    if prompt is not None:
+        lg, _, _ = orc.forward_window(prompt)
+        tok = int(O.argmax_last(lg[0]))
+        cpu_stream = [tok]
+    n, t0 = 0, time.perf_counter()
+    while n < max_steps and orc.len() < cfg.seq:
         lg = orc.decode_logits_from_id(tok)
         tok = int(O.argmax_lower(lg))
         n += 1
+        if prompt is not None:
+            cpu_stream.append(tok)
         if time.perf_counter() - t0 > budget_s:
             break
     dt = time.perf_counter() - t0
+    if prompt is not None and gpu_stream is not None:
+        m = min(len(cpu_stream), len(gpu_stream))
+        div = next((i for i in range(m) if cpu_stream[i] != int(gpu_stream[i])), None)
+        extra = {"greedy_tokens_compared": m, "first_divergence_step": div}
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    return {"value": n / dt, "unit": "tok/s", "cores": cores, "kind": "port",
-            "sample": "%d KV-cached greedy steps of the same model from an empty cache, fp32 CPU oracle" % n}
+    what = "after the workload's prompt" if prompt is not None else "from an empty cache"
+    out = {"value": n / dt, "unit": "tok/s", "cores": cores, "kind": "port",
+           "sample": "%d KV-cached greedy steps of the same model %s, fp32 CPU oracle" % (n, what)}
+    out.update(extra)
+    return out
+
+
+def run_c4_sampled(args, cfg, dev, kvdt, prompt_logits, n_prompt, gen_steps, prefill_dev_ms, prefill_wall_ms,
+                   prefill_flops, mfma_peak):
+    """The 5B workload as defined: full-vocabulary sampling at temperature 1.0 through the exact
+    block-stats path (crates/engine/src/inference.rs:600-625) -- per token one decode step that
+    leaves per-block (max, sum exp) on the device, a block drawn on the host, that block's logits
+    fetched, the token drawn inside it (two uniforms per token, the reference's LCG, seed 1)."""
+    import ctypes as C
+    from rustane_amd import engine as E
+    L = E.lib()
+    fp = C.POINTER(C.c_float)
+    rng = C.c_uint64(1)
+    T = 1.0
+    lg = np.ascontiguousarray(prompt_logits, np.float32)
+    cur = int(L.rs_sample_next(lg.ctypes.data_as(fp), lg.size, T, 0, C.byref(rng)))
+    K, W = args.steps, args.warmup
+    K = min(K, gen_steps - 1, cfg.seq - n_prompt - W - 1)
+
+    def step(tok):
+        mx, sm = dev.decode_token_block_stats_from_id(tok, 1.0 / T, 0.0)
+        ms = dev.last_device_ms()
+        blk = int(L.rs_sample_block_from_stats(mx.ctypes.data_as(fp), sm.ctypes.data_as(fp), mx.size, C.byref(rng)))
+        bl = dev.materialize_current_logits_block(blk, 0.0)
+        return int(L.rs_sample_block_logits(blk * 256, bl.ctypes.data_as(fp), bl.size, T, C.byref(rng))), ms
+    for _ in range(W):
+        cur, _ = step(cur)
+    kv0 = dev.len()
+    dev_ms, t0 = 0.0, time.perf_counter()
+    for _ in range(K):
+        cur, ms = step(cur)
+        dev_ms += ms
+    wall = time.perf_counter() - t0
+    mean_kv = kv0 + (K + 1) // 2
+    bytes_per_step = dev.bytes_per_token(mean_kv)
+    achieved = bytes_per_step * K / (dev_ms * 1e-3) / 1e9
+    return {
+        "metric": "decode tok/s @600M bf16 bs1; % of HBM peak GB/s; prefill ms",
+        "value": K / wall, "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": wall * 1e3 / K,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "prompt_tokens": n_prompt, "batch": 1, "kv_dtype": kvdt.name.lower(),
+                   "sampler": "full-vocab block stats, temperature 1.0", "params": cfg.param_count(), "mean_kv_len": mean_kv},
+        "prefill_ms": prefill_dev_ms, "prefill_wall_ms": prefill_wall_ms,
+        "prefill_roofline": {"bound": "mfma", "achieved": prefill_flops / (prefill_dev_ms * 1e-3) / 1e12,
+                             "peak": mfma_peak / 1e12, "unit": "TFLOP/s",
+                             "frac": prefill_flops / (prefill_dev_ms * 1e-3) / mfma_peak},
+        "device_ms_per_step": dev_ms / K,
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "bytes_per_step": bytes_per_step},
+    }
 
 
 def main():
@@ -154,6 +220,10 @@ def main():
 
     room = cfg.seq - n_prompt
     K, W = args.steps, args.warmup
+    if args.workload == "c4_5b_bf16_bs1":
+        print(json.dumps(run_c4_sampled(args, cfg, dev, kvdt, logits, n_prompt, gen_steps, prefill_dev_ms, prefill_wall_ms,
+                                        prefill_flops, mfma_peak)))
+        return
     if W > 0:
         dev.decode_greedy_run(first, min(W, room))
     # timed region: exactly K greedy steps, in runs that restart at the end of the prompt so every
@@ -164,8 +234,10 @@ def main():
         n = min(run_len, K - done)
         dev.set_len(n_prompt)
         t0 = time.perf_counter()
-        dev.decode_greedy_run(first, n)
+        run = dev.decode_greedy_run(first, n)
         wall += time.perf_counter() - t0
+        if done == 0:
+            gpu_stream = [first] + [int(t) for t in run]
         dev_ms += dev.last_device_ms()
         kv_sum += sum(range(n_prompt + 1, n_prompt + n + 1))
         done += n
@@ -202,7 +274,9 @@ def main():
                      "bytes_per_step": bytes_per_step},
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cfg, weights, kvdt == KvDtype.BF16)
+        replay = args.workload in ("c1_tiny_fp32", "c2_600m_bf16_bs1")      # the oracle can afford the prompt here
+        out["cpu_baseline"] = cpu_baseline(cfg, weights, kvdt == KvDtype.BF16, prompt if replay else None,
+                                           gpu_stream if replay else None)
     print(json.dumps(out))
 
 

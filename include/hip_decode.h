@@ -170,8 +170,9 @@ int hipdec_materialize_current_logits_block_batch(hipdec_model *m, size_t row, s
  * out_tokens[n_steps].  Equivalent to n_steps calls of hipdec_decode_token_argmax_from_id. */
 int hipdec_decode_greedy_run(hipdec_model *m, uint32_t token, size_t n_steps, uint32_t *out_tokens);
 
-/* Per-step device time of the last hipdec_decode_greedy_run / hipdec_prefill, measured with HIP
- * events on the model's stream: total milliseconds over that call. */
+/* Device time of the last call that ran a step (a single decode step, a multi-row step,
+ * hipdec_decode_greedy_run, hipdec_prefill), measured with HIP events on the model's stream: total
+ * milliseconds of that call's kernels. */
 int hipdec_last_device_ms(const hipdec_model *m, float *out_ms);
 
 /* Bytes of device memory the model streams per decoded token at the given live KV length

@@ -83,6 +83,8 @@ struct hipdec_model {
     float alpha = 1.0f;
     hipGraphExec_t graphs[V_COUNT] = {};
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    hipEvent_t ev_s0 = nullptr, ev_s1 = nullptr;      // around a single step
+    bool step_timed = false;
     float last_ms = 0.0f;
     // persistent one-launch-per-token step (hipdec_mega.h)
     bool mega_ok = false;
@@ -344,7 +346,12 @@ int run_step(hipdec_model *m, int variant) {
 int step_with(hipdec_model *m, int variant, size_t slot, const StepParams &p) {
     m->h_sp[slot] = p;
     HCHK(hipMemcpyAsync(m->d_sp, &m->h_sp[slot], sizeof(StepParams), hipMemcpyHostToDevice, m->stream));
-    return run_step(m, variant);
+    HCHK(hipEventRecord(m->ev_s0, m->stream));
+    int rc = run_step(m, variant);
+    if (rc) return rc;
+    HCHK(hipEventRecord(m->ev_s1, m->stream));
+    m->step_timed = true;
+    return HIPDEC_OK;
 }
 
 int check_step(hipdec_model *m, uint32_t token, bool from_id) {
@@ -364,6 +371,10 @@ StepParams base_params(hipdec_model *m, uint32_t token) {
 // stream sync after a step; a persistent-kernel wait that timed out shows up as an error here
 int sync_checked(hipdec_model *m) {
     HCHK(hipStreamSynchronize(m->stream));
+    if (m->step_timed) {           // device time of the single step that was just waited for
+        m->step_timed = false;
+        HCHK(hipEventElapsedTime(&m->last_ms, m->ev_s0, m->ev_s1));
+    }
     if (m->mega_ok) {
         unsigned flag = 0;
         HCHK(hipMemcpy(&flag, m->d_epochs + 2, 4, hipMemcpyDeviceToHost));
@@ -742,6 +753,8 @@ void hipdec_destroy(hipdec_model *m) {
     if (m->bt.h_stage) (void)hipHostFree(m->bt.h_stage);
     if (m->ev0) (void)hipEventDestroy(m->ev0);
     if (m->ev1) (void)hipEventDestroy(m->ev1);
+    if (m->ev_s0) (void)hipEventDestroy(m->ev_s0);
+    if (m->ev_s1) (void)hipEventDestroy(m->ev_s1);
     if (m->stream) (void)hipStreamDestroy(m->stream);
     delete m;
 }
@@ -756,6 +769,8 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
     HCHK(hipStreamCreate(&m->stream));
     HCHK(hipEventCreate(&m->ev0));
     HCHK(hipEventCreate(&m->ev1));
+    HCHK(hipEventCreate(&m->ev_s0));
+    HCHK(hipEventCreate(&m->ev_s1));
 
     size_t max_elems = V * D;
     if (D * H > max_elems) max_elems = D * H;
