@@ -405,8 +405,9 @@ bool prefill_batched_ok(const hipdec_model *m, size_t n) {
     const hipdec_config &c = m->cfg;
     if (m->opt.flags & HIPDEC_FLAG_PREFILL_STEPS) return false;
     if (n < (size_t)kPrefillMinRows) return false;
-    if (m->wt != WT_BF16 && m->wt != WT_FP8) return false;          // fp32 and 4-bit weights: token steps
+    if (m->wt == WT_F32) return false;                               // fp32 weights: token steps
     if (c.dim % PF_BK || c.q_dim % PF_BK || c.hidden % PF_BK) return false;
+    if (m->wt == WT_INT4 && (c.dim % 128 || c.q_dim % 128 || c.hidden % 128)) return false;   // whole scale groups
     if (c.hd != 64 && c.hd != 128) return false;
     return true;
 }
@@ -414,9 +415,9 @@ bool prefill_batched_ok(const hipdec_model *m, size_t n) {
 struct PfSplit { int splits, steps_per_split; };
 constexpr int kSkinnyRows = 32;          // at most this many rows: the streaming GEMM without LDS weight tiles
 constexpr int kSkinnyLdsBytes = 40 * 1024;   // dynamic LDS for the staged activation slice
-PfSplit pf_split_k(const hipdec_model *m, int T, int N, int K) {
+PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K) {
     const int nsteps = K / PF_BK;
-    if (T <= kSkinnyRows) {
+    if (T <= kSkinnyRows && wt != WT_INT4) {      // (4-bit weights always take the tiled kernel)
         // 4 waves per workgroup share a K range; aim at ~8 waves per CU over the whole grid
         const int tiles = (N + 31) / 32;
         int s = std::max(1, (2 * m->num_cu) / tiles);
@@ -433,7 +434,8 @@ PfSplit pf_split_k(const hipdec_model *m, int T, int N, int K) {
     s = std::min(s, 8);
     s = std::min(s, std::max(1, lsteps / 4));
     s = std::max(s, 1);
-    const int sps = (lsteps + s - 1) / s;
+    int sps = (lsteps + s - 1) / s;
+    if (wt == WT_INT4) sps = (sps + 1) & ~1;       // a split covers whole scale groups (two steps each)
     return PfSplit{(lsteps + sps - 1) / sps, sps};
 }
 
@@ -460,8 +462,8 @@ int pf_ensure(hipdec_model *m, int T, bool with_head = false) {
     }
     size_t need = 0;
     const int dims[4][2] = {{(int)(Q + 2 * KV), (int)D}, {(int)D, (int)Q}, {(int)(2 * H), (int)D}, {(int)D, (int)H}};
-    for (auto &d : dims) need = std::max(need, (size_t)pf_split_k(m, T, d[0], d[1]).splits * T * d[0]);
-    if (with_head) need = std::max(need, (size_t)pf_split_k(m, T, (int)c.vocab, (int)D).splits * T * c.vocab);
+    for (auto &d : dims) need = std::max(need, (size_t)pf_split_k(m, m->wt, T, d[0], d[1]).splits * T * d[0]);
+    if (with_head) need = std::max(need, (size_t)pf_split_k(m, m->embed_wt, T, (int)c.vocab, (int)D).splits * T * c.vocab);
     if (need > w.P_floats) {
         if ((rc = dalloc(m, &w.P, need * 4))) return rc;
         w.P_floats = need;
@@ -470,10 +472,11 @@ int pf_ensure(hipdec_model *m, int T, bool with_head = false) {
 }
 
 // P[z][t][n] = sum over the z-th K slice of A[t][k] * W[n][k]; returns the number of planes
-int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, const void *W, int T, int N, int K) {
-    const PfSplit sp = pf_split_k(m, T, N, K);
-    PfGemm g{Ahi, Alo, W, m->pf.P, T, N, K, sp.steps_per_split};
-    if (T <= kSkinnyRows) {
+int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, const void *W, const void *scales,
+            int T, int N, int K) {
+    const PfSplit sp = pf_split_k(m, wt, T, N, K);
+    PfGemm g{Ahi, Alo, W, wt == WT_INT4 ? (const uint16_t *)scales : nullptr, m->pf.P, T, N, K, sp.steps_per_split};
+    if (T <= kSkinnyRows && wt != WT_INT4) {
         dim3 grid((N + 31) / 32, sp.splits), block(256);
         const size_t lds = (size_t)2 * T * (sp.steps_per_split * PF_BK + PF_SK_PAD) * 2;
         if (wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_BF16>, grid, block, lds, m->stream, g);
@@ -482,7 +485,8 @@ int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, c
     }
     dim3 grid((N + PF_BN - 1) / PF_BN, (T + PF_BM - 1) / PF_BM, sp.splits), block(256);
     if (wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm<WT_BF16>, grid, block, 0, m->stream, g);
-    else hipLaunchKernelGGL(k_pf_gemm<WT_FP8>, grid, block, 0, m->stream, g);
+    else if (wt == WT_FP8) hipLaunchKernelGGL(k_pf_gemm<WT_FP8>, grid, block, 0, m->stream, g);
+    else hipLaunchKernelGGL(k_pf_gemm<WT_INT4>, grid, block, 0, m->stream, g);
     return sp.splits;
 }
 
@@ -541,7 +545,7 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
             const bool fp8 = m->wt == WT_FP8;
             // q/k/v projections, RoPE, cache append
             int N = Q + 2 * KV;
-            int sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.wqkv, T, N, D);
+            int sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.wqkv, L.s_qkv, T, N, D);
             {
                 const size_t items = (size_t)T * (N / 2);
                 dim3 grid((unsigned)((items + 255) / 256)), block(256);
@@ -565,13 +569,13 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
 #undef PFATT
             }
             // output projection, residual, second norm
-            sp = pf_gemm(m, m->wt, w.att_hi, w.att_lo, L.wo, T, D, Q);
+            sp = pf_gemm(m, m->wt, w.att_hi, w.att_lo, L.wo, L.s_wo, T, D, Q);
             pf_launch_resid(m, T, sp, L.s_wo, w.x, w.x2, L.g2);
             // gate/up, activation
-            sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.w13, T, 2 * H, D);
+            sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.w13, L.s_w13, T, 2 * H, D);
             pf_launch_gate(m, T, sp, L.s_w13);
             // down projection, residual, next layer's first norm
-            sp = pf_gemm(m, m->wt, w.gate_hi, w.gate_lo, L.w2, T, D, H);
+            sp = pf_gemm(m, m->wt, w.gate_hi, w.gate_lo, L.w2, L.s_w2, T, D, H);
             pf_launch_resid(m, T, sp, L.s_w2, w.x2, w.x, l + 1 < c.nlayers ? m->layers[l + 1].g1 : nullptr);
         }
         HCHK(hipGetLastError());
@@ -677,7 +681,7 @@ void batch_enqueue(hipdec_model *m, int variant) {
     for (uint32_t l = 0; l < c.nlayers; ++l) {
         const DevLayer &L = m->layers[l];
         const int N = Q + 2 * KV;
-        int sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.wqkv, R, N, D);
+        int sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.wqkv, L.s_qkv, R, N, D);
         {
             const size_t items = (size_t)R * (N / 2);
             dim3 grid((unsigned)((items + 255) / 256)), block(256);
@@ -699,17 +703,17 @@ void batch_enqueue(hipdec_model *m, int variant) {
             else { if (c.hd == 64) BDATT(0, 64); else BDATT(0, 128); }
 #undef BDATT
         }
-        sp = pf_gemm(m, m->wt, w.att_hi, w.att_lo, L.wo, R, D, Q);
+        sp = pf_gemm(m, m->wt, w.att_hi, w.att_lo, L.wo, L.s_wo, R, D, Q);
         pf_launch_resid(m, R, sp, L.s_wo, w.x, w.x2, L.g2);
-        sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.w13, R, 2 * H, D);
+        sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.w13, L.s_w13, R, 2 * H, D);
         pf_launch_gate(m, R, sp, L.s_w13);
-        sp = pf_gemm(m, m->wt, w.gate_hi, w.gate_lo, L.w2, R, D, H);
+        sp = pf_gemm(m, m->wt, w.gate_hi, w.gate_lo, L.w2, L.s_w2, R, D, H);
         // the last layer's residual kernel prepares the final norm instead of the next layer's first one
         pf_launch_resid(m, R, sp, L.s_w2, w.x2, w.x, l + 1 < c.nlayers ? m->layers[l + 1].g1 : m->gfinal);
     }
     // tied LM head for every row (full_model.rs:419-428), then the per-row head kernel
     {
-        const int sp = pf_gemm(m, m->embed_wt, w.xn_hi, w.xn_lo, m->embed, R, V, D);
+        const int sp = pf_gemm(m, m->embed_wt, w.xn_hi, w.xn_lo, m->embed, nullptr, R, V, D);
         const size_t n = (size_t)R * V;
         hipLaunchKernelGGL(k_bd_sum_planes, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, m->stream, w.P, sp, n,
                            b.logits, n, w.ssq, nch, D, V);
@@ -1198,7 +1202,7 @@ int hipdec_batch_begin(hipdec_model *m, size_t n_rows) {
     if (!m) return HIPDEC_ERR_ARG;
     if (n_rows == 0 || n_rows > (size_t)kBatchMaxRows) return fail(m, HIPDEC_ERR_ARG, "n_rows must be in 1..32");
     if (!prefill_batched_ok(m, kPrefillMinRows))
-        return fail(m, HIPDEC_ERR_UNSUPPORTED, "multi-row decode needs bf16 or e4m3 weights and dimensions that are multiples of 32");
+        return fail(m, HIPDEC_ERR_UNSUPPORTED, "multi-row decode needs bf16, e4m3 or 4-bit weights and dimensions that are multiples of 32 (128 with 4-bit weights)");
     if (m->len >= m->cfg.seq) return fail(m, HIPDEC_ERR_FULL, "decode only supports lengths within cfg.seq");
     int rc = batch_alloc(m, (int)n_rows);
     if (rc) return rc;

@@ -169,7 +169,8 @@ __global__ __launch_bounds__(256) void k_pf_gate_epi(const float *__restrict__ P
 // ---------------------------------------------------------------- GEMM on the bf16 matrix cores
 struct PfGemm {
     const uint16_t *Ahi, *Alo;   // activations [T][K], hi and lo parts
-    const void *W;               // weights [N][K], bf16 or e4m3
+    const void *W;               // weights [N][K]: bf16, e4m3, or 4-bit (two per byte)
+    const uint16_t *S;           // 4-bit weights: bf16 scale per row and 128 reduction elements, [N][K/128]
     float *P;                    // partial planes [splits][T][N]
     int T, N, K;
     int steps_per_split;         // reduction steps (PF_BKL tiled, PF_BK streaming) each K split covers
@@ -202,6 +203,18 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
         for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.0f;
+    // 4-bit weights enter the matrix cores as the exact integers -8..7; the products of one scale
+    // group (128 reduction elements = two steps) are summed separately and scaled once, in fp32,
+    // like the per-piece scale of the decode GEMV
+    pf_f32x16 accg[WT == WT_INT4 ? 2 : 1][WT == WT_INT4 ? 2 : 1];
+    if (WT == WT_INT4) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) accg[a % (WT == WT_INT4 ? 2 : 1)][b % (WT == WT_INT4 ? 2 : 1)][i] = 0.0f;
+    }
 
     // global -> register staging, two steps ahead of the multiply.  Activation tiles: 128 rows x 8
     // chunks of 8 elements, four chunks per thread for hi and for lo.  Weight tile: bf16 the same;
@@ -233,6 +246,11 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
                 if (k < g.K) s.w[j] = *(const uint4 *)((const uint8_t *)g.W + na * g.K + k);
             }
         }
+        if (WT == WT_INT4) {       // 128 rows x 2 halves of 32 elements (16 bytes)
+            const int row = tid >> 1, k = k0 + (tid & 1) * 32;
+            const size_t na = (size_t)min(n0 + row, g.N - 1);
+            if (k < g.K) s.w[0] = *(const uint4 *)((const uint8_t *)g.W + na * (size_t)(g.K / 2) + k / 2);
+        }
     };
     auto lstore = [&](const Stage &s) {
 #pragma unroll
@@ -261,6 +279,24 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
                 *(uint4 *)(dst + 8) = make_uint4(o[4], o[5], o[6], o[7]);
             }
         }
+        if (WT == WT_INT4) {
+            // nibble n (offset-binary, element 2j = low nibble of byte j) -> bf16 bits of the integer n - 8:
+            // 2^23 + n is exact in fp32, subtracting 2^23 + 8 leaves n - 8, whose upper 16 bits are its bf16 form
+            const int row = tid >> 1, half = tid & 1;
+            const uint32_t u[4] = {s.w[0].x, s.w[0].y, s.w[0].z, s.w[0].w};
+            uint16_t *dst = sW + row * PF_LDS_STRIDE + half * 32;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                uint32_t o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float f0 = __uint_as_float(0x4B000000u | ((u[i] >> (8 * e)) & 0xfu)) - 8388616.0f;
+                    const float f1 = __uint_as_float(0x4B000000u | ((u[i] >> (8 * e + 4)) & 0xfu)) - 8388616.0f;
+                    o[e] = (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xffff0000u);
+                }
+                *(uint4 *)(dst + 8 * i) = make_uint4(o[0], o[1], o[2], o[3]);
+            }
+        }
     };
     auto multiply = [&]() {
         const int r = lane & 31, kq = 8 * (lane >> 5);
@@ -278,9 +314,32 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                 for (int nt = 0; nt < 2; ++nt) {
-                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mt], b[nt], acc[mt][nt], 0, 0, 0);
-                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], b[nt], acc[mt][nt], 0, 0, 0);
+                    if (WT == WT_INT4) {
+                        pf_f32x16 &t = accg[mt % (WT == WT_INT4 ? 2 : 1)][nt % (WT == WT_INT4 ? 2 : 1)];
+                        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mt], b[nt], t, 0, 0, 0);
+                        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], b[nt], t, 0, 0, 0);
+                    } else {
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mt], b[nt], acc[mt][nt], 0, 0, 0);
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], b[nt], acc[mt][nt], 0, 0, 0);
+                    }
                 }
+        }
+    };
+    // 4-bit weights: the group that steps (i, i + 1) of this split make up, scaled into the result.
+    // Result register columns are weight rows (lane % 32), so the scale is one value per lane and tile.
+    auto scale_group = [&](int step) {
+        if (WT != WT_INT4) return;
+        const int grp = step / (128 / PF_BKL), kg = g.K / 128;
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+            const size_t na = (size_t)min(n0 + 64 * wn + 32 * nt + (lane & 31), g.N - 1);
+            const float sc = __uint_as_float((uint32_t)g.S[na * kg + grp] << 16);
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+                pf_f32x16 &t = accg[mt % (WT == WT_INT4 ? 2 : 1)][nt % (WT == WT_INT4 ? 2 : 1)];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) { acc[mt][nt][i] = fmaf(t[i], sc, acc[mt][nt][i]); t[i] = 0.0f; }
+            }
         }
     };
 
@@ -301,6 +360,7 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
             if (i + 3 < n) gload(S1, s_begin + i + 3);
             multiply();
         }
+        scale_group(s_begin + i);              // (splits of 4-bit weights start on a group boundary)
     }
 
     float *Pz = g.P + (size_t)z * g.T * g.N;

@@ -19,7 +19,11 @@ def rel_err(a, b):
 
 def setup(cfg, rows, n_prompt, wdt=WeightDtype.BF16, kvdt=KvDtype.F32, std=0.07, seed=17):
     w = synth.make_weights(cfg, seed=seed, std=std, round_bf16=True)
-    wo = O.dequantised_weights(cfg, w, "fp8")[0] if wdt == WeightDtype.FP8_E4M3 else w
+    wo = w
+    if wdt == WeightDtype.FP8_E4M3:
+        wo = O.dequantised_weights(cfg, w, "fp8")[0]
+    if wdt == WeightDtype.INT4_G128:
+        wo = O.dequantised_weights(cfg, w, "int4")[0]
     dev = HipDecodeModel(cfg, w, weight_dtype=wdt, kv_dtype=kvdt)
     ids = synth.make_prompt(3, cfg.vocab, n_prompt)
     dev.prefill(ids, want_logits=False)
@@ -91,9 +95,9 @@ def test_batched_head_variants_match_oracle():
     dev.batch_end()
 
 
-def test_batched_bf16_cache_and_fp8_weights():
+def test_batched_bf16_cache_and_quantised_weights():
     cfg = Config.make(dim=512, hidden=1024, heads=4, hd=128, seq=96, nlayers=2, vocab=512)
-    for wdt in (WeightDtype.BF16, WeightDtype.FP8_E4M3):
+    for wdt in (WeightDtype.BF16, WeightDtype.FP8_E4M3, WeightDtype.INT4_G128):
         rows = 2
         w, dev, orcs, ids = setup(cfg, rows, 33, wdt=wdt, kvdt=KvDtype.BF16, std=0.05)
         dev.batch_begin(rows)

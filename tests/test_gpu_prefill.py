@@ -24,6 +24,8 @@ def make(cfg, wdt=WeightDtype.BF16, kvdt=KvDtype.F32, std=0.06, seed=31, act=0, 
     wo = w
     if wdt == WeightDtype.FP8_E4M3:
         wo, _ = O.dequantised_weights(cfg, w, "fp8")
+    if wdt == WeightDtype.INT4_G128:
+        wo, _ = O.dequantised_weights(cfg, w, "int4")
     orc = O.Oracle(cfg, wo, kv_round_bf16=(kvdt == KvDtype.BF16), ffn_activation=act)
     dev = HipDecodeModel(cfg, w, weight_dtype=wdt, kv_dtype=kvdt, ffn_activation=act, flags=flags)
     return w, orc, dev
@@ -64,6 +66,27 @@ def test_prefill_bf16_cache():
 def test_prefill_fp8_weights():
     cfg = Config.make(dim=512, hidden=1024, heads=4, hd=128, seq=128, nlayers=2, vocab=512)
     check_prefill_then_decode(cfg, 65, 2e-3, wdt=WeightDtype.FP8_E4M3, kvdt=KvDtype.BF16, std=0.05)
+
+
+@pytest.mark.parametrize("n_prompt", [20, 65, 140])
+def test_prefill_int4_weights(n_prompt):
+    # 4-bit weights enter the matrix cores as exact integers and are scaled per group in fp32, so the
+    # result is fp32-grade against the oracle run on the de-quantised weights
+    cfg = Config.make(dim=512, hidden=1024, heads=4, hd=128, seq=160, nlayers=2, vocab=512)
+    check_prefill_then_decode(cfg, n_prompt, 1e-4, wdt=WeightDtype.INT4_G128, kvdt=KvDtype.F32, std=0.05)
+
+
+def test_prefill_int4_matches_token_step_prefill():
+    cfg = Config.make(dim=384, hidden=1152, heads=3, hd=128, seq=200, nlayers=3, vocab=1024)
+    w = synth.make_weights(cfg, seed=5, std=0.06, round_bf16=True)
+    ids = synth.make_prompt(4, cfg.vocab, 150)
+    a = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.INT4_G128, kv_dtype=KvDtype.BF16)
+    b = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.INT4_G128, kv_dtype=KvDtype.BF16, flags=FLAG_PREFILL_STEPS)
+    la, lb = a.prefill(ids), b.prefill(ids)
+    assert rel_err(la, lb) < 2e-3                 # bf16 cache: a 1-ulp difference can flip a cached rounding
+    ta = a.decode_greedy_run(int(np.argmax(la)), 16)
+    tb = b.decode_greedy_run(int(np.argmax(lb)), 16)
+    np.testing.assert_array_equal(ta, tb)
 
 
 def test_prefill_in_two_calls_equals_one():
