@@ -1,0 +1,155 @@
+#include "checkpoint.h"
+
+#include <errno.h>
+#include <fcntl.h>
+#include <string.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <cstdio>
+
+namespace rustane {
+namespace {
+
+constexpr uint32_t kVersion = 2;                  // checkpoint.rs:15
+constexpr size_t kHeaderV1 = 4 + 6 * 4;           // :16
+constexpr size_t kHeaderV2 = 4 + 7 * 4;           // :17
+
+bool bad(std::string *err, const std::string &msg) {
+    if (err) *err = msg;
+    return false;
+}
+
+// checkpoint.rs:216-225
+bool read_u32(const uint8_t *b, size_t len, size_t *cur, uint32_t *v, std::string *err) {
+    if (*cur + 4 > len) return bad(err, "unexpected EOF reading u32");
+    *v = (uint32_t)b[*cur] | ((uint32_t)b[*cur + 1] << 8) | ((uint32_t)b[*cur + 2] << 16) | ((uint32_t)b[*cur + 3] << 24);
+    *cur += 4;
+    return true;
+}
+
+// checkpoint.rs:227-247 (the host is little-endian, as every machine this backend runs on)
+bool read_f32_vec(const uint8_t *b, size_t len, size_t *cur, size_t count, std::vector<float> *out, std::string *err) {
+    if (count > (SIZE_MAX >> 2)) return bad(err, "checkpoint tensor size overflow");
+    const size_t bytes = count * 4;
+    if (bytes > len - *cur) return bad(err, "unexpected EOF reading tensor with " + std::to_string(count) + " f32 values");
+    out->resize(count);
+    memcpy(out->data(), b + *cur, bytes);
+    *cur += bytes;
+    return true;
+}
+
+// checkpoint.rs:168-214
+bool infer_hidden(size_t dim, size_t nlayers, size_t vocab, size_t payload_floats, size_t *hidden, std::string *err) {
+    size_t fixed, layer_fixed, denom;
+    if (__builtin_mul_overflow(vocab, dim, &fixed) || __builtin_add_overflow(fixed, dim, &fixed))
+        return bad(err, "checkpoint dimensions overflow");
+    if (__builtin_mul_overflow((size_t)4, dim, &layer_fixed) || __builtin_mul_overflow(layer_fixed, dim, &layer_fixed) ||
+        __builtin_add_overflow(layer_fixed, 2 * dim, &layer_fixed))
+        return bad(err, "checkpoint dimensions overflow");
+    size_t all_layers;
+    if (__builtin_mul_overflow(nlayers, layer_fixed, &all_layers) || __builtin_add_overflow(all_layers, fixed, &all_layers))
+        return bad(err, "checkpoint dimensions overflow");
+    if (payload_floats < all_layers) return bad(err, "checkpoint payload too small for fixed-size tensors");
+    const size_t hidden_total = payload_floats - all_layers;
+    if (__builtin_mul_overflow(nlayers, (size_t)3, &denom) || __builtin_mul_overflow(denom, dim, &denom))
+        return bad(err, "checkpoint dimensions overflow");
+    if (denom == 0 || hidden_total % denom != 0)
+        return bad(err, "checkpoint payload does not imply an integer hidden size");
+    *hidden = hidden_total / denom;
+    if (*hidden == 0) return bad(err, "checkpoint hidden size inferred as zero");
+    return true;
+}
+
+}  // namespace
+
+bool parse_checkpoint(const uint8_t *bytes, size_t len, Checkpoint *out, std::string *err) {
+    if (len < kHeaderV1) return bad(err, "checkpoint too small for header");
+    if (memcmp(bytes, "RSTK", 4) != 0) return bad(err, "invalid checkpoint magic");
+    size_t cur = 4;
+    uint32_t version, step, dim, nlayers, vocab, seq, code = 0;
+    if (!read_u32(bytes, len, &cur, &version, err)) return false;
+    if (version < 1 || version > kVersion) return bad(err, "unsupported checkpoint version " + std::to_string(version));
+    if (version >= 2 && len < kHeaderV2) return bad(err, "checkpoint too small for v2 header");
+    if (!read_u32(bytes, len, &cur, &step, err) || !read_u32(bytes, len, &cur, &dim, err) ||
+        !read_u32(bytes, len, &cur, &nlayers, err) || !read_u32(bytes, len, &cur, &vocab, err) ||
+        !read_u32(bytes, len, &cur, &seq, err))
+        return false;
+    FfnActivation act = FfnActivation::SwiGlu;             // version 1 has no activation field
+    if (version >= 2) {
+        if (!read_u32(bytes, len, &cur, &code, err)) return false;
+        if (code > 1) return bad(err, "unsupported checkpoint activation code " + std::to_string(code));   // model.rs:17-23
+        act = (FfnActivation)code;
+    }
+    if (dim == 0 || nlayers == 0 || vocab == 0 || seq == 0) return bad(err, "checkpoint config contains zero dimension");
+    if (dim % 128 != 0) return bad(err, "checkpoint dim " + std::to_string(dim) + " is not divisible by 128");
+    if ((len - cur) % 4 != 0) return bad(err, "checkpoint payload is not aligned to f32 values");
+    const size_t payload_floats = (len - cur) / 4;
+    const size_t heads = dim / 128;
+    size_t hidden = 0;
+    if (!infer_hidden(dim, nlayers, vocab, payload_floats, &hidden, err)) return false;
+    out->cfg = ModelConfig::make(dim, hidden, heads, heads, 128, seq, nlayers, vocab, act);
+    out->step = step;
+    const ModelConfig &c = out->cfg;
+    ModelWeights &w = out->weights;
+    if (!read_f32_vec(bytes, len, &cur, c.vocab * c.dim, &w.embed, err)) return false;
+    if (!read_f32_vec(bytes, len, &cur, c.dim, &w.gamma_final, err)) return false;
+    w.layers.assign(c.nlayers, LayerWeights());
+    for (LayerWeights &L : w.layers) {
+        if (!read_f32_vec(bytes, len, &cur, c.dim * c.q_dim, &L.wq, err) ||
+            !read_f32_vec(bytes, len, &cur, c.dim * c.kv_dim, &L.wk, err) ||
+            !read_f32_vec(bytes, len, &cur, c.dim * c.kv_dim, &L.wv, err) ||
+            !read_f32_vec(bytes, len, &cur, c.q_dim * c.dim, &L.wo, err) ||
+            !read_f32_vec(bytes, len, &cur, c.dim * c.hidden, &L.w1, err) ||
+            !read_f32_vec(bytes, len, &cur, c.dim * c.hidden, &L.w3, err) ||
+            !read_f32_vec(bytes, len, &cur, c.dim * c.hidden, &L.w2, err) ||
+            !read_f32_vec(bytes, len, &cur, c.dim, &L.gamma1, err) ||
+            !read_f32_vec(bytes, len, &cur, c.dim, &L.gamma2, err))
+            return false;
+    }
+    if (cur != len) return bad(err, "checkpoint had trailing bytes");
+    return true;
+}
+
+bool load_checkpoint(const std::string &path, Checkpoint *out, std::string *err) {
+    const int fd = open(path.c_str(), O_RDONLY);
+    if (fd < 0) return bad(err, "cannot open " + path + ": " + strerror(errno));
+    struct stat st;
+    if (fstat(fd, &st) != 0) { close(fd); return bad(err, "cannot stat " + path + ": " + strerror(errno)); }
+    const size_t len = (size_t)st.st_size;
+    if (len == 0) { close(fd); return bad(err, "checkpoint too small for header"); }
+    void *p = mmap(nullptr, len, PROT_READ, MAP_PRIVATE, fd, 0);
+    close(fd);
+    if (p == MAP_FAILED) return bad(err, "cannot map " + path + ": " + strerror(errno));
+    const bool ok = parse_checkpoint((const uint8_t *)p, len, out, err);
+    munmap(p, len);
+    return ok;
+}
+
+bool write_checkpoint(const std::string &path, const ModelConfig &c, const ModelWeights &w, uint32_t step,
+                      std::string *err) {
+    if (c.hd != 128 || c.kv_heads != c.heads || c.dim != c.heads * 128)
+        return bad(err, "the checkpoint header cannot describe this model (needs hd 128, kv_heads = heads, dim = heads * 128)");
+    if (w.layers.size() != c.nlayers) return bad(err, "layer count does not match the configuration");
+    FILE *f = fopen(path.c_str(), "wb");
+    if (!f) return bad(err, "cannot create " + path + ": " + strerror(errno));
+    const uint32_t head[7] = {kVersion, step, (uint32_t)c.dim, (uint32_t)c.nlayers, (uint32_t)c.vocab, (uint32_t)c.seq,
+                              (uint32_t)c.ffn_activation};
+    bool ok = fwrite("RSTK", 1, 4, f) == 4 && fwrite(head, 4, 7, f) == 7;
+    auto put = [&](const std::vector<float> &v, size_t want) {
+        ok = ok && v.size() == want && fwrite(v.data(), 4, v.size(), f) == v.size();
+    };
+    put(w.embed, c.vocab * c.dim);
+    put(w.gamma_final, c.dim);
+    for (const LayerWeights &L : w.layers) {
+        put(L.wq, c.dim * c.q_dim); put(L.wk, c.dim * c.kv_dim); put(L.wv, c.dim * c.kv_dim); put(L.wo, c.q_dim * c.dim);
+        put(L.w1, c.dim * c.hidden); put(L.w3, c.dim * c.hidden); put(L.w2, c.dim * c.hidden);
+        put(L.gamma1, c.dim); put(L.gamma2, c.dim);
+    }
+    ok = (fclose(f) == 0) && ok;
+    if (!ok) return bad(err, "short write or tensor size mismatch writing " + path);
+    return true;
+}
+
+}  // namespace rustane

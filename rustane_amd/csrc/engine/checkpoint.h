@@ -1,0 +1,30 @@
+// RSTK checkpoint files (crates/engine/src/checkpoint.rs:1-242; written by
+// crates/engine/src/bin/train.rs:609-647):
+//   "RSTK", version u32, step u32, dim u32, nlayers u32, vocab u32, seq u32, [activation u32 if version >= 2],
+//   then little-endian f32 tensors: embed[V*D], gamma_final[D], and per layer
+//   wq wk wv wo w1 w3 w2 gamma1 gamma2.
+// The header carries neither heads nor hidden: heads = dim / 128 (hd = 128, MHA) and hidden follows
+// from the payload size (checkpoint.rs:101-117, :168-214).
+#pragma once
+#include <string>
+
+#include "model.h"
+
+namespace rustane {
+
+struct Checkpoint {
+    ModelConfig cfg;
+    ModelWeights weights;
+    uint32_t step = 0;
+};
+
+// checkpoint.rs:30-166.  Returns false and the reference's message in *err on malformed input.
+bool parse_checkpoint(const uint8_t *bytes, size_t len, Checkpoint *out, std::string *err);
+// checkpoint.rs:25-28 (the file is mapped, not read into a second buffer)
+bool load_checkpoint(const std::string &path, Checkpoint *out, std::string *err);
+// train.rs:609-647: version-2 header and tensor order; the model must be one the header can
+// describe (hd = 128, kv_heads = heads, dim = heads * 128)
+bool write_checkpoint(const std::string &path, const ModelConfig &cfg, const ModelWeights &w, uint32_t step,
+                      std::string *err);
+
+}  // namespace rustane

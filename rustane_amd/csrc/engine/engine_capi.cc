@@ -7,6 +7,7 @@
 #include <string>
 #include <vector>
 
+#include "checkpoint.h"
 #include "inference.h"
 
 using namespace rustane;
@@ -69,6 +70,49 @@ rs_weights *rs_weights_from_arrays(const rs_config *c, const float *const *layer
     return w;
 }
 void rs_weights_free(rs_weights *w) { delete w; }
+
+// ---- RSTK checkpoints (crates/engine/src/checkpoint.rs)
+static void from_cfg(const ModelConfig &c, rs_config *o) {
+    o->dim = c.dim; o->hidden = c.hidden; o->heads = c.heads; o->kv_heads = c.kv_heads; o->hd = c.hd; o->seq = c.seq;
+    o->nlayers = c.nlayers; o->vocab = c.vocab; o->ffn_activation = (uint32_t)c.ffn_activation;
+}
+static rs_weights *take_checkpoint(Checkpoint &ck, rs_config *cfg_out, uint32_t *step) {
+    rs_weights *w = new rs_weights();
+    w->w = std::move(ck.weights);
+    if (cfg_out) from_cfg(ck.cfg, cfg_out);
+    if (step) *step = ck.step;
+    return w;
+}
+rs_weights *rs_checkpoint_parse(const uint8_t *bytes, size_t n, rs_config *cfg_out, uint32_t *step, char *err, size_t errcap) {
+    Checkpoint ck;
+    std::string e;
+    if (!parse_checkpoint(bytes, n, &ck, &e)) { put_err(err, errcap, e); return nullptr; }
+    return take_checkpoint(ck, cfg_out, step);
+}
+rs_weights *rs_checkpoint_load(const char *path, rs_config *cfg_out, uint32_t *step, char *err, size_t errcap) {
+    Checkpoint ck;
+    std::string e;
+    if (!load_checkpoint(path, &ck, &e)) { put_err(err, errcap, e); return nullptr; }
+    return take_checkpoint(ck, cfg_out, step);
+}
+int rs_checkpoint_write(const char *path, const rs_config *c, const rs_weights *w, uint32_t step, char *err, size_t errcap) {
+    std::string e;
+    if (!write_checkpoint(path, to_cfg(c), w->w, step, &e)) { put_err(err, errcap, e); return 1; }
+    return 0;
+}
+// tensor `which` of layer `layer` in the order wq wk wv wo w1 w3 w2 gamma1 gamma2; layer < 0: 0 embed, 1 gamma_final
+int rs_weights_tensor(const rs_weights *w, int64_t layer, int which, const float **ptr, uint64_t *n) {
+    const std::vector<float> *v = nullptr;
+    if (layer < 0) v = which == 0 ? &w->w.embed : which == 1 ? &w->w.gamma_final : nullptr;
+    else if ((size_t)layer < w->w.layers.size() && which >= 0 && which < 9) {
+        const LayerWeights &L = w->w.layers[(size_t)layer];
+        const std::vector<float> *t[9] = {&L.wq, &L.wk, &L.wv, &L.wo, &L.w1, &L.w3, &L.w2, &L.gamma1, &L.gamma2};
+        v = t[which];
+    }
+    if (!v) return 1;
+    *ptr = v->data(); *n = v->size();
+    return 0;
+}
 
 rs_session *rs_session_new(const rs_config *c, const rs_weights *w, const uint32_t *prompt, size_t n, float softcap,
                            uint32_t weight_dtype, uint32_t kv_dtype, uint32_t flags, char *err, size_t errcap) {

@@ -9,6 +9,7 @@
 #include <string>
 #include <vector>
 
+#include "checkpoint.h"
 #include "inference.h"
 #include "synth.h"
 
@@ -22,7 +23,7 @@ namespace {
 }
 
 void usage() {
-    printf("usage: generate --model <preset|custom:dim,hidden,nlayers,seq[,heads,hd,vocab]> --prompt-ids 1,2,3\n"
+    printf("usage: generate (--checkpoint PATH | --model <preset|custom:dim,hidden,nlayers,seq[,heads,hd,vocab]>) --prompt-ids 1,2,3\n"
            "  [--steps N] [--temperature T] [--top-k K] [--softcap C] [--samples N] [--seed S]\n"
            "  [--decode-backend auto|naive|hip] [--kv-cache] [--weight-dtype f32|bf16|fp8|int4] [--kv-dtype f32|bf16]\n"
            "  [--weight-seed S] [--weight-std X] [--random-prompt N]\n"
@@ -76,7 +77,7 @@ std::string format_ids(const std::vector<uint32_t> &ids) {
 }  // namespace
 
 int main(int argc, char **argv) {
-    std::string model = "gpt_1024", prompt_ids_raw, wdt = "f32", kvdt = "f32";
+    std::string model = "gpt_1024", checkpoint, prompt_ids_raw, wdt = "f32", kvdt = "f32";
     GenerationRequest req;
     float softcap = 0.0f, weight_std = 0.02f;
     uint64_t weight_seed = 1234;
@@ -85,6 +86,7 @@ int main(int argc, char **argv) {
         std::string a = argv[i];
         auto val = [&]() -> std::string { if (i + 1 >= argc) fail(a + " needs a value"); return argv[++i]; };
         if (a == "--model") model = val();
+        else if (a == "--checkpoint") checkpoint = val();                               // generate.rs:165-167
         else if (a == "--prompt-ids") prompt_ids_raw = val();
         else if (a == "--random-prompt") random_prompt = strtoull(val().c_str(), nullptr, 10);
         else if (a == "--steps") req.steps = strtoull(val().c_str(), nullptr, 10);
@@ -107,7 +109,15 @@ int main(int argc, char **argv) {
     }
     if (req.samples == 0) fail("samples must be >= 1");
     ModelConfig cfg;
-    if (!model_from_name(model, &cfg)) fail("unknown --model " + model);
+    Checkpoint ckpt;
+    if (!checkpoint.empty()) {
+        std::string cerr;
+        if (!load_checkpoint(checkpoint, &ckpt, &cerr)) fail("failed to load checkpoint: " + cerr);   // generate.rs:495
+        cfg = ckpt.cfg;
+        model = checkpoint;
+        printf("loaded checkpoint: step=%u model=%zuL %zuD %zuH %zuV seq=%zu\n", ckpt.step, cfg.nlayers, cfg.dim, cfg.hidden,
+               cfg.vocab, cfg.seq);                                                       // generate.rs:526
+    } else if (!model_from_name(model, &cfg)) fail("unknown --model " + model);
     SessionOptions opts;
     if (wdt == "f32") opts.weight_dtype = WeightDtype::F32;
     else if (wdt == "bf16") opts.weight_dtype = WeightDtype::BF16;
@@ -134,7 +144,9 @@ int main(int argc, char **argv) {
     if (planned.auto_reason) printf(" auto_reason=%s", planned.auto_reason);
     printf("\n");
 
-    ModelWeights weights = ModelWeights::synthetic(cfg, weight_seed, weight_std, opts.weight_dtype != WeightDtype::F32);
+    ModelWeights weights = checkpoint.empty()
+                               ? ModelWeights::synthetic(cfg, weight_seed, weight_std, opts.weight_dtype != WeightDtype::F32)
+                               : std::move(ckpt.weights);
     std::string err;
     InferenceSession session(cfg, weights, prompt, softcap, opts, &err);
     if (!session.ok()) fail(err);

@@ -64,6 +64,12 @@ def lib():
         L.rs_weights_from_arrays.restype = C.c_void_p
         L.rs_weights_from_arrays.argtypes = [C.POINTER(RsConfig), C.POINTER(fp), fp, fp]
         L.rs_weights_free.argtypes = [C.c_void_p]
+        L.rs_checkpoint_parse.restype = C.c_void_p
+        L.rs_checkpoint_parse.argtypes = [C.c_char_p, C.c_size_t, C.POINTER(RsConfig), u32p, C.c_char_p, C.c_size_t]
+        L.rs_checkpoint_load.restype = C.c_void_p
+        L.rs_checkpoint_load.argtypes = [C.c_char_p, C.POINTER(RsConfig), u32p, C.c_char_p, C.c_size_t]
+        L.rs_checkpoint_write.argtypes = [C.c_char_p, C.POINTER(RsConfig), C.c_void_p, C.c_uint32, C.c_char_p, C.c_size_t]
+        L.rs_weights_tensor.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.POINTER(fp), u64p]
         L.rs_session_new.restype = C.c_void_p
         L.rs_session_new.argtypes = [C.POINTER(RsConfig), C.c_void_p, u32p, C.c_size_t, C.c_float, C.c_uint32,
                                      C.c_uint32, C.c_uint32, C.c_char_p, C.c_size_t]
@@ -264,3 +270,71 @@ class InferenceSession:
 
     def stream_count(self):
         return int(self._L.rs_session_stream_count(self._s))
+
+
+# ---------------------------------------------------------------- RSTK checkpoints (crates/engine/src/checkpoint.rs)
+class CheckpointError(ValueError):
+    pass
+
+
+_TENSORS = ("wq", "wk", "wv", "wo", "w1", "w3", "w2", "gamma1", "gamma2")
+
+
+def _take_checkpoint(L, handle, rc, step):
+    from .hipdec import Config
+    cfg = Config.make(dim=rc.dim, hidden=rc.hidden, heads=rc.heads, hd=rc.hd, seq=rc.seq, nlayers=rc.nlayers,
+                      vocab=rc.vocab, kv_heads=rc.kv_heads)
+
+    def tensor(layer, which):
+        p, n = fp(), C.c_uint64()
+        if L.rs_weights_tensor(handle, layer, which, C.byref(p), C.byref(n)):
+            raise CheckpointError("no such tensor")
+        return np.ctypeslib.as_array(p, shape=(n.value,)).copy()
+
+    try:
+        weights = {"embed": tensor(-1, 0), "gamma_final": tensor(-1, 1),
+                   "layers": [{nme: tensor(l, k) for k, nme in enumerate(_TENSORS)} for l in range(cfg.nlayers)]}
+    finally:
+        L.rs_weights_free(handle)
+    return cfg, weights, int(step.value), int(rc.ffn_activation)
+
+
+def parse_checkpoint(data):
+    """checkpoint.rs:30-166 on a bytes object -> (cfg, weights dict, step, ffn_activation code)."""
+    L = lib()
+    rc, step, err = RsConfig(), C.c_uint32(), C.create_string_buffer(256)
+    h = L.rs_checkpoint_parse(bytes(data), len(data), C.byref(rc), C.byref(step), err, 256)
+    if not h:
+        raise CheckpointError(err.value.decode())
+    return _take_checkpoint(L, C.c_void_p(h), rc, step)
+
+
+def load_checkpoint(path):
+    """checkpoint.rs:25-28 -> (cfg, weights dict, step, ffn_activation code)."""
+    L = lib()
+    rc, step, err = RsConfig(), C.c_uint32(), C.create_string_buffer(512)
+    h = L.rs_checkpoint_load(str(path).encode(), C.byref(rc), C.byref(step), err, 512)
+    if not h:
+        raise CheckpointError(err.value.decode())
+    return _take_checkpoint(L, C.c_void_p(h), rc, step)
+
+
+def write_checkpoint(path, cfg, weights, step=0, ffn_activation=0):
+    """The version-2 file crates/engine/src/bin/train.rs:609-647 writes."""
+    L = lib()
+    rc = RsConfig.of(cfg, ffn_activation)
+    keep, ptrs = [], (fp * (9 * cfg.nlayers))()
+    for l, lw in enumerate(weights["layers"]):
+        for k, nme in enumerate(_TENSORS):
+            a = np.ascontiguousarray(lw[nme], np.float32)
+            keep.append(a)
+            ptrs[l * 9 + k] = a.ctypes.data_as(fp)
+    gf = np.ascontiguousarray(weights["gamma_final"], np.float32)
+    em = np.ascontiguousarray(weights["embed"], np.float32)
+    h = C.c_void_p(L.rs_weights_from_arrays(C.byref(rc), ptrs, gf.ctypes.data_as(fp), em.ctypes.data_as(fp)))
+    err = C.create_string_buffer(512)
+    try:
+        if L.rs_checkpoint_write(str(path).encode(), C.byref(rc), h, step, err, 512):
+            raise CheckpointError(err.value.decode())
+    finally:
+        L.rs_weights_free(h)

@@ -1,0 +1,113 @@
+"""RSTK checkpoint reader/writer of the host engine against the format the reference defines
+(crates/engine/src/checkpoint.rs:1-242, writer crates/engine/src/bin/train.rs:609-647).  The files
+under test are assembled here with numpy straight from that description, the way the reference's
+own test assembles them (checkpoint.rs:262-313), so the reader is not checked against its own writer
+alone; every rejection the reference's parser has is provoked with its message."""
+import struct
+
+import numpy as np
+import pytest
+
+from rustane_amd import engine, synth
+from rustane_amd.hipdec import Config
+
+NAMES = ("wq", "wk", "wv", "wo", "w1", "w3", "w2", "gamma1", "gamma2")
+
+
+def cfg_small(hidden=640):
+    # the shape of the reference's own parser test (checkpoint.rs:264-277)
+    return Config.make(dim=256, hidden=hidden, heads=2, hd=128, seq=64, nlayers=2, vocab=32)
+
+
+def file_bytes(cfg, w, version=2, step=123, act=0, magic=b"RSTK"):
+    head = magic + struct.pack("<I", version) + struct.pack("<5I", step, cfg.dim, cfg.nlayers, cfg.vocab, cfg.seq)
+    if version >= 2:
+        head += struct.pack("<I", act)
+    parts = [head, np.asarray(w["embed"], "<f4").tobytes(), np.asarray(w["gamma_final"], "<f4").tobytes()]
+    for lw in w["layers"]:
+        parts += [np.asarray(lw[n], "<f4").tobytes() for n in NAMES]
+    return b"".join(parts)
+
+
+def assert_same_weights(a, b):
+    np.testing.assert_array_equal(a["embed"], b["embed"])
+    np.testing.assert_array_equal(a["gamma_final"], b["gamma_final"])
+    assert len(a["layers"]) == len(b["layers"])
+    for la, lb in zip(a["layers"], b["layers"]):
+        for n in NAMES:
+            np.testing.assert_array_equal(la[n], lb[n])
+
+
+@pytest.mark.parametrize("hidden,act", [(640, 0), (384, 1)])
+def test_parses_checkpoint_and_infers_hidden(hidden, act):
+    cfg = cfg_small(hidden)
+    w = synth.make_weights(cfg, seed=3, std=0.05)
+    got_cfg, got_w, step, got_act = engine.parse_checkpoint(file_bytes(cfg, w, act=act))
+    assert step == 123 and got_act == act
+    for f in ("dim", "hidden", "heads", "kv_heads", "hd", "seq", "nlayers", "vocab", "q_dim", "kv_dim"):
+        assert getattr(got_cfg, f) == getattr(cfg, f), f
+    assert_same_weights(got_w, w)
+
+
+def test_version_1_has_no_activation_field():
+    cfg = cfg_small()
+    w = synth.make_weights(cfg, seed=4, std=0.05)
+    got_cfg, got_w, step, act = engine.parse_checkpoint(file_bytes(cfg, w, version=1, step=7))
+    assert (step, act, got_cfg.hidden) == (7, 0, 640)
+    assert_same_weights(got_w, w)
+
+
+def test_rejections_carry_the_reference_messages():
+    cfg = cfg_small()
+    w = synth.make_weights(cfg, seed=5, std=0.05)
+    good = file_bytes(cfg, w)
+
+    def msg(data):
+        with pytest.raises(engine.CheckpointError) as e:
+            engine.parse_checkpoint(data)
+        return str(e.value)
+
+    assert msg(good[:20]) == "checkpoint too small for header"
+    assert msg(file_bytes(cfg, w, magic=b"RSTX")) == "invalid checkpoint magic"
+    assert msg(file_bytes(cfg, w, version=3)) == "unsupported checkpoint version 3"
+    assert msg(file_bytes(cfg, w, version=0)) == "unsupported checkpoint version 0"
+    assert msg(b"RSTK" + struct.pack("<6I", 2, 0, 256, 2, 32, 64)) == "checkpoint too small for v2 header"
+    assert msg(file_bytes(cfg, w, act=2)) == "unsupported checkpoint activation code 2"
+    zero = bytearray(good); zero[12:16] = struct.pack("<I", 0)
+    assert msg(bytes(zero)) == "checkpoint config contains zero dimension"
+    odd = bytearray(good); odd[12:16] = struct.pack("<I", 200)
+    assert msg(bytes(odd)) == "checkpoint dim 200 is not divisible by 128"
+    assert msg(good + b"\0\0") == "checkpoint payload is not aligned to f32 values"
+    assert msg(good[:32 + 4 * 100]) == "checkpoint payload too small for fixed-size tensors"
+    assert msg(good + b"\0" * 4) == "checkpoint payload does not imply an integer hidden size"
+
+
+def test_writer_emits_the_documented_layout_and_round_trips(tmp_path):
+    cfg = cfg_small()
+    w = synth.make_weights(cfg, seed=6, std=0.05)
+    path = tmp_path / "ckpt_000042.bin"
+    engine.write_checkpoint(path, cfg, w, step=42, ffn_activation=1)
+    assert path.read_bytes() == file_bytes(cfg, w, step=42, act=1)
+    got_cfg, got_w, step, act = engine.load_checkpoint(path)
+    assert (step, act, got_cfg.hidden) == (42, 1, 640)
+    assert_same_weights(got_w, w)
+    with pytest.raises(engine.CheckpointError):
+        engine.load_checkpoint(tmp_path / "missing.bin")
+    # the header has no place for hd or kv_heads: such models are refused, not written wrongly
+    gqa = Config.make(dim=256, hidden=384, heads=4, hd=64, seq=64, nlayers=1, vocab=32, kv_heads=2)
+    with pytest.raises(engine.CheckpointError):
+        engine.write_checkpoint(tmp_path / "x.bin", gqa, synth.make_weights(gqa, seed=1, std=0.05))
+
+
+@pytest.mark.gpu
+def test_session_from_checkpoint_equals_session_from_arrays(tmp_path):
+    cfg = cfg_small()
+    w = synth.make_weights(cfg, seed=8, std=0.08, round_bf16=True)
+    path = tmp_path / "ckpt.bin"
+    engine.write_checkpoint(path, cfg, w, step=1)
+    cfg2, w2, _, act = engine.load_checkpoint(path)
+    prompt = synth.make_prompt(3, cfg.vocab, 9)
+    req = engine.GenerationRequest(decode_backend=engine.DecodeBackendRequest.HIP, steps=12, temperature=0.0)
+    a = engine.InferenceSession(cfg, w, prompt, weight_dtype=1, kv_dtype=0).generate(req)
+    b = engine.InferenceSession(cfg2, w2, prompt, weight_dtype=1, kv_dtype=0, ffn_activation=act).generate(req)
+    np.testing.assert_array_equal(a.results[0].sampled, b.results[0].sampled)
