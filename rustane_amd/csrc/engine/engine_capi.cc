@@ -9,6 +9,7 @@
 
 #include "checkpoint.h"
 #include "inference.h"
+#include "jsonl_session.h"
 
 using namespace rustane;
 
@@ -198,6 +199,28 @@ int rs_parse_decode_backend(const char *raw, uint32_t *out) {
     if (!parse_decode_backend(raw, &r)) return 0;
     *out = r == DecodeBackendRequest::Naive ? 1 : r == DecodeBackendRequest::Hip ? 2 : 0;
     return 1;
+}
+
+// ---- one request line of the JSONL session protocol (bin/generate.rs:39-144), without running it:
+// 0 = ok (request and suffix filled), 1 = rejected (err holds the message the session would answer with)
+int rs_jsonl_parse(const char *line, const rs_request *defaults, rs_request *out, uint32_t *suffix, size_t cap,
+                   uint64_t *n_suffix, char *err, size_t errcap) {
+    GenerationRequest d, req;
+    d.decode_backend = (DecodeBackendRequest)defaults->backend; d.steps = defaults->steps; d.temperature = defaults->temperature;
+    d.top_k = defaults->top_k; d.samples = defaults->samples; d.seed = defaults->seed;
+    JsonlRequest parsed;
+    std::vector<uint32_t> sfx;
+    std::string e;
+    if (!parse_jsonl_request(line, &parsed, &e) || !jsonl_to_generation_request(parsed, d, &req, &e) ||
+        !jsonl_prompt_suffix(parsed, &sfx, &e)) {
+        put_err(err, errcap, e);
+        return 1;
+    }
+    out->backend = (uint32_t)req.decode_backend; out->steps = req.steps; out->temperature = req.temperature;
+    out->top_k = req.top_k; out->samples = req.samples; out->seed = req.seed;
+    *n_suffix = sfx.size();
+    for (size_t i = 0; i < sfx.size() && i < cap; ++i) suffix[i] = sfx[i];
+    return 0;
 }
 
 uint64_t rs_next_u64(uint64_t *state) { return next_u64(state); }

@@ -11,6 +11,7 @@
 
 #include "checkpoint.h"
 #include "inference.h"
+#include "jsonl_session.h"
 #include "synth.h"
 
 using namespace rustane;
@@ -26,7 +27,7 @@ void usage() {
     printf("usage: generate (--checkpoint PATH | --model <preset|custom:dim,hidden,nlayers,seq[,heads,hd,vocab]>) --prompt-ids 1,2,3\n"
            "  [--steps N] [--temperature T] [--top-k K] [--softcap C] [--samples N] [--seed S]\n"
            "  [--decode-backend auto|naive|hip] [--kv-cache] [--weight-dtype f32|bf16|fp8|int4] [--kv-dtype f32|bf16]\n"
-           "  [--weight-seed S] [--weight-std X] [--random-prompt N]\n"
+           "  [--weight-seed S] [--weight-std X] [--random-prompt N] [--jsonl-session]\n"
            "presets: gpt_karpathy gpt_1024 target_600m target_800m target_1b target_1_5b bench_tiny bench_600m bench_5b\n");
 }
 
@@ -82,6 +83,7 @@ int main(int argc, char **argv) {
     float softcap = 0.0f, weight_std = 0.02f;
     uint64_t weight_seed = 1234;
     size_t random_prompt = 0;
+    bool jsonl_session = false;
     for (int i = 1; i < argc; ++i) {
         std::string a = argv[i];
         auto val = [&]() -> std::string { if (i + 1 >= argc) fail(a + " needs a value"); return argv[++i]; };
@@ -99,6 +101,7 @@ int main(int argc, char **argv) {
         else if (a == "--weight-std") weight_std = strtof(val().c_str(), nullptr);
         else if (a == "--weight-dtype") wdt = val();
         else if (a == "--kv-dtype") kvdt = val();
+        else if (a == "--jsonl-session") jsonl_session = true;                          // generate.rs:236-238
         else if (a == "--kv-cache") req.decode_backend = DecodeBackendRequest::Hip;     // generate.rs:189-192
         else if (a == "--decode-backend") {
             std::string raw = val();
@@ -115,7 +118,8 @@ int main(int argc, char **argv) {
         if (!load_checkpoint(checkpoint, &ckpt, &cerr)) fail("failed to load checkpoint: " + cerr);   // generate.rs:495
         cfg = ckpt.cfg;
         model = checkpoint;
-        printf("loaded checkpoint: step=%u model=%zuL %zuD %zuH %zuV seq=%zu\n", ckpt.step, cfg.nlayers, cfg.dim, cfg.hidden,
+        if (!jsonl_session)                                                              // generate.rs:523 (stdout carries only answers)
+            printf("loaded checkpoint: step=%u model=%zuL %zuD %zuH %zuV seq=%zu\n", ckpt.step, cfg.nlayers, cfg.dim, cfg.hidden,
                cfg.vocab, cfg.seq);                                                       // generate.rs:526
     } else if (!model_from_name(model, &cfg)) fail("unknown --model " + model);
     SessionOptions opts;
@@ -135,14 +139,17 @@ int main(int argc, char **argv) {
     }
     if (prompt.empty()) fail("pass --prompt-ids or --random-prompt");
 
-    printf("model=%s dim=%zu hidden=%zu heads=%zu hd=%zu nlayers=%zu seq=%zu vocab=%zu params=%zu\n", model.c_str(),
-           cfg.dim, cfg.hidden, cfg.heads, cfg.hd, cfg.nlayers, cfg.seq, cfg.vocab, cfg.param_count());
+    if (!jsonl_session)
+        printf("model=%s dim=%zu hidden=%zu heads=%zu hd=%zu nlayers=%zu seq=%zu vocab=%zu params=%zu\n", model.c_str(),
+               cfg.dim, cfg.hidden, cfg.heads, cfg.hd, cfg.nlayers, cfg.seq, cfg.vocab, cfg.param_count());
     DecodeSelection planned = select_decode_mode(cfg, req.decode_backend, prompt.size() < cfg.seq ? prompt.size() : cfg.seq,
                                                  req.steps);
-    printf("decode_backend_request=%s decode_mode=%s", decode_backend_str(req.decode_backend), decode_mode_str(planned.mode));
-    if (planned.fallback_reason) printf(" fallback_reason=%s", planned.fallback_reason);
-    if (planned.auto_reason) printf(" auto_reason=%s", planned.auto_reason);
-    printf("\n");
+    if (!jsonl_session) {
+        printf("decode_backend_request=%s decode_mode=%s", decode_backend_str(req.decode_backend), decode_mode_str(planned.mode));
+        if (planned.fallback_reason) printf(" fallback_reason=%s", planned.fallback_reason);
+        if (planned.auto_reason) printf(" auto_reason=%s", planned.auto_reason);
+        printf("\n");
+    }
 
     ModelWeights weights = checkpoint.empty()
                                ? ModelWeights::synthetic(cfg, weight_seed, weight_std, opts.weight_dtype != WeightDtype::F32)
@@ -150,6 +157,12 @@ int main(int argc, char **argv) {
     std::string err;
     InferenceSession session(cfg, weights, prompt, softcap, opts, &err);
     if (!session.ok()) fail(err);
+    if (jsonl_session) {                                                                 // generate.rs:571-588
+        fprintf(stderr, "jsonl_session_ready checkpoint_step=%u prompt_len=%zu decode_backend_default=%s\n", ckpt.step,
+                prompt.size(), decode_backend_str(req.decode_backend));
+        run_jsonl_session(stdin, stdout, req, prompt, &session);
+        return 0;
+    }
     GenerationBatch batch;
     if (!session.generate(req, &batch, &err)) fail(err);
 

@@ -69,6 +69,8 @@ def lib():
         L.rs_checkpoint_load.restype = C.c_void_p
         L.rs_checkpoint_load.argtypes = [C.c_char_p, C.POINTER(RsConfig), u32p, C.c_char_p, C.c_size_t]
         L.rs_checkpoint_write.argtypes = [C.c_char_p, C.POINTER(RsConfig), C.c_void_p, C.c_uint32, C.c_char_p, C.c_size_t]
+        L.rs_jsonl_parse.argtypes = [C.c_char_p, C.POINTER(RsRequest), C.POINTER(RsRequest), u32p, C.c_size_t, u64p,
+                                     C.c_char_p, C.c_size_t]
         L.rs_weights_tensor.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.POINTER(fp), u64p]
         L.rs_session_new.restype = C.c_void_p
         L.rs_session_new.argtypes = [C.POINTER(RsConfig), C.c_void_p, u32p, C.c_size_t, C.c_float, C.c_uint32,
@@ -338,3 +340,20 @@ def write_checkpoint(path, cfg, weights, step=0, ffn_activation=0):
             raise CheckpointError(err.value.decode())
     finally:
         L.rs_weights_free(h)
+
+
+# ---------------------------------------------------------------- JSONL session protocol (bin/generate.rs:39-144)
+class JsonlRequestError(ValueError):
+    pass
+
+
+def parse_jsonl_request(line, defaults=None):
+    """One request line -> (GenerationRequest with the defaults filled in, appended prompt ids)."""
+    L = lib()
+    d = (defaults or GenerationRequest())._c()
+    out, n, err = RsRequest(), C.c_uint64(), C.create_string_buffer(512)
+    buf = np.zeros(4096, np.uint32)
+    if L.rs_jsonl_parse(line.encode(), C.byref(d), C.byref(out), buf.ctypes.data_as(u32p), buf.size, C.byref(n), err, 512):
+        raise JsonlRequestError(err.value.decode())
+    req = GenerationRequest(DecodeBackendRequest(out.backend), out.steps, out.temperature, out.top_k, out.samples, out.seed)
+    return req, buf[:n.value].copy()
