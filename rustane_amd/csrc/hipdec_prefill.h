@@ -21,6 +21,9 @@
 typedef __bf16 pf_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float pf_f32x16 __attribute__((ext_vector_type(16)));
 
+#ifndef PF_REG_STAGES
+#define PF_REG_STAGES 1     // K steps of operand loads held in registers ahead of the multiply (1 or 2)
+#endif
 #define PF_BM 128           // prompt rows per GEMM workgroup tile
 #define PF_BN 128           // weight rows (output channels) per GEMM workgroup tile
 #define PF_BK 32            // reduction elements per step of the streaming (few-row) GEMM; K must be a multiple
@@ -343,8 +346,22 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
         }
     };
 
-    Stage S0, S1;
     const int n = s_end - s_begin;
+#if PF_REG_STAGES == 1
+    // one step of operand loads in flight in registers: 48 registers fewer than two, which lets two
+    // workgroups share a CU (one multiplies while the other stages)
+    Stage S0;
+    if (n > 0) gload(S0, s_begin);
+    for (int i = 0; i < n; ++i) {
+        __syncthreads();                       // the previous step's operand reads are done
+        lstore(S0);
+        __syncthreads();
+        if (i + 1 < n) gload(S0, s_begin + i + 1);
+        multiply();
+        if (i & 1) scale_group(s_begin + i);   // (splits of 4-bit weights start on a group boundary)
+    }
+#else
+    Stage S0, S1;
     if (n > 0) gload(S0, s_begin);
     if (n > 1) gload(S1, s_begin + 1);
     for (int i = 0; i < n; i += 2) {
@@ -362,6 +379,7 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
         }
         scale_group(s_begin + i);              // (splits of 4-bit weights start on a group boundary)
     }
+#endif
 
     float *Pz = g.P + (size_t)z * g.T * g.N;
     const int r = lane & 31, gq = lane >> 5;
