@@ -514,7 +514,7 @@ void pf_launch_resid(hipdec_model *m, int T, int splits, const void *wscale, con
 void pf_launch_gate(hipdec_model *m, int T, int splits, const void *wscale) {
     PrefillWork &w = m->pf;
     const int D = (int)m->cfg.dim, H = (int)m->cfg.hidden;
-    const size_t items = (size_t)T * H;
+    const size_t items = (size_t)T * (H / 4);
     hipLaunchKernelGGL(k_pf_gate_epi, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, m->stream, w.P, splits,
                        (size_t)T * 2 * H, m->wt == WT_FP8 ? (const float *)wscale : nullptr, w.gate_hi, w.gate_lo, w.ssq,
                        (D + PF_CHUNK - 1) / PF_CHUNK, D, T, H, (int)m->opt.ffn_activation);
@@ -560,7 +560,7 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
             }
             // causal attention of the chunk's rows over positions 0 .. pos0 + t
             {
-                dim3 grid((T + 31) / 32, c.heads), block(64);
+                dim3 grid((T + 31) / 32, c.heads), block(64 * PF_ATT_WAVES);
 #define PFATT(KVB, HD)                                                                                             \
     hipLaunchKernelGGL((k_pf_attn<KVB, HD>), grid, block, 0, m->stream, w.q, L.kc, L.vc, w.att_hi, w.att_lo, T, Q, KV, \
                        gqa, pos0, (int)c.seq, scale)

@@ -147,26 +147,40 @@ __global__ __launch_bounds__(256) void k_pf_qkv_epi(const float *__restrict__ P,
 }
 
 // gate[t][j] = act(h1) * h3 with h1 = row 2j and h3 = row 2j+1 of the interleaved gate/up product
-// (kernels/ffn_fused.rs:114-150), written as the hi/lo pair the down projection reads.
+// (kernels/ffn_fused.rs:114-150), written as the hi/lo pair the down projection reads.  One thread
+// per four gate elements of a row (H % 4 == 0): 32 bytes of each plane in, 8 + 8 bytes out, the row
+// factor computed once.
 __global__ __launch_bounds__(256) void k_pf_gate_epi(const float *__restrict__ P, int splits, size_t plane,
                                                      const float *__restrict__ wscale, uint16_t *__restrict__ hi,
                                                      uint16_t *__restrict__ lo, const float *__restrict__ ssq, int nch,
                                                      int D, int T, int H, int act) {
+    const int hq = H >> 2;
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (gid >= (size_t)T * H) return;
-    const int t = (int)(gid / H), j = (int)(gid - (size_t)t * H);
-    float h1 = 0.0f, h3 = 0.0f;
+    if (gid >= (size_t)T * hq) return;
+    const int t = (int)(gid / hq), j = 4 * (int)(gid - (size_t)t * hq);
+    float h[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     for (int z = 0; z < splits; ++z) {
-        const float2 v = *(const float2 *)(P + z * plane + (size_t)t * 2 * H + 2 * j);
-        h1 += v.x; h3 += v.y;
+        const float4 a = *(const float4 *)(P + z * plane + (size_t)t * 2 * H + 2 * j);
+        const float4 b = *(const float4 *)(P + z * plane + (size_t)t * 2 * H + 2 * j + 4);
+        h[0] += a.x; h[1] += a.y; h[2] += a.z; h[3] += a.w; h[4] += b.x; h[5] += b.y; h[6] += b.z; h[7] += b.w;
     }
-    if (wscale) { h1 *= wscale[2 * j]; h3 *= wscale[2 * j + 1]; }
+    if (wscale) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) h[e] *= wscale[2 * j + e];
+    }
     const float inv = pf_row_inv(ssq, t, nch, D);
-    h1 *= inv; h3 *= inv;
-    float g;
-    if (act == 1) { const float lr = h1 > 0.0f ? h1 : 0.5f * h1; g = lr * lr * h3; }
-    else { const float sig = 1.0f / (1.0f + expf(-h1)); g = h1 * sig * h3; }
-    pf_split(g, hi[gid], lo[gid]);
+    uint16_t oh[4], ol[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float h1 = h[2 * e] * inv, h3 = h[2 * e + 1] * inv;
+        float g;
+        if (act == 1) { const float lr = h1 > 0.0f ? h1 : 0.5f * h1; g = lr * lr * h3; }
+        else { const float sig = 1.0f / (1.0f + expf(-h1)); g = h1 * sig * h3; }
+        pf_split(g, oh[e], ol[e]);
+    }
+    const size_t o = (size_t)t * H + j;
+    *(uint2 *)(hi + o) = make_uint2((uint32_t)oh[0] | ((uint32_t)oh[1] << 16), (uint32_t)oh[2] | ((uint32_t)oh[3] << 16));
+    *(uint2 *)(lo + o) = make_uint2((uint32_t)ol[0] | ((uint32_t)ol[1] << 16), (uint32_t)ol[2] | ((uint32_t)ol[3] << 16));
 }
 
 // ---------------------------------------------------------------- GEMM on the bf16 matrix cores
@@ -504,14 +518,18 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
 }
 
 // ---------------------------------------------------------------- causal attention over the chunk
-// One wave per (32 query rows, head).  S^T = K . Q^T on the fp32 MFMA (32x32x2: lane l supplies
+// One workgroup of PF_ATT_WAVES waves per (32 query rows, head); wave w takes the key tiles w,
+// w + PF_ATT_WAVES, ... with its own running maximum, sum and output tile, and the partial results
+// are merged through LDS at the end (a single wave walking up to T/32 tiles one after the other is
+// the critical path of the whole kernel under the causal mask).  S^T = K . Q^T on the fp32 MFMA (32x32x2: lane l supplies
 // row l % 32 and reduction element l / 32 of both operands), so lane (q = l % 32, g = l / 32) ends
 // up with the scores of query q against keys 8 * (i / 4) + 4 * g + i % 4, i = 0..15 -- exactly the
 // operand layout P needs in O += P . V.  Softmax statistics are per lane (+ one exchange with lane
 // l ^ 32); the rescale factors of the O rows travel through LDS.
 // (kernels/sdpa_fwd.rs:325-354: softmax(q . k^T / sqrt(hd) + causal mask) . v)
+#define PF_ATT_WAVES 4
 template <int KVBF16, int HD>
-__global__ __launch_bounds__(64) void k_pf_attn(const float *__restrict__ q, const void *__restrict__ kc,
+__global__ __launch_bounds__(64 * PF_ATT_WAVES) void k_pf_attn(const float *__restrict__ q, const void *__restrict__ kc,
                                                 const void *__restrict__ vc, uint16_t *__restrict__ ohi,
                                                 uint16_t *__restrict__ olo, int T, int Q, int KV, int gqa, int pos0,
                                                 int seq, float scale) {
@@ -522,9 +540,18 @@ __global__ __launch_bounds__(64) void k_pf_attn(const float *__restrict__ q, con
     constexpr int CPR = HD * KESZ / 16;        // 16-byte chunks per cache row
     constexpr int KCH = HK * KESZ / 16;        // chunks of this lane's half row
     constexpr int VCH = 32 * CPR / 64;         // V-tile chunks per lane
-    __shared__ __align__(16) float sV[32 * VS];
-    __shared__ __align__(16) float sfac[32];
-    const int lane = threadIdx.x, r = lane & 31, g = lane >> 5;
+    __shared__ __align__(16) float sVw[PF_ATT_WAVES][32 * VS];
+    __shared__ __align__(16) float sfacw[PF_ATT_WAVES][32];
+    __shared__ float s_m[PF_ATT_WAVES][32], s_l[PF_ATT_WAVES][32];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, g = lane >> 5;
+    float *sV = sVw[wave], *sfac = sfacw[wave];
+    // LDS traffic inside the key loop stays within one wave (its own tile and factors): program order
+    // is enough for the hardware, the fence keeps the compiler from reordering across it
+    auto wave_sync = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
     const int q0 = blockIdx.x * 32, h = blockIdx.y, kvh = h / gqa;
     const int tq = min(q0 + r, T - 1);
     const int qpos = pos0 + q0 + r;            // position of this lane's query row
@@ -549,7 +576,7 @@ __global__ __launch_bounds__(64) void k_pf_attn(const float *__restrict__ q, con
     const char *kbase = (const char *)kc + (size_t)kvh * HD * KESZ;
     const char *vbase = (const char *)vc + (size_t)kvh * HD * KESZ;
     const size_t rowb = (size_t)KV * KESZ;
-    for (int kt0 = 0; kt0 <= last_pos; kt0 += 32) {
+    for (int kt0 = 32 * wave; kt0 <= last_pos; kt0 += 32 * PF_ATT_WAVES) {
         // this lane's key row (its half of the head dimension) and its share of the V tile
         uint4 kr[KCH], vr[VCH];
         {
@@ -574,7 +601,7 @@ __global__ __launch_bounds__(64) void k_pf_attn(const float *__restrict__ q, con
             for (int e = 0; e < 16 / KESZ; ++e)
                 accS = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[c * (16 / KESZ) + e], accS, 0, 0, 0);
         }
-        __syncthreads();                       // the previous tile's V reads are done
+        wave_sync();                           // the previous tile's V reads are done
 #pragma unroll
         for (int c = 0; c < VCH; ++c) {
             const int ch = lane + 64 * c, vrow = ch / CPR, cc = ch % CPR;
@@ -607,7 +634,7 @@ __global__ __launch_bounds__(64) void k_pf_attn(const float *__restrict__ q, con
         l_run = l_run * corr + psum;
         m_run = m_new;
         if (g == 0) sfac[r] = corr;
-        __syncthreads();                       // V tile and rescale factors are in LDS
+        wave_sync();                           // V tile and rescale factors are in LDS
 #pragma unroll
         for (int j4 = 0; j4 < 4; ++j4) {
             const float4 f = *(const float4 *)(sfac + 8 * j4 + 4 * g);
@@ -625,19 +652,31 @@ __global__ __launch_bounds__(64) void k_pf_attn(const float *__restrict__ q, con
                 accO[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(p[s], sV[key * VS + 32 * nt + r], accO[nt], 0, 0, 0);
         }
     }
-    __syncthreads();
-    if (g == 0) sfac[r] = l_run > 0.0f ? 1.0f / l_run : 0.0f;
-    __syncthreads();
+    // merge the waves' partial results: O = sum_w e_w O_w / sum_w e_w l_w with e_w = exp(m_w - max m)
+    wave_sync();
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-        const int qi = 8 * (i >> 2) + 4 * g + (i & 3), t = q0 + qi;
-        const float f = sfac[qi];
-        if (t < T) {
+        const int qi = 8 * (i >> 2) + 4 * g + (i & 3);
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const size_t o = (size_t)t * Q + h * HD + 32 * nt + r;
-                pf_split(accO[nt][i] * f, ohi[o], olo[o]);
-            }
+        for (int nt = 0; nt < NT; ++nt) sV[qi * VS + 32 * nt + r] = accO[nt][i];
+    }
+    if (g == 0) { s_m[wave][r] = m_run; s_l[wave][r] = l_run; }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 32 * HD; idx += 64 * PF_ATT_WAVES) {
+        const int qi = idx / HD, d = idx - qi * HD, t = q0 + qi;
+        float M = -1e30f;
+#pragma unroll
+        for (int w = 0; w < PF_ATT_WAVES; ++w) M = fmaxf(M, s_m[w][qi]);
+        float num = 0.0f, den = 0.0f;
+#pragma unroll
+        for (int w = 0; w < PF_ATT_WAVES; ++w) {
+            const float e = __expf(s_m[w][qi] - M);
+            den += e * s_l[w][qi];
+            num += e * sVw[w][qi * VS + d];
+        }
+        if (t < T) {
+            const size_t o = (size_t)t * Q + h * HD + d;
+            pf_split(den > 0.0f ? num / den : 0.0f, ohi[o], olo[o]);
         }
     }
 }
