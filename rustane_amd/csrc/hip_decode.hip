@@ -428,7 +428,8 @@ PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K) {
         const int sps = (nsteps + s - 1) / s;
         return PfSplit{(nsteps + sps - 1) / sps, sps};
     }
-    const int tiles = ((N + PF_BN - 1) / PF_BN) * ((T + PF_BM - 1) / PF_BM);
+    const int bn = PF_BN_OF(wt);
+    const int tiles = ((N + bn - 1) / bn) * ((T + PF_BM - 1) / PF_BM);
     const int lsteps = (K + PF_BKL - 1) / PF_BKL;
     int s = (2 * m->num_cu + tiles - 1) / tiles;
     s = std::min(s, 8);
@@ -483,7 +484,8 @@ int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, c
         else hipLaunchKernelGGL(k_pf_gemm_skinny<WT_FP8>, grid, block, lds, m->stream, g);
         return sp.splits;
     }
-    dim3 grid((N + PF_BN - 1) / PF_BN, (T + PF_BM - 1) / PF_BM, sp.splits), block(256);
+    const int bn = PF_BN_OF(wt);
+    dim3 grid((N + bn - 1) / bn, (T + PF_BM - 1) / PF_BM, sp.splits), block(256);
     if (wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm<WT_BF16>, grid, block, 0, m->stream, g);
     else if (wt == WT_FP8) hipLaunchKernelGGL(k_pf_gemm<WT_FP8>, grid, block, 0, m->stream, g);
     else hipLaunchKernelGGL(k_pf_gemm<WT_INT4>, grid, block, 0, m->stream, g);

@@ -25,7 +25,12 @@ typedef float pf_f32x16 __attribute__((ext_vector_type(16)));
 #define PF_REG_STAGES 1     // K steps of operand loads held in registers ahead of the multiply (1 or 2)
 #endif
 #define PF_BM 128           // prompt rows per GEMM workgroup tile
-#define PF_BN 128           // weight rows (output channels) per GEMM workgroup tile
+// weight rows (output channels) per GEMM workgroup tile (a wave owns half of them as 32-wide
+// matrix-core tiles): the widest that still leaves two workgroups per CU.  e4m3 tiles need half the
+// staging registers of bf16 ones, so they can be 256 wide (5B, 512 rows: 25.2 -> 19.5 ms); bf16 at
+// 256 spills 11 registers at two workgroups per CU (48 ms) and is slower at one (39.7 - 43.9 ms
+// against 40 ms at 128); 4-bit tiles carry a second accumulator set and stay at one workgroup per CU.
+#define PF_BN_OF(WT) ((WT) == WT_FP8 ? 256 : 128)
 #define PF_BK 32            // reduction elements per step of the streaming (few-row) GEMM; K must be a multiple
 #define PF_BKL 64           // reduction elements per step of the tiled GEMM
 #define PF_LDS_STRIDE 72    // bf16 elements per LDS tile row (144 bytes: 16-byte aligned; 16 consecutive rows
@@ -203,7 +208,8 @@ __device__ __forceinline__ pf_bf16x8 pf_frag(const uint16_t *p) {
 // reduction elements 8 * (l / 32) .. + 7 of both operands; result register i of lane l is
 // C[8 * (i / 4) + 4 * (l / 32) + i % 4][l % 32].
 template <int WT>
-__global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
+__global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g) {
+    constexpr int PF_BN = PF_BN_OF(WT);
     __shared__ __align__(16) uint16_t sAh[PF_BM * PF_LDS_STRIDE];
     __shared__ __align__(16) uint16_t sAl[PF_BM * PF_LDS_STRIDE];
     __shared__ __align__(16) uint16_t sW[PF_BN * PF_LDS_STRIDE];
@@ -213,31 +219,33 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
     const int nsteps = (g.K + PF_BKL - 1) / PF_BKL;
     const int s_begin = z * g.steps_per_split, s_end = min(nsteps, s_begin + g.steps_per_split);
 
-    pf_f32x16 acc[2][2];
+    constexpr int NT = PF_BN / 64;             // 32-channel tiles per wave (a wave owns PF_BN / 2 channels)
+    constexpr int WCH = PF_BN / 32;            // 16-byte chunks of the bf16 weight tile per thread
+    pf_f32x16 acc[2][NT];
 #pragma unroll
     for (int a = 0; a < 2; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < NT; ++b)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.0f;
     // 4-bit weights enter the matrix cores as the exact integers -8..7; the products of one scale
     // group (128 reduction elements = two steps) are summed separately and scaled once, in fp32,
     // like the per-piece scale of the decode GEMV
-    pf_f32x16 accg[WT == WT_INT4 ? 2 : 1][WT == WT_INT4 ? 2 : 1];
+    pf_f32x16 accg[WT == WT_INT4 ? 2 : 1][WT == WT_INT4 ? NT : 1];
     if (WT == WT_INT4) {
 #pragma unroll
         for (int a = 0; a < 2; ++a)
 #pragma unroll
-            for (int b = 0; b < 2; ++b)
+            for (int b = 0; b < NT; ++b)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) accg[a % (WT == WT_INT4 ? 2 : 1)][b % (WT == WT_INT4 ? 2 : 1)][i] = 0.0f;
+                for (int i = 0; i < 16; ++i) accg[a % (WT == WT_INT4 ? 2 : 1)][b % (WT == WT_INT4 ? NT : 1)][i] = 0.0f;
     }
 
     // global -> register staging, two steps ahead of the multiply.  Activation tiles: 128 rows x 8
     // chunks of 8 elements, four chunks per thread for hi and for lo.  Weight tile: bf16 the same;
     // e4m3 128 rows x 4 chunks of 16 elements, two per thread.  Rows past the end re-read the last
     // valid row (their results are not stored); chunks past K are zero.
-    struct Stage { uint4 ah[4], al[4], w[4]; };
+    struct Stage { uint4 ah[4], al[4], w[WCH]; };
     const uint4 zero4 = make_uint4(0, 0, 0, 0);
     auto gload = [&](Stage &s, int step) {
         const int k0 = step * PF_BKL;
@@ -245,28 +253,37 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
         for (int j = 0; j < 4; ++j) {
             const int c = tid + 256 * j, row = c >> 3, k = k0 + (c & 7) * 8;
             const size_t ta = (size_t)min(t0 + row, g.T - 1);
-            s.ah[j] = zero4; s.al[j] = zero4; s.w[j] = zero4;
+            s.ah[j] = zero4; s.al[j] = zero4;
             if (k < g.K) {
                 s.ah[j] = *(const uint4 *)(g.Ahi + ta * g.K + k);
                 s.al[j] = *(const uint4 *)(g.Alo + ta * g.K + k);
-                if (WT == WT_BF16) {
-                    const size_t na = (size_t)min(n0 + row, g.N - 1);
-                    s.w[j] = *(const uint4 *)((const uint16_t *)g.W + na * g.K + k);
-                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < WCH; ++j) s.w[j] = zero4;
+        if (WT == WT_BF16) {
+#pragma unroll
+            for (int j = 0; j < WCH; ++j) {
+                const int c = tid + 256 * j, row = c >> 3, k = k0 + (c & 7) * 8;
+                const size_t na = (size_t)min(n0 + row, g.N - 1);
+                if (k < g.K) s.w[j] = *(const uint4 *)((const uint16_t *)g.W + na * g.K + k);
             }
         }
         if (WT == WT_FP8) {
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            for (int j = 0; j < WCH / 2; ++j) {
                 const int c = tid + 256 * j, row = c >> 2, k = k0 + (c & 3) * 16;
                 const size_t na = (size_t)min(n0 + row, g.N - 1);
                 if (k < g.K) s.w[j] = *(const uint4 *)((const uint8_t *)g.W + na * g.K + k);
             }
         }
-        if (WT == WT_INT4) {       // 128 rows x 2 halves of 32 elements (16 bytes)
-            const int row = tid >> 1, k = k0 + (tid & 1) * 32;
-            const size_t na = (size_t)min(n0 + row, g.N - 1);
-            if (k < g.K) s.w[0] = *(const uint4 *)((const uint8_t *)g.W + na * (size_t)(g.K / 2) + k / 2);
+        if (WT == WT_INT4) {       // PF_BN rows x 2 halves of 32 elements (16 bytes)
+#pragma unroll
+            for (int j = 0; j < WCH / 4; ++j) {
+                const int c = tid + 256 * j, row = c >> 1, k = k0 + (c & 1) * 32;
+                const size_t na = (size_t)min(n0 + row, g.N - 1);
+                if (k < g.K) s.w[j] = *(const uint4 *)((const uint8_t *)g.W + na * (size_t)(g.K / 2) + k / 2);
+            }
         }
     };
     auto lstore = [&](const Stage &s) {
@@ -275,11 +292,17 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
             const int c = tid + 256 * j, row = c >> 3, kc = c & 7;
             *(uint4 *)(sAh + row * PF_LDS_STRIDE + kc * 8) = s.ah[j];
             *(uint4 *)(sAl + row * PF_LDS_STRIDE + kc * 8) = s.al[j];
-            if (WT == WT_BF16) *(uint4 *)(sW + row * PF_LDS_STRIDE + kc * 8) = s.w[j];
+        }
+        if (WT == WT_BF16) {
+#pragma unroll
+            for (int j = 0; j < WCH; ++j) {
+                const int c = tid + 256 * j, row = c >> 3, kc = c & 7;
+                *(uint4 *)(sW + row * PF_LDS_STRIDE + kc * 8) = s.w[j];
+            }
         }
         if (WT == WT_FP8) {
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            for (int j = 0; j < WCH / 2; ++j) {
                 const int c = tid + 256 * j, row = c >> 2, q = c & 3;
                 const uint32_t u[4] = {s.w[j].x, s.w[j].y, s.w[j].z, s.w[j].w};
                 uint32_t o[8];
@@ -299,19 +322,22 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
         if (WT == WT_INT4) {
             // nibble n (offset-binary, element 2j = low nibble of byte j) -> bf16 bits of the integer n - 8:
             // 2^23 + n is exact in fp32, subtracting 2^23 + 8 leaves n - 8, whose upper 16 bits are its bf16 form
-            const int row = tid >> 1, half = tid & 1;
-            const uint32_t u[4] = {s.w[0].x, s.w[0].y, s.w[0].z, s.w[0].w};
-            uint16_t *dst = sW + row * PF_LDS_STRIDE + half * 32;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                uint32_t o[4];
+            for (int j = 0; j < WCH / 4; ++j) {
+                const int c = tid + 256 * j, row = c >> 1, half = c & 1;
+                const uint32_t u[4] = {s.w[j].x, s.w[j].y, s.w[j].z, s.w[j].w};
+                uint16_t *dst = sW + row * PF_LDS_STRIDE + half * 32;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float f0 = __uint_as_float(0x4B000000u | ((u[i] >> (8 * e)) & 0xfu)) - 8388616.0f;
-                    const float f1 = __uint_as_float(0x4B000000u | ((u[i] >> (8 * e + 4)) & 0xfu)) - 8388616.0f;
-                    o[e] = (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xffff0000u);
+                for (int i = 0; i < 4; ++i) {
+                    uint32_t o[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float f0 = __uint_as_float(0x4B000000u | ((u[i] >> (8 * e)) & 0xfu)) - 8388616.0f;
+                        const float f1 = __uint_as_float(0x4B000000u | ((u[i] >> (8 * e + 4)) & 0xfu)) - 8388616.0f;
+                        o[e] = (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xffff0000u);
+                    }
+                    *(uint4 *)(dst + 8 * i) = make_uint4(o[0], o[1], o[2], o[3]);
                 }
-                *(uint4 *)(dst + 8 * i) = make_uint4(o[0], o[1], o[2], o[3]);
             }
         }
     };
@@ -319,27 +345,27 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
         const int r = lane & 31, kq = 8 * (lane >> 5);
 #pragma unroll
         for (int j = 0; j < PF_BKL / 16; ++j) {
-            pf_bf16x8 b[2], ah[2], al[2];
-#pragma unroll
-            for (int nt = 0; nt < 2; ++nt) b[nt] = pf_frag(sW + (64 * wn + 32 * nt + r) * PF_LDS_STRIDE + 16 * j + kq);
+            pf_bf16x8 ah[2], al[2];
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt) {
                 ah[mt] = pf_frag(sAh + (64 * wm + 32 * mt + r) * PF_LDS_STRIDE + 16 * j + kq);
                 al[mt] = pf_frag(sAl + (64 * wm + 32 * mt + r) * PF_LDS_STRIDE + 16 * j + kq);
             }
 #pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
+            for (int nt = 0; nt < NT; ++nt) {
+                const pf_bf16x8 bf = pf_frag(sW + (32 * NT * wn + 32 * nt + r) * PF_LDS_STRIDE + 16 * j + kq);
 #pragma unroll
-                for (int nt = 0; nt < 2; ++nt) {
+                for (int mt = 0; mt < 2; ++mt) {
                     if (WT == WT_INT4) {
-                        pf_f32x16 &t = accg[mt % (WT == WT_INT4 ? 2 : 1)][nt % (WT == WT_INT4 ? 2 : 1)];
-                        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mt], b[nt], t, 0, 0, 0);
-                        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], b[nt], t, 0, 0, 0);
+                        pf_f32x16 &t = accg[mt % (WT == WT_INT4 ? 2 : 1)][nt % (WT == WT_INT4 ? NT : 1)];
+                        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mt], bf, t, 0, 0, 0);
+                        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], bf, t, 0, 0, 0);
                     } else {
-                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mt], b[nt], acc[mt][nt], 0, 0, 0);
-                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], b[nt], acc[mt][nt], 0, 0, 0);
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mt], bf, acc[mt][nt], 0, 0, 0);
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], bf, acc[mt][nt], 0, 0, 0);
                     }
                 }
+            }
         }
     };
     // 4-bit weights: the group that steps (i, i + 1) of this split make up, scaled into the result.
@@ -348,12 +374,12 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
         if (WT != WT_INT4) return;
         const int grp = step / (128 / PF_BKL), kg = g.K / 128;
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-            const size_t na = (size_t)min(n0 + 64 * wn + 32 * nt + (lane & 31), g.N - 1);
+        for (int nt = 0; nt < NT; ++nt) {
+            const size_t na = (size_t)min(n0 + 32 * NT * wn + 32 * nt + (lane & 31), g.N - 1);
             const float sc = __uint_as_float((uint32_t)g.S[na * kg + grp] << 16);
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt) {
-                pf_f32x16 &t = accg[mt % (WT == WT_INT4 ? 2 : 1)][nt % (WT == WT_INT4 ? 2 : 1)];
+                pf_f32x16 &t = accg[mt % (WT == WT_INT4 ? 2 : 1)][nt % (WT == WT_INT4 ? NT : 1)];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) { acc[mt][nt][i] = fmaf(t[i], sc, acc[mt][nt][i]); t[i] = 0.0f; }
             }
@@ -400,8 +426,8 @@ __global__ __launch_bounds__(256) void k_pf_gemm(PfGemm g) {
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-            const int n = n0 + 64 * wn + 32 * nt + r;
+        for (int nt = 0; nt < NT; ++nt) {
+            const int n = n0 + 32 * NT * wn + 32 * nt + r;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int t = t0 + 64 * wm + 32 * mt + 8 * (i >> 2) + 4 * gq + (i & 3);
