@@ -21,9 +21,6 @@
 typedef __bf16 pf_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float pf_f32x16 __attribute__((ext_vector_type(16)));
 
-#ifndef PF_REG_STAGES
-#define PF_REG_STAGES 1     // K steps of operand loads held in registers ahead of the multiply (1 or 2)
-#endif
 #define PF_BM 128           // prompt rows per GEMM workgroup tile
 // weight rows (output channels) per GEMM workgroup tile (a wave owns half of them as 32-wide
 // matrix-core tiles): the widest that still leaves two workgroups per CU.  e4m3 tiles need half the
@@ -351,9 +348,19 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
                 ah[mt] = pf_frag(sAh + (64 * wm + 32 * mt + r) * PF_LDS_STRIDE + 16 * j + kq);
                 al[mt] = pf_frag(sAl + (64 * wm + 32 * mt + r) * PF_LDS_STRIDE + 16 * j + kq);
             }
+            // two workgroups per CU: one weight fragment at a time keeps the kernel within 128 registers
+            // (the other workgroup covers the LDS latency); alone on the CU, all fragments are requested first
+            constexpr bool PRELOAD = (WT == WT_INT4);
+            pf_bf16x8 bpre[PRELOAD ? NT : 1];
+            if (PRELOAD) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    bpre[PRELOAD ? nt : 0] = pf_frag(sW + (32 * NT * wn + 32 * nt + r) * PF_LDS_STRIDE + 16 * j + kq);
+            }
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const pf_bf16x8 bf = pf_frag(sW + (32 * NT * wn + 32 * nt + r) * PF_LDS_STRIDE + 16 * j + kq);
+                const pf_bf16x8 bf = PRELOAD ? bpre[PRELOAD ? nt : 0]
+                                             : pf_frag(sW + (32 * NT * wn + 32 * nt + r) * PF_LDS_STRIDE + 16 * j + kq);
 #pragma unroll
                 for (int mt = 0; mt < 2; ++mt) {
                     if (WT == WT_INT4) {
@@ -387,7 +394,7 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
     };
 
     const int n = s_end - s_begin;
-#if PF_REG_STAGES == 1
+    if constexpr (WT != WT_INT4) {
     // one step of operand loads in flight in registers: 48 registers fewer than two, which lets two
     // workgroups share a CU (one multiplies while the other stages)
     Stage S0;
@@ -398,9 +405,9 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
         __syncthreads();
         if (i + 1 < n) gload(S0, s_begin + i + 1);
         multiply();
-        if (i & 1) scale_group(s_begin + i);   // (splits of 4-bit weights start on a group boundary)
     }
-#else
+    } else {
+    // alone on the CU (the second accumulator set of the 4-bit path): two steps in flight
     Stage S0, S1;
     if (n > 0) gload(S0, s_begin);
     if (n > 1) gload(S1, s_begin + 1);
@@ -419,7 +426,7 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
         }
         scale_group(s_begin + i);              // (splits of 4-bit weights start on a group boundary)
     }
-#endif
+    }
 
     float *Pz = g.P + (size_t)z * g.T * g.N;
     const int r = lane & 31, gq = lane >> 5;
