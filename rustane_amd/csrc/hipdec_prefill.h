@@ -200,9 +200,9 @@ __device__ __forceinline__ pf_bf16x8 pf_frag(const uint16_t *p) {
     return __builtin_bit_cast(pf_bf16x8, v);
 }
 
-// 256 threads = 4 waves in a 2 x 2 arrangement; each wave owns a 64 (rows) x 64 (channels) tile =
-// 2 x 2 MFMA tiles.  Operand layout of v_mfma_f32_32x32x16_bf16: lane l supplies row (l % 32),
-// reduction elements 8 * (l / 32) .. + 7 of both operands; result register i of lane l is
+// 256 threads = 4 waves in a 2 x 2 arrangement; each wave owns 64 rows x PF_BN / 2 channels =
+// 2 x (PF_BN / 64) MFMA tiles.  Operand layout of v_mfma_f32_32x32x16_bf16: lane l supplies row
+// (l % 32), reduction elements 8 * (l / 32) .. + 7 of both operands; result register i of lane l is
 // C[8 * (i / 4) + 4 * (l / 32) + i % 4][l % 32].
 template <int WT>
 __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g) {
@@ -238,10 +238,10 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
                 for (int i = 0; i < 16; ++i) accg[a % (WT == WT_INT4 ? 2 : 1)][b % (WT == WT_INT4 ? NT : 1)][i] = 0.0f;
     }
 
-    // global -> register staging, two steps ahead of the multiply.  Activation tiles: 128 rows x 8
-    // chunks of 8 elements, four chunks per thread for hi and for lo.  Weight tile: bf16 the same;
-    // e4m3 128 rows x 4 chunks of 16 elements, two per thread.  Rows past the end re-read the last
-    // valid row (their results are not stored); chunks past K are zero.
+    // global -> register staging ahead of the multiply.  Activation tiles: 128 rows x 8 chunks of
+    // 8 elements, four chunks per thread for hi and for lo.  Weight tile of PF_BN rows: bf16 8 chunks
+    // per row, e4m3 4 chunks of 16 elements, 4-bit 2 chunks of 32.  Rows past the end re-read the
+    // last valid row (their results are not stored); chunks past K are zero.
     struct Stage { uint4 ah[4], al[4], w[WCH]; };
     const uint4 zero4 = make_uint4(0, 0, 0, 0);
     auto gload = [&](Stage &s, int step) {
