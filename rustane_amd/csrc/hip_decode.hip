@@ -549,7 +549,7 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
             int N = Q + 2 * KV;
             int sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.wqkv, L.s_qkv, T, N, D);
             {
-                const size_t items = (size_t)T * (N / 2);
+                const size_t items = (size_t)T * (N / 4);
                 dim3 grid((unsigned)((items + 255) / 256)), block(256);
                 if (m->kvbf16)
                     hipLaunchKernelGGL(k_pf_qkv_epi<1>, grid, block, 0, m->stream, w.P, sp, (size_t)T * N,

@@ -104,7 +104,8 @@ __global__ __launch_bounds__(PF_CHUNK) void k_pf_resid(const float *__restrict__
 
 // q/k/v rows of the chunk: sum the split planes, scale (8-bit weights), RoPE on interleaved pairs
 // (kernels/sdpa_fwd.rs:18-33, :258-321), q kept as fp32, k and v written into the caches at
-// positions pos0 + t in cache precision.  One thread per (row, channel pair).
+// positions pos0 + t in cache precision.  One thread per (row, two channel pairs): the q, k and v
+// sections are multiples of 4 channels wide, so the two pairs lie in the same section and head.
 template <int KVBF16>
 __global__ __launch_bounds__(256) void k_pf_qkv_epi(const float *__restrict__ P, int splits, size_t plane,
                                                     const float *__restrict__ wscale, float *__restrict__ q,
@@ -112,38 +113,44 @@ __global__ __launch_bounds__(256) void k_pf_qkv_epi(const float *__restrict__ P,
                                                     const float *__restrict__ rope_cos, const float *__restrict__ rope_sin,
                                                     const float *__restrict__ ssq, int nch, int D,
                                                     int T, int Q, int KV, int hd, int pos0) {
-    const int N = Q + 2 * KV, npairs = N >> 1;
+    const int N = Q + 2 * KV, nquads = N >> 2;
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (gid >= (size_t)T * npairs) return;
-    const int t = (int)(gid / npairs), p = (int)(gid - (size_t)t * npairs), row0 = 2 * p;
-    float s0 = 0.0f, s1 = 0.0f;
+    if (gid >= (size_t)T * nquads) return;
+    const int t = (int)(gid / nquads), row0 = 4 * (int)(gid - (size_t)t * nquads);
+    float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     for (int z = 0; z < splits; ++z) {
-        const float2 v = *(const float2 *)(P + z * plane + (size_t)t * N + row0);
-        s0 += v.x; s1 += v.y;
+        const float4 v = *(const float4 *)(P + z * plane + (size_t)t * N + row0);
+        s[0] += v.x; s[1] += v.y; s[2] += v.z; s[3] += v.w;
     }
-    if (wscale) { s0 *= wscale[row0]; s1 *= wscale[row0 + 1]; }
+    if (wscale) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s[e] *= wscale[row0 + e];
+    }
     const float inv = pf_row_inv(ssq, t, nch, D);
-    s0 *= inv; s1 *= inv;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s[e] *= inv;
     const int pos = pos0 + t;
     if (row0 < Q + KV) {
         const int rr = row0 < Q ? row0 : row0 - Q;
         const int pi2 = (rr % hd) >> 1;
-        const float c = rope_cos[(size_t)pos * (hd / 2) + pi2], s = rope_sin[(size_t)pos * (hd / 2) + pi2];
-        const float e = s0 * c - s1 * s, o = s1 * c + s0 * s;
-        s0 = e; s1 = o;
+        const float2 c = *(const float2 *)(rope_cos + (size_t)pos * (hd / 2) + pi2);
+        const float2 sn = *(const float2 *)(rope_sin + (size_t)pos * (hd / 2) + pi2);
+        const float e0 = s[0] * c.x - s[1] * sn.x, o0 = s[1] * c.x + s[0] * sn.x;
+        const float e1 = s[2] * c.y - s[3] * sn.y, o1 = s[3] * c.y + s[2] * sn.y;
+        s[0] = e0; s[1] = o0; s[2] = e1; s[3] = o1;
     }
     if (row0 < Q) {
-        *(float2 *)(q + (size_t)t * Q + row0) = make_float2(s0, s1);
+        *(float4 *)(q + (size_t)t * Q + row0) = make_float4(s[0], s[1], s[2], s[3]);
     } else {
         const bool isk = row0 < Q + KV;
         const int rr = isk ? row0 - Q : row0 - Q - KV;
         void *cache = isk ? kc : vc;
         if (KVBF16) {
             uint16_t *cp = (uint16_t *)cache + (size_t)pos * KV + rr;
-            cp[0] = f32_to_bf16_rne(s0); cp[1] = f32_to_bf16_rne(s1);
+            *(uint2 *)cp = make_uint2((uint32_t)f32_to_bf16_rne(s[0]) | ((uint32_t)f32_to_bf16_rne(s[1]) << 16),
+                                      (uint32_t)f32_to_bf16_rne(s[2]) | ((uint32_t)f32_to_bf16_rne(s[3]) << 16));
         } else {
-            float *cp = (float *)cache + (size_t)pos * KV + rr;
-            cp[0] = s0; cp[1] = s1;
+            *(float4 *)((float *)cache + (size_t)pos * KV + rr) = make_float4(s[0], s[1], s[2], s[3]);
         }
     }
 }
