@@ -111,3 +111,18 @@ def test_chunked_prefill_matches_token_step_prefill():
     ta = a.decode_greedy_run(int(np.argmax(la)), 16)
     tb = b.decode_greedy_run(int(np.argmax(lb)), 16)
     np.testing.assert_array_equal(ta, tb)
+
+
+def test_prefill_longer_than_one_chunk_and_empty_prefill():
+    # 1100 rows = one full 1024-row chunk + a 76-row chunk whose attention starts at position 1024
+    cfg = Config.make(dim=256, hidden=640, heads=2, hd=128, seq=1200, nlayers=2, vocab=320)
+    w, orc, dev = make(cfg)
+    ids = synth.make_prompt(11, cfg.vocab, 1100)
+    lg_o, _, _ = orc.forward_window(ids)
+    dev.prefill(ids[:0], want_logits=False)            # nothing to do, nothing changes
+    assert dev.len() == 0
+    lg_d = dev.prefill(ids)
+    assert dev.len() == 1100
+    assert rel_err(lg_d, lg_o[0]) < 1e-4
+    tok = int(O.argmax_lower(lg_o[0]))
+    assert rel_err(dev.decode_logits_from_id(tok), orc.decode_logits_from_id(tok)) < 1e-4
