@@ -46,8 +46,9 @@ MEASURED_TRAFFIC_BYTES = {"c2_600m_bf16_bs1": 1.514e9}
 
 def run_c3(args, cfg, weights, n_prompt):
     """Multi-sample workload through the session layer: a step is one pass of the weights that
-    advances all 8 samples by one token (top-k candidates on the device, the reference's sampler on
-    the host); value = sampled tokens per second over all samples."""
+    advances all 8 samples by one token (per-block top-k candidates, their merge and the reference's
+    draw, all on the device: the whole request is one enqueued run); value = sampled tokens per
+    second over all samples."""
     from rustane_amd import engine as E
     from rustane_amd import synth
     prompt = synth.make_prompt(7, cfg.vocab, n_prompt)
@@ -128,8 +129,9 @@ def run_c4_sampled(args, cfg, dev, kvdt, prompt_logits, n_prompt, gen_steps, pre
                    prefill_flops, mfma_peak):
     """The 5B workload as defined: full-vocabulary sampling at temperature 1.0 through the exact
     block-stats path (crates/engine/src/inference.rs:600-625) -- per token one decode step that
-    leaves per-block (max, sum exp) on the device, a block drawn on the host, that block's logits
-    fetched, the token drawn inside it (two uniforms per token, the reference's LCG, seed 1)."""
+    leaves per-block (max, sum exp) on the device, a block drawn from them, the token drawn inside
+    that block's logits (two uniforms per token, the reference's LCG, seed 1).  Both draws run on the
+    device with the host's arithmetic, so the K steps are one enqueued run."""
     import ctypes as C
     from rustane_amd import engine as E
     L = E.lib()
@@ -141,20 +143,15 @@ def run_c4_sampled(args, cfg, dev, kvdt, prompt_logits, n_prompt, gen_steps, pre
     K, W = args.steps, args.warmup
     K = min(K, gen_steps - 1, cfg.seq - n_prompt - W - 1)
 
-    def step(tok):
-        mx, sm = dev.decode_token_block_stats_from_id(tok, 1.0 / T, 0.0)
-        ms = dev.last_device_ms()
-        blk = int(L.rs_sample_block_from_stats(mx.ctypes.data_as(fp), sm.ctypes.data_as(fp), mx.size, C.byref(rng)))
-        bl = dev.materialize_current_logits_block(blk, 0.0)
-        return int(L.rs_sample_block_logits(blk * 256, bl.ctypes.data_as(fp), bl.size, T, C.byref(rng))), ms
-    for _ in range(W):
-        cur, _ = step(cur)
+    state = rng.value
+    if W > 0:
+        toks, state = dev.decode_fullvocab_sampled_run(cur, T, state, W)
+        cur = int(toks[-1])
     kv0 = dev.len()
-    dev_ms, t0 = 0.0, time.perf_counter()
-    for _ in range(K):
-        cur, ms = step(cur)
-        dev_ms += ms
+    t0 = time.perf_counter()
+    toks, state = dev.decode_fullvocab_sampled_run(cur, T, state, K)
     wall = time.perf_counter() - t0
+    dev_ms = dev.last_device_ms()
     mean_kv = kv0 + (K + 1) // 2
     bytes_per_step = dev.bytes_per_token(mean_kv)
     achieved = bytes_per_step * K / (dev_ms * 1e-3) / 1e9
@@ -171,6 +168,7 @@ def run_c4_sampled(args, cfg, dev, kvdt, prompt_logits, n_prompt, gen_steps, pre
         "device_ms_per_step": dev_ms / K,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "bytes_per_step": bytes_per_step},
+        "sampled_head": [int(t) for t in toks[:4]],
     }
 
 

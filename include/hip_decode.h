@@ -170,6 +170,30 @@ int hipdec_materialize_current_logits_block_batch(hipdec_model *m, size_t row, s
  * out_tokens[n_steps].  Equivalent to n_steps calls of hipdec_decode_token_argmax_from_id. */
 int hipdec_decode_greedy_run(hipdec_model *m, uint32_t token, size_t n_steps, uint32_t *out_tokens);
 
+/* Sampled runs without a host round trip per token.  The reference finishes every sampled step on
+ * the CPU: it merges the per-block candidates and draws among them (engine/src/inference.rs:586-599,
+ * engine/src/decode.rs:218-253, inference.rs:823-849), or draws a block from the block statistics
+ * and then a token from that block's logits (inference.rs:600-625, :851-921).  These calls do the
+ * same merge and the same draws on the GPU, in the host's operation order and with the host C
+ * library's expf reproduced bit for bit, feed each drawn token to the next step on the device and
+ * return n_steps tokens at once; *rng_state is the sampler's 64-bit LCG state (inference.rs:759-768),
+ * read at entry and advanced exactly as the host loop would advance it.  Equivalent to n_steps
+ * rounds of hipdec_decode_token_topk_from_id + host merge + host draw (resp.
+ * hipdec_decode_token_block_stats_from_id + block draw + hipdec_materialize_current_logits_block +
+ * token draw).  The top-k form returns HIPDEC_ERR_UNSUPPORTED with softcap > 0 (the host applies
+ * tanhf to the merged candidates; that function is not reproduced on the device): use the per-step
+ * calls then.  Needs vocab <= 262144. */
+int hipdec_decode_topk_sampled_run(hipdec_model *m, uint32_t token, uint32_t top_k, float temperature, float softcap,
+                                   uint64_t *rng_state, size_t n_steps, uint32_t *out_tokens);
+int hipdec_decode_fullvocab_sampled_run(hipdec_model *m, uint32_t token, float temperature, float softcap,
+                                        uint64_t *rng_state, size_t n_steps, uint32_t *out_tokens);
+/* The same for every row of an open batch: tokens[n_rows], rng_states[n_rows] (row r draws from its
+ * own state, the reference's seed + r, inference.rs:256), out_tokens[n_steps][n_rows]. */
+int hipdec_decode_topk_sampled_run_batch(hipdec_model *m, const uint32_t *tokens, uint32_t top_k, float temperature,
+                                         float softcap, uint64_t *rng_states, size_t n_steps, uint32_t *out_tokens);
+int hipdec_decode_fullvocab_sampled_run_batch(hipdec_model *m, const uint32_t *tokens, float temperature, float softcap,
+                                              uint64_t *rng_states, size_t n_steps, uint32_t *out_tokens);
+
 /* Device time of the last call that ran a step (a single decode step, a multi-row step,
  * hipdec_decode_greedy_run, hipdec_prefill), measured with HIP events on the model's stream: total
  * milliseconds of that call's kernels. */
@@ -192,6 +216,16 @@ int hipdec_debug_step_profile(hipdec_model *m, uint32_t token, uint64_t *out, si
 /* Diagnostic: `reps` launches of a plain device-to-device copy kernel (k_calib_copy) of `bytes` bytes,
  * the known-size yardstick that hardware memory-traffic counters are scaled by. */
 int hipdec_debug_calibration_copy(size_t bytes, int reps);
+
+/* Verification of the exponential the on-device sampler uses (a restatement of the host C library's
+ * expf): evaluate it for n inputs on the host (on_device = 0) or on the GPU; */
+int hipdec_debug_expf(const float *in, float *out, size_t n, int on_device);
+/* an order-independent checksum of its results over `count` consecutive float bit patterns starting
+ * at first_bits, computed on the host (with host_threads threads) or on the GPU: equal checksums
+ * mean equal results; */
+int hipdec_debug_expf_checksum(uint32_t first_bits, uint64_t count, int on_device, int host_threads, uint64_t *out);
+/* and the number of those inputs for which the host evaluation differs from the C library's expf. */
+int hipdec_debug_expf_count_mismatch(uint32_t first_bits, uint64_t count, int host_threads, uint64_t *out_mismatches);
 
 #ifdef __cplusplus
 }

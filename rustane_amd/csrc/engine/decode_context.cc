@@ -165,6 +165,42 @@ void DecodeContext::decode_greedy_run(uint32_t token, size_t n_steps, uint32_t *
     check(hipdec_decode_greedy_run(m_, token, n_steps, out), "decode_greedy_run");
 }
 
+bool DecodeContext::sample_topk_run(uint32_t token, size_t top_k, float temperature, float softcap, uint64_t *rng,
+                                    size_t n_steps, uint32_t *out) {
+    if (top_k > MAX_GPU_TOPK) top_k = MAX_GPU_TOPK;            // decode.rs:140
+    if (top_k > vocab_) top_k = vocab_;
+    const int rc = hipdec_decode_topk_sampled_run(m_, token, (uint32_t)top_k, temperature, softcap, rng, n_steps, out);
+    if (rc == HIPDEC_ERR_UNSUPPORTED) return false;
+    check(rc, "sample_topk_run");
+    return true;
+}
+
+bool DecodeContext::sample_fullvocab_run(uint32_t token, float temperature, float softcap, uint64_t *rng, size_t n_steps,
+                                         uint32_t *out) {
+    const int rc = hipdec_decode_fullvocab_sampled_run(m_, token, temperature, softcap, rng, n_steps, out);
+    if (rc == HIPDEC_ERR_UNSUPPORTED) return false;
+    check(rc, "sample_fullvocab_run");
+    return true;
+}
+
+bool DecodeContext::sample_topk_run_batch(const uint32_t *tokens, size_t top_k, float temperature, float softcap,
+                                          uint64_t *rngs, size_t n_steps, uint32_t *out) {
+    if (top_k > MAX_GPU_TOPK) top_k = MAX_GPU_TOPK;            // decode.rs:140
+    if (top_k > vocab_) top_k = vocab_;
+    const int rc = hipdec_decode_topk_sampled_run_batch(m_, tokens, (uint32_t)top_k, temperature, softcap, rngs, n_steps, out);
+    if (rc == HIPDEC_ERR_UNSUPPORTED) return false;
+    check(rc, "sample_topk_run_batch");
+    return true;
+}
+
+bool DecodeContext::sample_fullvocab_run_batch(const uint32_t *tokens, float temperature, float softcap, uint64_t *rngs,
+                                               size_t n_steps, uint32_t *out) {
+    const int rc = hipdec_decode_fullvocab_sampled_run_batch(m_, tokens, temperature, softcap, rngs, n_steps, out);
+    if (rc == HIPDEC_ERR_UNSUPPORTED) return false;
+    check(rc, "sample_fullvocab_run_batch");
+    return true;
+}
+
 bool DecodeContext::batch_begin(size_t rows) {
     const int rc = hipdec_batch_begin(m_, rows);
     if (rc == HIPDEC_ERR_UNSUPPORTED) return false;

@@ -52,6 +52,18 @@ public:
     // not in the reference: prompt prefill on the GPU and greedy runs without per-token host round trips
     const std::vector<float> &prefill(const uint32_t *ids, size_t n, float softcap);
     void decode_greedy_run(uint32_t token, size_t n_steps, uint32_t *out);
+    // The sampled loops of inference.rs:586-625 run on the device for n_steps tokens: candidates merged
+    // and drawn (top_k in 1..=MAX_GPU_TOPK), or block then token drawn from the block statistics.
+    // *rng advances as the host loop would advance it.  false: the backend does not serve this
+    // request on the device (nothing has run; use the per-step calls).
+    bool sample_topk_run(uint32_t token, size_t top_k, float temperature, float softcap, uint64_t *rng, size_t n_steps,
+                         uint32_t *out);
+    bool sample_fullvocab_run(uint32_t token, float temperature, float softcap, uint64_t *rng, size_t n_steps, uint32_t *out);
+    // the same for every row of an open batch; out[n_steps][rows]
+    bool sample_topk_run_batch(const uint32_t *tokens, size_t top_k, float temperature, float softcap, uint64_t *rngs,
+                               size_t n_steps, uint32_t *out);
+    bool sample_fullvocab_run_batch(const uint32_t *tokens, float temperature, float softcap, uint64_t *rngs,
+                                    size_t n_steps, uint32_t *out);
     // not in the reference: `rows` continuations of the current cache contents stepped together
     // (the reference runs its samples one after the other, inference.rs:247-262).  batch_begin
     // returns false when the backend has no multi-row path for this model.

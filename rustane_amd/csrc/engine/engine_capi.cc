@@ -122,6 +122,7 @@ rs_session *rs_session_new(const rs_config *c, const rs_weights *w, const uint32
     o.kv_dtype = (KvDtype)kv_dtype;
     o.flags = flags & 0xffu;                  // HIPDEC_FLAG_* for the backend
     o.batch_samples = !(flags & 0x100u);      // 0x100: run the samples of a request one after the other
+    o.device_sampling = !(flags & 0x200u);    // 0x200: draw every sampled token on the host, as the reference does
     std::string e;
     std::unique_ptr<rs_session> s(new rs_session());
     s->s.reset(new InferenceSession(to_cfg(c), w->w, std::vector<uint32_t>(prompt, prompt + n), softcap, o, &e));

@@ -116,8 +116,9 @@ uint32_t sample_next(const float *logits, size_t n, float temperature, size_t to
     std::vector<size_t> &ix = scratch ? *scratch : local;
     ix.resize(n);
     for (size_t i = 0; i < n; ++i) ix[i] = i;
-    // descending by total_cmp; the reference's sort is unstable, equal values are ordered by index here
-    std::sort(ix.begin(), ix.end(), [&](size_t a, size_t b) {
+    // descending by total_cmp; the reference's sort is unstable, equal values are ordered by index here.
+    // Only the first top_k places survive the truncate (inference.rs:795-797), so only they are sorted.
+    std::partial_sort(ix.begin(), ix.begin() + (ptrdiff_t)top_k, ix.end(), [&](size_t a, size_t b) {
         int32_t ka = total_key(logits[a]), kb = total_key(logits[b]);
         return ka != kb ? ka > kb : a < b;
     });
@@ -196,7 +197,8 @@ size_t fill_input_window(const std::vector<uint32_t> &generated, size_t seq, std
 InferenceSession::InferenceSession(const ModelConfig &cfg, const ModelWeights &weights,
                                    const std::vector<uint32_t> &prompt_ids, float softcap, const SessionOptions &opts,
                                    std::string *err)
-    : cfg_(cfg), prompt_ids_(prompt_ids), softcap_(softcap), batch_samples_(opts.batch_samples) {
+    : cfg_(cfg), prompt_ids_(prompt_ids), softcap_(softcap), device_sampling_(opts.device_sampling),
+      batch_samples_(opts.batch_samples) {
     err->clear();
     if (prompt_ids.empty()) { *err = "prompt must contain at least one token"; return; }           // inference.rs:131-133
     *err = validate_token_ids(prompt_ids.data(), prompt_ids.size(), cfg.vocab, "prompt");
@@ -340,21 +342,34 @@ bool InferenceSession::run_cached_sample(const std::vector<uint32_t> &prompt, co
                 }
             }
         } else if (req.top_k > 0 && req.top_k <= MAX_GPU_TOPK) {                   // :586-599
-            for (size_t i = 1; i < req.steps; ++i) {
-                const uint32_t *idxs; const float *lg; size_t n;
-                ctx_->decode_next_topk_candidates(cur, req.top_k, softcap_, &idxs, &lg, &n);
-                cur = sample_topk_candidates(idxs, lg, n, req.temperature, &rng);
-                if (!emit(cur)) return false;
+            // no per-token consumer: merge and draw on the device, the run returns all tokens at once
+            std::vector<uint32_t> run(req.steps - 1);
+            if (!cb && device_sampling_ && req.steps > 1 &&
+                ctx_->sample_topk_run(cur, req.top_k, req.temperature, softcap_, &rng, run.size(), run.data())) {
+                for (uint32_t tok : run) emit(tok);
+            } else {
+                for (size_t i = 1; i < req.steps; ++i) {
+                    const uint32_t *idxs; const float *lg; size_t n;
+                    ctx_->decode_next_topk_candidates(cur, req.top_k, softcap_, &idxs, &lg, &n);
+                    cur = sample_topk_candidates(idxs, lg, n, req.temperature, &rng);
+                    if (!emit(cur)) return false;
+                }
             }
         } else if (req.top_k == 0) {                                               // :600-625
-            for (size_t i = 1; i < req.steps; ++i) {
-                const float *mx, *sm; size_t nb;
-                ctx_->decode_next_fullvocab_block_stats(cur, req.temperature, softcap_, &mx, &sm, &nb);
-                const size_t blk = sample_block_from_stats(mx, sm, nb, &rng);
-                const float *bl; size_t nv;
-                ctx_->materialize_current_logits_block(blk, softcap_, &bl, &nv);
-                cur = sample_block_logits((uint32_t)(blk * 256), bl, nv, req.temperature, &rng);   // :613
-                if (!emit(cur)) return false;
+            std::vector<uint32_t> run(req.steps - 1);
+            if (!cb && device_sampling_ && req.steps > 1 &&
+                ctx_->sample_fullvocab_run(cur, req.temperature, softcap_, &rng, run.size(), run.data())) {
+                for (uint32_t tok : run) emit(tok);
+            } else {
+                for (size_t i = 1; i < req.steps; ++i) {
+                    const float *mx, *sm; size_t nb;
+                    ctx_->decode_next_fullvocab_block_stats(cur, req.temperature, softcap_, &mx, &sm, &nb);
+                    const size_t blk = sample_block_from_stats(mx, sm, nb, &rng);
+                    const float *bl; size_t nv;
+                    ctx_->materialize_current_logits_block(blk, softcap_, &bl, &nv);
+                    cur = sample_block_logits((uint32_t)(blk * 256), bl, nv, req.temperature, &rng);   // :613
+                    if (!emit(cur)) return false;
+                }
             }
         } else {                                                                   // :626-638
             for (size_t i = 1; i < req.steps; ++i) {
@@ -395,7 +410,25 @@ bool InferenceSession::run_cached_batch(const std::vector<uint32_t> &prompt, con
         res[r].sampled.push_back(cur[r]);
     }
     batch_device_ms_ = 0.0;
-    for (size_t i = 1; i < req.steps; ++i) {
+    size_t first_host_step = 1;
+    if (device_sampling_ && req.steps > 1 && req.temperature > 0.0f && req.top_k != 1 && req.top_k <= MAX_GPU_TOPK) {
+        // every remaining step of every row on the device (the draws of :586-625 included)
+        const size_t n = req.steps - 1;
+        std::vector<uint32_t> run(n * R);
+        const bool ran = req.top_k > 0
+            ? ctx_->sample_topk_run_batch(cur.data(), req.top_k, req.temperature, softcap_, rng.data(), n, run.data())
+            : ctx_->sample_fullvocab_run_batch(cur.data(), req.temperature, softcap_, rng.data(), n, run.data());
+        if (ran) {
+            batch_device_ms_ += ctx_->last_device_ms();
+            for (size_t i = 0; i < n; ++i)
+                for (size_t r = 0; r < R; ++r) {
+                    res[r].generated.push_back(run[i * R + r]);
+                    res[r].sampled.push_back(run[i * R + r]);
+                }
+            first_host_step = req.steps;
+        }
+    }
+    for (size_t i = first_host_step; i < req.steps; ++i) {
         if (req.temperature <= 0.0f || req.top_k == 1) {                           // :576-585
             ctx_->decode_next_greedy_tokens(cur.data(), nxt.data());
             batch_device_ms_ += ctx_->last_device_ms();

@@ -87,6 +87,10 @@ struct SessionOptions {
     // (the reference runs them one after the other, inference.rs:247-262; results per sample are
     // the same).  false restores the sequential loop.
     bool batch_samples = true;
+    // sampled requests without a per-token consumer draw their tokens on the device and run without a
+    // host round trip per token; false restores the reference's loop (candidates or block statistics
+    // read back and drawn on the host each step, inference.rs:586-625).  Tokens are the same.
+    bool device_sampling = true;
 };
 
 // inference.rs:107-452.  Errors the reference returns as Err(String) come back through `err`
@@ -132,6 +136,7 @@ private:
     std::vector<uint32_t> prompt_ids_, input_;
     size_t prompt_len_ = 0;
     float softcap_ = 0.0f;
+    bool device_sampling_ = true;
     double prefill_elapsed_ = 0.0;
     std::vector<float> prompt_logits_;
     std::vector<size_t> sampler_scratch_;

@@ -4,6 +4,7 @@
 #include "hipdec_mega.h"
 #include "hipdec_prefill.h"
 #include "hipdec_batch.h"
+#include "hipdec_sample.h"
 
 #include <math.h>
 #include <stdio.h>
@@ -12,10 +13,12 @@
 #include <string>
 #include <vector>
 #include <algorithm>
+#include <thread>
 
 namespace {
 
-enum Variant { V_X = 0, V_ARGMAX, V_TOPK, V_STATS, V_LOGITS, V_COUNT };
+// V_TOPK_S / V_STATS_S: the same step followed by the on-device draw (hipdec_sample.h)
+enum Variant { V_X = 0, V_ARGMAX, V_TOPK, V_STATS, V_LOGITS, V_TOPK_S, V_STATS_S, V_COUNT };
 
 struct DevLayer {
     void *wqkv = nullptr, *wo = nullptr, *w13 = nullptr, *w2 = nullptr;
@@ -41,7 +44,7 @@ struct PrefillWork {
 
 // State of the multi-sample decode (hipdec_batch.h): rows share cache positions [0, prefix) and
 // append to their own suffix caches.
-enum BatchVariant { B_LOGITS = 0, B_ARGMAX, B_TOPK, B_STATS };
+enum BatchVariant { B_LOGITS = 0, B_ARGMAX, B_TOPK, B_STATS, B_TOPK_S, B_STATS_S, B_COUNT };
 struct BatchState {
     int rows = 0;                        // 0: no batch open
     size_t prefix = 0, slot = 0;
@@ -54,11 +57,19 @@ struct BatchState {
     float *h_stage = nullptr;            // pinned, cap_rows * max(vocab, 2 * blocks * 32) floats
     size_t h_stage_floats = 0;
     bool have_logits = false;            // a step has run since hipdec_batch_begin
-    hipGraphExec_t graphs[4] = {};       // one captured step per head variant, for graph_rows rows
+    hipGraphExec_t graphs[B_COUNT] = {}; // one captured step per head variant, for graph_rows rows
+    uint32_t *d_ring = nullptr, *h_ring = nullptr;   // tokens of a sampled run, [steps][rows]; h_ring pinned
+    size_t ring_elems = 0;
     int graph_rows = 0;
 };
 
 }  // namespace
+
+// run state of the on-device sampler as the host stages it (pinned)
+struct SampleHost {
+    SampleParams ss;
+    uint64_t rng[32];
+};
 
 struct hipdec_model {
     hipdec_config cfg{};
@@ -94,6 +105,9 @@ struct hipdec_model {
     unsigned *d_epochs = nullptr;
     PrefillWork pf;
     BatchState bt;
+    SampleParams *d_ss = nullptr;                     // on-device sampler (hipdec_sample.h)
+    uint64_t *d_rng = nullptr;                        // [32], one state per row
+    SampleHost *h_samp = nullptr;                     // pinned
     std::vector<void *> allocs;
     std::string err;
 };
@@ -240,6 +254,18 @@ template <int WT> hipError_t mega_set_lds_t(hipdec_model *m) {
 void enqueue_step(hipdec_model *m, int variant) {
     const hipdec_config &c = m->cfg;
     const int D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden, V = c.vocab;
+    if (variant == V_TOPK_S || variant == V_STATS_S) {
+        // the candidate / statistics step, then the draw; the drawn token becomes the next step's input
+        enqueue_step(m, variant == V_TOPK_S ? V_TOPK : V_STATS);
+        uint32_t *tok_out = (uint32_t *)&m->d_sp->tok;
+        if (variant == V_TOPK_S)
+            hipLaunchKernelGGL(k_sample_topk, dim3(1), dim3(256), 0, m->stream, m->d_topk_vals, m->d_topk_idxs, m->blocks,
+                               m->d_ss, m->d_rng, tok_out, m->d_ring, (BatchParams *)nullptr);
+        else
+            hipLaunchKernelGGL(k_sample_fullvocab, dim3(1), dim3(256), 0, m->stream, m->logits, V, m->d_bmax, m->d_bsum,
+                               m->blocks, m->d_ss, m->d_rng, tok_out, m->d_ring, (BatchParams *)nullptr);
+        return;
+    }
     if (m->mega_ok) {
         // the whole step in one persistent launch; with 8-bit/4-bit weights the (bf16) LM head
         // stays a separate GEMV
@@ -612,6 +638,10 @@ int batch_alloc(hipdec_model *m, int rows) {
     if ((rc = dalloc(m, &b.d_bmax, (size_t)rows * blocks * 4))) return rc;
     if ((rc = dalloc(m, &b.d_bsum, (size_t)rows * blocks * 4))) return rc;
     if ((rc = dalloc(m, &b.d_tok, (size_t)rows * 4))) return rc;
+    b.ring_elems = (size_t)rows * c.seq;
+    if ((rc = dalloc(m, &b.d_ring, b.ring_elems * 4))) return rc;
+    if (b.h_ring) (void)hipHostFree(b.h_ring);
+    HCHK(hipHostMalloc((void **)&b.h_ring, b.ring_elems * 4));
     if (b.h_stage) (void)hipHostFree(b.h_stage);
     b.h_stage_floats = (size_t)rows * std::max(V, 2 * blocks * HIPDEC_MAX_GPU_TOPK);
     HCHK(hipHostMalloc((void **)&b.h_stage, b.h_stage_floats * 4));
@@ -620,6 +650,33 @@ int batch_alloc(hipdec_model *m, int rows) {
 }
 
 void batch_enqueue(hipdec_model *m, int variant);
+
+// Everything that changes from step to step (tokens, position, sampler parameters) lives in device
+// memory, so the ~210 launches of a step are captured once per (rows, head variant) and replayed.
+int batch_launch(hipdec_model *m, int variant) {
+    BatchState &b = m->bt;
+    const int R = b.rows;
+    if (m->opt.flags & HIPDEC_FLAG_NO_GRAPH) {
+        batch_enqueue(m, variant);
+        HCHK(hipGetLastError());
+        return HIPDEC_OK;
+    }
+    if (b.graph_rows != R) {
+        for (auto &g : b.graphs) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
+        b.graph_rows = R;
+    }
+    if (!b.graphs[variant]) {
+        hipGraph_t g = nullptr;
+        HCHK(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
+        batch_enqueue(m, variant);
+        hipError_t e = hipStreamEndCapture(m->stream, &g);
+        if (e != hipSuccess || !g) { m->err = std::string("graph capture failed: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+        HCHK(hipGraphInstantiate(&b.graphs[variant], g, nullptr, nullptr, 0));
+        HCHK(hipGraphDestroy(g));
+    }
+    HCHK(hipGraphLaunch(b.graphs[variant], m->stream));
+    return HIPDEC_OK;
+}
 
 // one step of every open row: tokens[r] at position prefix + slot
 int batch_step(hipdec_model *m, const uint32_t *tokens, int variant, uint32_t top_k, float inv_t, float softcap) {
@@ -640,28 +697,7 @@ int batch_step(hipdec_model *m, const uint32_t *tokens, int variant, uint32_t to
     HCHK(hipMemcpyAsync(w.ids, w.h_ids, (size_t)R * 4, hipMemcpyHostToDevice, m->stream));
     HCHK(hipMemcpyAsync(b.d_bp, b.h_bp, sizeof(BatchParams), hipMemcpyHostToDevice, m->stream));
     HCHK(hipEventRecord(m->ev0, m->stream));
-    // Everything that changes from step to step (tokens, position, sampler parameters) was just
-    // written to device memory, so the ~210 launches of a step are captured once per (rows, head
-    // variant) and replayed.
-    if (m->opt.flags & HIPDEC_FLAG_NO_GRAPH) {
-        batch_enqueue(m, variant);
-        HCHK(hipGetLastError());
-    } else {
-        if (b.graph_rows != R) {
-            for (auto &g : b.graphs) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
-            b.graph_rows = R;
-        }
-        if (!b.graphs[variant]) {
-            hipGraph_t g = nullptr;
-            HCHK(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
-            batch_enqueue(m, variant);
-            hipError_t e = hipStreamEndCapture(m->stream, &g);
-            if (e != hipSuccess || !g) { m->err = std::string("graph capture failed: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
-            HCHK(hipGraphInstantiate(&b.graphs[variant], g, nullptr, nullptr, 0));
-            HCHK(hipGraphDestroy(g));
-        }
-        HCHK(hipGraphLaunch(b.graphs[variant], m->stream));
-    }
+    if ((rc = batch_launch(m, variant))) return rc;
     HCHK(hipEventRecord(m->ev1, m->stream));
     b.slot += 1;
     b.have_logits = true;
@@ -722,11 +758,18 @@ void batch_enqueue(hipdec_model *m, int variant) {
     }
     if (variant == B_ARGMAX)
         hipLaunchKernelGGL(k_bd_argmax, dim3(R), dim3(1024), 0, m->stream, b.logits, V, b.d_tok);
-    else if (variant == B_TOPK)
+    else if (variant == B_TOPK || variant == B_TOPK_S)
         hipLaunchKernelGGL(k_bd_topk, dim3(m->blocks, R), dim3(256), 0, m->stream, b.logits, V, b.d_bp, b.d_vals, b.d_idxs);
-    else if (variant == B_STATS)
+    else if (variant == B_STATS || variant == B_STATS_S)
         hipLaunchKernelGGL(k_bd_block_stats, dim3(m->blocks, R), dim3(256), 0, m->stream, b.logits, V, b.d_bp, b.d_bmax,
                            b.d_bsum);
+    // the draw on the device: each row's token goes where the next step's embedding lookup reads it
+    if (variant == B_TOPK_S)
+        hipLaunchKernelGGL(k_sample_topk, dim3(R), dim3(256), 0, m->stream, b.d_vals, b.d_idxs, m->blocks, m->d_ss, m->d_rng,
+                           w.ids, b.d_ring, b.d_bp);
+    else if (variant == B_STATS_S)
+        hipLaunchKernelGGL(k_sample_fullvocab, dim3(R), dim3(256), 0, m->stream, b.logits, V, b.d_bmax, b.d_bsum, m->blocks,
+                           m->d_ss, m->d_rng, w.ids, b.d_ring, b.d_bp);
 }
 
 // copies `floats` values from device memory to the caller through the pinned staging buffer
@@ -738,6 +781,112 @@ int batch_fetch(hipdec_model *m, const void *dev, void *host, size_t floats) {
     HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
     memcpy(host, b.h_stage, floats * 4);
     return HIPDEC_OK;
+}
+
+// ---- sampled runs that stay on the device (hipdec_sample.h)
+float sample_inv_temperature(float temperature) {              // engine/src/decode.rs:174
+    const float tiny = 1.17549435e-38f;                        // f32::MIN_POSITIVE
+    return 1.0f / (temperature > tiny ? temperature : tiny);
+}
+
+int sampled_args_ok(hipdec_model *m, bool topk, uint32_t top_k, float temperature, float softcap, const uint64_t *rng,
+                    const uint32_t *out_tokens) {
+    if (!rng || !out_tokens) return fail(m, HIPDEC_ERR_ARG, "null buffer");
+    if (m->blocks > SAMPLE_MAX_BLOCKS) return fail(m, HIPDEC_ERR_UNSUPPORTED, "on-device sampling serves up to 1024 vocab blocks");
+    if (topk) {
+        if (top_k == 0 || top_k > HIPDEC_MAX_GPU_TOPK) return fail(m, HIPDEC_ERR_ARG, "gpu top-k only supports k in 1..32");
+        if (softcap > 0.0f)
+            return fail(m, HIPDEC_ERR_UNSUPPORTED, "on-device top-k sampling does not reproduce the host's tanh: use the per-step calls with a softcap");
+    } else if (!(temperature > 0.0f)) {
+        return fail(m, HIPDEC_ERR_ARG, "full-vocab sampling needs a positive temperature");
+    }
+    return HIPDEC_OK;
+}
+
+int sampled_run(hipdec_model *m, int variant, uint32_t token, uint32_t top_k, float temperature, float softcap,
+                uint64_t *rng_state, size_t n_steps, uint32_t *out_tokens) {
+    int rc = check_step(m, token, true);
+    if (rc) return rc;
+    if (n_steps == 0) return HIPDEC_OK;
+    if ((rc = sampled_args_ok(m, variant == V_TOPK_S, top_k, temperature, softcap, rng_state, out_tokens))) return rc;
+    if (m->bt.rows) return fail(m, HIPDEC_ERR_ARG, "a batch is open: use the *_batch calls");
+    if (m->len + n_steps > m->cfg.seq) return fail(m, HIPDEC_ERR_FULL, "sampled run exceeds cfg.seq");
+    StepParams p = base_params(m, token);
+    p.top_k = (int)top_k; p.inv_t = sample_inv_temperature(temperature); p.softcap = softcap;
+    m->h_sp[0] = p;
+    m->h_samp->ss = SampleParams{temperature, softcap, (int)top_k, 0, (int)m->cfg.seq, 0u};
+    m->h_samp->rng[0] = *rng_state;
+    HCHK(hipMemcpyAsync(m->d_sp, &m->h_sp[0], sizeof(StepParams), hipMemcpyHostToDevice, m->stream));
+    HCHK(hipMemcpyAsync(m->d_ss, &m->h_samp->ss, sizeof(SampleParams), hipMemcpyHostToDevice, m->stream));
+    HCHK(hipMemcpyAsync(m->d_rng, m->h_samp->rng, sizeof(uint64_t), hipMemcpyHostToDevice, m->stream));
+    HCHK(hipEventRecord(m->ev0, m->stream));
+    for (size_t i = 0; i < n_steps; ++i)
+        if ((rc = run_step(m, variant))) return rc;
+    HCHK(hipEventRecord(m->ev1, m->stream));
+    HCHK(hipMemcpyAsync(m->h_out, m->d_ring, n_steps * 4, hipMemcpyDeviceToHost, m->stream));
+    HCHK(hipMemcpyAsync(m->h_samp->rng, m->d_rng, sizeof(uint64_t), hipMemcpyDeviceToHost, m->stream));
+    SYNC_CHECKED(m);
+    HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+    memcpy(out_tokens, m->h_out, n_steps * 4);
+    *rng_state = m->h_samp->rng[0];
+    m->len += n_steps;
+    return HIPDEC_OK;
+}
+
+int batch_sampled_run(hipdec_model *m, int variant, const uint32_t *tokens, uint32_t top_k, float temperature, float softcap,
+                      uint64_t *rng_states, size_t n_steps, uint32_t *out_tokens) {
+    if (!m) return HIPDEC_ERR_ARG;
+    const hipdec_config &c = m->cfg;
+    BatchState &b = m->bt;
+    if (b.rows <= 0) return fail(m, HIPDEC_ERR_ARG, "no batch is open (hipdec_batch_begin)");
+    if (!tokens) return fail(m, HIPDEC_ERR_ARG, "null buffer");
+    if (n_steps == 0) return HIPDEC_OK;
+    int rc = sampled_args_ok(m, variant == B_TOPK_S, top_k, temperature, softcap, rng_states, out_tokens);
+    if (rc) return rc;
+    if (b.prefix + b.slot + n_steps > c.seq) return fail(m, HIPDEC_ERR_FULL, "sampled run exceeds cfg.seq");
+    const int R = b.rows;
+    for (int r = 0; r < R; ++r)
+        if (tokens[r] >= c.vocab) return fail(m, HIPDEC_ERR_ARG, "token id must fit vocab");
+    if ((size_t)R * n_steps > b.ring_elems) return fail(m, HIPDEC_ERR_ARG, "internal: token ring too small");
+    if ((rc = pf_ensure(m, R, true))) return rc;
+    PrefillWork &w = m->pf;
+    HCHK(hipStreamSynchronize(m->stream));                      // pinned staging is free again
+    memcpy(w.h_ids, tokens, (size_t)R * 4);
+    *b.h_bp = BatchParams{(int)(b.prefix + b.slot), (int)b.slot, (int)b.prefix, (int)top_k, sample_inv_temperature(temperature),
+                          softcap};
+    m->h_samp->ss = SampleParams{temperature, softcap, (int)top_k, 0, (int)(b.ring_elems / (size_t)R), 0u};
+    memcpy(m->h_samp->rng, rng_states, (size_t)R * sizeof(uint64_t));
+    HCHK(hipMemcpyAsync(w.ids, w.h_ids, (size_t)R * 4, hipMemcpyHostToDevice, m->stream));
+    HCHK(hipMemcpyAsync(b.d_bp, b.h_bp, sizeof(BatchParams), hipMemcpyHostToDevice, m->stream));
+    HCHK(hipMemcpyAsync(m->d_ss, &m->h_samp->ss, sizeof(SampleParams), hipMemcpyHostToDevice, m->stream));
+    HCHK(hipMemcpyAsync(m->d_rng, m->h_samp->rng, (size_t)R * sizeof(uint64_t), hipMemcpyHostToDevice, m->stream));
+    HCHK(hipEventRecord(m->ev0, m->stream));
+    for (size_t i = 0; i < n_steps; ++i)
+        if ((rc = batch_launch(m, variant))) return rc;
+    HCHK(hipEventRecord(m->ev1, m->stream));
+    HCHK(hipMemcpyAsync(b.h_ring, b.d_ring, (size_t)R * n_steps * 4, hipMemcpyDeviceToHost, m->stream));
+    HCHK(hipMemcpyAsync(m->h_samp->rng, m->d_rng, (size_t)R * sizeof(uint64_t), hipMemcpyDeviceToHost, m->stream));
+    HCHK(hipStreamSynchronize(m->stream));
+    HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+    memcpy(out_tokens, b.h_ring, (size_t)R * n_steps * 4);
+    memcpy(rng_states, m->h_samp->rng, (size_t)R * sizeof(uint64_t));
+    b.slot += n_steps;
+    b.have_logits = true;
+    return HIPDEC_OK;
+}
+
+// expf_as_host on the host over consecutive bit patterns, split over threads
+template <typename F> void expf_host_range(uint32_t first_bits, uint64_t count, int threads, F &&per_chunk) {
+    if (threads < 1) threads = 1;
+    if (threads > 64) threads = 64;
+    std::vector<std::thread> pool;
+    const uint64_t per = (count + (uint64_t)threads - 1) / (uint64_t)threads;
+    for (int t = 0; t < threads; ++t) {
+        const uint64_t lo = per * (uint64_t)t, hi = std::min<uint64_t>(count, lo + per);
+        if (lo >= hi) break;
+        pool.emplace_back([=, &per_chunk] { per_chunk(t, first_bits + (uint32_t)lo, hi - lo); });
+    }
+    for (auto &th : pool) th.join();
 }
 
 }  // namespace
@@ -757,6 +906,8 @@ void hipdec_destroy(hipdec_model *m) {
     if (m->pf.h_ids) (void)hipHostFree(m->pf.h_ids);
     if (m->bt.h_bp) (void)hipHostFree(m->bt.h_bp);
     if (m->bt.h_stage) (void)hipHostFree(m->bt.h_stage);
+    if (m->bt.h_ring) (void)hipHostFree(m->bt.h_ring);
+    if (m->h_samp) (void)hipHostFree(m->h_samp);
     if (m->ev0) (void)hipEventDestroy(m->ev0);
     if (m->ev1) (void)hipEventDestroy(m->ev1);
     if (m->ev_s0) (void)hipEventDestroy(m->ev_s0);
@@ -848,6 +999,10 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
     TRY(dalloc(m, &m->d_bmax, (size_t)m->blocks * 4));
     TRY(dalloc(m, &m->d_bsum, (size_t)m->blocks * 4));
     TRY(dalloc(m, &m->d_ring, S * 4));
+    TRY(dalloc(m, &m->d_ss, sizeof(SampleParams)));
+    HCHK(hipMemset(m->d_ss, 0, sizeof(SampleParams)));
+    TRY(dalloc(m, &m->d_rng, sizeof(uint64_t) * 32));
+    HCHK(hipHostMalloc((void **)&m->h_samp, sizeof(SampleHost), hipHostMallocDefault));
     // ---- persistent per-token kernel: exchange buffers, layer table, eligibility
     {
         const int G = m->num_cu;
@@ -1310,6 +1465,99 @@ int hipdec_decode_greedy_run(hipdec_model *m, uint32_t token, size_t n_steps, ui
     HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
     memcpy(out_tokens, m->h_out, n_steps * 4);
     m->len += n_steps;
+    return HIPDEC_OK;
+}
+
+int hipdec_decode_topk_sampled_run(hipdec_model *m, uint32_t token, uint32_t top_k, float temperature, float softcap,
+                                   uint64_t *rng_state, size_t n_steps, uint32_t *out_tokens) {
+    return sampled_run(m, V_TOPK_S, token, top_k, temperature, softcap, rng_state, n_steps, out_tokens);
+}
+
+int hipdec_decode_fullvocab_sampled_run(hipdec_model *m, uint32_t token, float temperature, float softcap,
+                                        uint64_t *rng_state, size_t n_steps, uint32_t *out_tokens) {
+    return sampled_run(m, V_STATS_S, token, 1, temperature, softcap, rng_state, n_steps, out_tokens);
+}
+
+int hipdec_decode_topk_sampled_run_batch(hipdec_model *m, const uint32_t *tokens, uint32_t top_k, float temperature,
+                                         float softcap, uint64_t *rng_states, size_t n_steps, uint32_t *out_tokens) {
+    return batch_sampled_run(m, B_TOPK_S, tokens, top_k, temperature, softcap, rng_states, n_steps, out_tokens);
+}
+
+int hipdec_decode_fullvocab_sampled_run_batch(hipdec_model *m, const uint32_t *tokens, float temperature, float softcap,
+                                              uint64_t *rng_states, size_t n_steps, uint32_t *out_tokens) {
+    return batch_sampled_run(m, B_STATS_S, tokens, 1, temperature, softcap, rng_states, n_steps, out_tokens);
+}
+
+int hipdec_debug_expf(const float *in, float *out, size_t n, int on_device) {
+    if (!in || !out) return HIPDEC_ERR_ARG;
+    if (!on_device) {
+        for (size_t i = 0; i < n; ++i) out[i] = expf_as_host(in[i]);
+        return HIPDEC_OK;
+    }
+    if (n == 0) return HIPDEC_OK;
+    float *d_in = nullptr, *d_out = nullptr;
+    hipError_t e = hipMalloc((void **)&d_in, n * 4);
+    if (e == hipSuccess) e = hipMalloc((void **)&d_out, n * 4);
+    if (e == hipSuccess) e = hipMemcpy(d_in, in, n * 4, hipMemcpyHostToDevice);
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(k_expf_eval, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, nullptr, d_in, d_out, n);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpy(out, d_out, n * 4, hipMemcpyDeviceToHost);
+    if (d_in) (void)hipFree(d_in);
+    if (d_out) (void)hipFree(d_out);
+    if (e != hipSuccess) { g_create_error = std::string("hipdec_debug_expf: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+    return HIPDEC_OK;
+}
+
+int hipdec_debug_expf_checksum(uint32_t first_bits, uint64_t count, int on_device, int host_threads, uint64_t *out) {
+    if (!out || count > (1ull << 32) || (uint64_t)first_bits + count > (1ull << 32)) return HIPDEC_ERR_ARG;
+    if (!on_device) {
+        uint64_t parts[64] = {};
+        expf_host_range(first_bits, count, host_threads, [&](int t, uint32_t lo, uint64_t n) {
+            uint64_t acc = 0;
+            for (uint64_t i = 0; i < n; ++i) acc += sample_exp_mix(lo + (uint32_t)i);
+            parts[t] = acc;
+        });
+        uint64_t total = 0;
+        for (uint64_t v : parts) total += v;
+        *out = total;
+        return HIPDEC_OK;
+    }
+    unsigned long long *d_acc = nullptr, h_acc = 0;
+    hipError_t e = hipMalloc((void **)&d_acc, 8);
+    if (e == hipSuccess) e = hipMemset(d_acc, 0, 8);
+    if (e == hipSuccess && count) {
+        hipLaunchKernelGGL(k_expf_checksum, dim3(4096), dim3(256), 0, nullptr, first_bits, count, d_acc);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpy(&h_acc, d_acc, 8, hipMemcpyDeviceToHost);
+    if (d_acc) (void)hipFree(d_acc);
+    if (e != hipSuccess) { g_create_error = std::string("hipdec_debug_expf_checksum: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+    *out = (uint64_t)h_acc;
+    return HIPDEC_OK;
+}
+
+int hipdec_debug_expf_count_mismatch(uint32_t first_bits, uint64_t count, int host_threads, uint64_t *out_mismatches) {
+    if (!out_mismatches || count > (1ull << 32) || (uint64_t)first_bits + count > (1ull << 32)) return HIPDEC_ERR_ARG;
+    uint64_t parts[64] = {};
+    expf_host_range(first_bits, count, host_threads, [&](int t, uint32_t lo, uint64_t n) {
+        uint64_t bad = 0;
+        for (uint64_t i = 0; i < n; ++i) {
+            const uint32_t bits = lo + (uint32_t)i;
+            float x;
+            memcpy(&x, &bits, 4);
+            const float a = expf(x), b = expf_as_host(x);
+            uint32_t ab, bb;
+            memcpy(&ab, &a, 4);
+            memcpy(&bb, &b, 4);
+            if (ab != bb && !(a != a && b != b)) ++bad;           // any two NaNs agree
+        }
+        parts[t] = bad;
+    });
+    uint64_t total = 0;
+    for (uint64_t v : parts) total += v;
+    *out_mismatches = total;
     return HIPDEC_OK;
 }
 

@@ -29,6 +29,9 @@ EXPORTS = [
     "hipdec_batch_begin", "hipdec_batch_end", "hipdec_batch_steps", "hipdec_decode_logits_from_ids_batch",
     "hipdec_decode_token_argmax_from_ids_batch", "hipdec_decode_token_topk_from_ids_batch",
     "hipdec_decode_token_block_stats_from_ids_batch", "hipdec_materialize_current_logits_block_batch",
+    "hipdec_decode_topk_sampled_run", "hipdec_decode_fullvocab_sampled_run", "hipdec_decode_topk_sampled_run_batch",
+    "hipdec_decode_fullvocab_sampled_run_batch", "hipdec_debug_expf", "hipdec_debug_expf_checksum",
+    "hipdec_debug_expf_count_mismatch",
 ]
 
 
@@ -132,9 +135,48 @@ def load_library(path=None):
                                                                    C.c_size_t, szp]
     lib.hipdec_materialize_current_logits_block_batch.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_float, fp,
                                                                   C.c_size_t, szp]
+    u64p = C.POINTER(C.c_uint64)
+    lib.hipdec_decode_topk_sampled_run.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.c_float, C.c_float, u64p,
+                                                   C.c_size_t, u32p]
+    lib.hipdec_decode_fullvocab_sampled_run.argtypes = [C.c_void_p, C.c_uint32, C.c_float, C.c_float, u64p, C.c_size_t,
+                                                        u32p]
+    lib.hipdec_decode_topk_sampled_run_batch.argtypes = [C.c_void_p, u32p, C.c_uint32, C.c_float, C.c_float, u64p,
+                                                         C.c_size_t, u32p]
+    lib.hipdec_decode_fullvocab_sampled_run_batch.argtypes = [C.c_void_p, u32p, C.c_float, C.c_float, u64p, C.c_size_t,
+                                                              u32p]
+    lib.hipdec_debug_expf.argtypes = [fp, fp, C.c_size_t, C.c_int]
+    lib.hipdec_debug_expf_checksum.argtypes = [C.c_uint32, C.c_uint64, C.c_int, C.c_int, u64p]
+    lib.hipdec_debug_expf_count_mismatch.argtypes = [C.c_uint32, C.c_uint64, C.c_int, u64p]
     if path is None:
         _LIB = lib
     return lib
+
+
+def debug_expf(x, on_device=False):
+    """The sampler's exponential (the host C library's expf restated) on the host or on the GPU."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    rc = load_library().hipdec_debug_expf(_fptr(x), _fptr(out), x.size, 1 if on_device else 0)
+    if rc != OK:
+        raise HipDecodeError(rc, "hipdec_debug_expf failed")
+    return out
+
+
+def debug_expf_checksum(first_bits, count, on_device=False, host_threads=8):
+    out = C.c_uint64()
+    rc = load_library().hipdec_debug_expf_checksum(first_bits, count, 1 if on_device else 0, host_threads, C.byref(out))
+    if rc != OK:
+        raise HipDecodeError(rc, "hipdec_debug_expf_checksum failed")
+    return out.value
+
+
+def debug_expf_count_mismatch(first_bits, count, host_threads=8):
+    """How many of `count` consecutive float bit patterns give a result different from libm's expf."""
+    out = C.c_uint64()
+    rc = load_library().hipdec_debug_expf_count_mismatch(first_bits, count, host_threads, C.byref(out))
+    if rc != OK:
+        raise HipDecodeError(rc, "hipdec_debug_expf_count_mismatch failed")
+    return out.value
 
 
 def calibration_copy(nbytes, reps=1):
@@ -279,6 +321,43 @@ class HipDecodeModel:
         self._chk(self._lib.hipdec_decode_greedy_run(self._h, token, n_steps,
                                                      out.ctypes.data_as(C.POINTER(C.c_uint32))))
         return out[:n_steps]
+
+    # ---- sampled runs with the draw on the device; return (tokens, new rng state)
+    def decode_topk_sampled_run(self, token, top_k, temperature, rng_state, n_steps, softcap=0.0):
+        out = np.empty(max(n_steps, 1), np.uint32)
+        st = C.c_uint64(int(rng_state) & 0xFFFFFFFFFFFFFFFF)
+        self._chk(self._lib.hipdec_decode_topk_sampled_run(self._h, token, top_k, temperature, softcap, C.byref(st),
+                                                           n_steps, out.ctypes.data_as(C.POINTER(C.c_uint32))))
+        return out[:n_steps], st.value
+
+    def decode_fullvocab_sampled_run(self, token, temperature, rng_state, n_steps, softcap=0.0):
+        out = np.empty(max(n_steps, 1), np.uint32)
+        st = C.c_uint64(int(rng_state) & 0xFFFFFFFFFFFFFFFF)
+        self._chk(self._lib.hipdec_decode_fullvocab_sampled_run(self._h, token, temperature, softcap, C.byref(st),
+                                                                n_steps, out.ctypes.data_as(C.POINTER(C.c_uint32))))
+        return out[:n_steps], st.value
+
+    def decode_topk_sampled_run_batch(self, tokens, top_k, temperature, rng_states, n_steps, softcap=0.0):
+        t = self._toks(tokens)
+        st = np.ascontiguousarray(rng_states, dtype=np.uint64).copy()
+        if st.size != self._rows:
+            raise ValueError("expected %d rng states, got %d" % (self._rows, st.size))
+        out = np.empty((max(n_steps, 1), self._rows), np.uint32)
+        self._chk(self._lib.hipdec_decode_topk_sampled_run_batch(
+            self._h, t.ctypes.data_as(C.POINTER(C.c_uint32)), top_k, temperature, softcap,
+            st.ctypes.data_as(C.POINTER(C.c_uint64)), n_steps, out.ctypes.data_as(C.POINTER(C.c_uint32))))
+        return out[:n_steps], st
+
+    def decode_fullvocab_sampled_run_batch(self, tokens, temperature, rng_states, n_steps, softcap=0.0):
+        t = self._toks(tokens)
+        st = np.ascontiguousarray(rng_states, dtype=np.uint64).copy()
+        if st.size != self._rows:
+            raise ValueError("expected %d rng states, got %d" % (self._rows, st.size))
+        out = np.empty((max(n_steps, 1), self._rows), np.uint32)
+        self._chk(self._lib.hipdec_decode_fullvocab_sampled_run_batch(
+            self._h, t.ctypes.data_as(C.POINTER(C.c_uint32)), temperature, softcap,
+            st.ctypes.data_as(C.POINTER(C.c_uint64)), n_steps, out.ctypes.data_as(C.POINTER(C.c_uint32))))
+        return out[:n_steps], st
 
     # ---- multi-sample decode: rows share positions [0, len) and step together
     def batch_begin(self, n_rows):

@@ -1,0 +1,239 @@
+"""The sampled token loops with the draw on the device (hipdec_decode_*_sampled_run*): the merge of
+engine/src/decode.rs:218-253 and the draws of engine/src/inference.rs:823-921 done on the GPU must
+give, token for token and with the same final RNG state, what the reference's loop gives when it
+reads the candidates / block statistics back and draws on the host (inference.rs:586-625).
+
+The draw needs exp() with the host C library's bits.  The restatement the kernels use is checked
+here (a) on the host against libm's expf for EVERY float <= 0 (the sampler's arguments are
+differences to a maximum, so never positive) and for 0..89, (b) against float64 exp, and (c) on the
+GPU against the host evaluation through checksums over the same ranges."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from rustane_amd import engine as E
+from rustane_amd import hipdec, synth
+from rustane_amd.hipdec import Config, HipDecodeModel, KvDtype, WeightDtype
+
+NEG_FIRST, NEG_COUNT = 0x80000000, 0xFF800000 - 0x80000000 + 1      # -0.0 .. -inf
+POS_FIRST, POS_COUNT = 0x00000000, 0x42B20000 + 1                   # +0.0 .. 89.0
+
+
+# ------------------------------------------------------------------ the exponential (CPU)
+def test_restated_expf_equals_libm_for_every_non_positive_float():
+    assert hipdec.debug_expf_count_mismatch(NEG_FIRST, NEG_COUNT, host_threads=8) == 0
+    assert hipdec.debug_expf_count_mismatch(POS_FIRST, POS_COUNT, host_threads=8) == 0
+
+
+def test_restated_expf_known_answers_and_float64_reference():
+    x = np.array([0.0, -0.0, -np.inf, np.inf, -104.0, -200.0, 89.0, 1.0, -1.0], np.float32)
+    y = hipdec.debug_expf(x)
+    assert y[0] == 1.0 and y[1] == 1.0 and y[2] == 0.0 and np.isinf(y[3]) and y[4] == 0.0 and y[5] == 0.0
+    assert np.isinf(y[6])                                            # exp(89) overflows float
+    assert y[7] == np.float32(np.e) and y[8] == np.float32(1.0 / np.e)
+    assert np.isnan(hipdec.debug_expf(np.array([np.nan], np.float32))[0])
+    rng = np.random.default_rng(5)
+    x = np.concatenate([-rng.random(200000) * 104.0, rng.random(50000) * 88.0, -rng.random(50000) * 1e-3]).astype(np.float32)
+    y = hipdec.debug_expf(x)
+    want = np.exp(x.astype(np.float64))
+    # the C library documents 0.502 units in the last place for this algorithm
+    ulp = np.maximum(np.spacing(want.astype(np.float32)).astype(np.float64), 2.0 ** -149)
+    assert np.all(np.abs(y.astype(np.float64) - want) <= 0.503 * ulp)
+    # subnormal results are produced, not flushed
+    assert hipdec.debug_expf(np.array([-100.0], np.float32))[0] == np.float32(np.exp(-100.0))
+
+
+# ------------------------------------------------------------------ the exponential (GPU)
+@pytest.mark.gpu
+def test_device_expf_equals_host_expf_for_every_non_positive_float():
+    for first, count in ((NEG_FIRST, NEG_COUNT), (POS_FIRST, POS_COUNT)):
+        host = hipdec.debug_expf_checksum(first, count, on_device=False, host_threads=16)
+        dev = hipdec.debug_expf_checksum(first, count, on_device=True)
+        assert host == dev, (hex(first), hex(host), hex(dev))
+    # element-wise on a sample, subnormal results and the special values included
+    rng = np.random.default_rng(9)
+    x = np.concatenate([-rng.random(100000) * 104.0, np.array([0.0, -0.0, -np.inf, -87.5, -88.0, -95.0, -103.9, -104.5])])
+    x = x.astype(np.float32)
+    np.testing.assert_array_equal(hipdec.debug_expf(x, on_device=True).view(np.uint32), hipdec.debug_expf(x).view(np.uint32))
+
+
+# ------------------------------------------------------------------ runs against the host loop
+def small_cfg(vocab=1000, seq=96):
+    return Config.make(dim=256, hidden=640, heads=2, hd=128, seq=seq, nlayers=2, vocab=vocab)
+
+
+def two_models(cfg, w, wd, kv, prompt):
+    a = HipDecodeModel(cfg, w, weight_dtype=wd, kv_dtype=kv)
+    b = HipDecodeModel(cfg, w, weight_dtype=wd, kv_dtype=kv)
+    la = a.prefill(np.array(prompt, np.uint32))
+    lb = b.prefill(np.array(prompt, np.uint32))
+    np.testing.assert_array_equal(la, lb)
+    return a, b, la
+
+
+def host_topk_loop(dev, tok, k, T, seed, steps):
+    """inference.rs:586-599 with the oracle's merge and draw over the device's candidates."""
+    rng = O.Rng(seed)
+    out = []
+    for _ in range(steps):
+        vals, idxs = dev.decode_token_topk_from_id(tok, k)
+        mv, mi = O.merge_topk(vals, idxs, k)
+        tok = int(O.lib().orc_sample_topk_candidates(O.PU(mi), O.P(mv), mi.size, T, rng.ref))
+        out.append(tok)
+    return np.array(out, np.uint32), rng.s.value
+
+
+def host_fullvocab_loop(dev, tok, T, softcap, seed, steps):
+    """inference.rs:600-625 with the oracle's two draws over the device's statistics and block logits."""
+    rng = O.Rng(seed)
+    inv_t = np.float32(1.0) / max(np.float32(T), np.finfo(np.float32).tiny)
+    out = []
+    for _ in range(steps):
+        mx, sm = dev.decode_token_block_stats_from_id(tok, float(inv_t), softcap)
+        blk = int(O.lib().orc_sample_block_from_stats(O.P(mx), O.P(sm), mx.size, rng.ref))
+        bl = dev.materialize_current_logits_block(blk, softcap)
+        tok = int(O.lib().orc_sample_block_logits(blk * 256, O.P(bl), bl.size, T, rng.ref))
+        out.append(tok)
+    return np.array(out, np.uint32), rng.s.value
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("wd,kv,vocab,k,T", [
+    (WeightDtype.BF16, KvDtype.BF16, 1000, 8, 0.8),      # last block holds 232 rows
+    (WeightDtype.F32, KvDtype.F32, 8192, 4, 1.3),
+    (WeightDtype.FP8_E4M3, KvDtype.BF16, 320, 32, 0.5),  # k > rows of the last block (64): padded lists
+    (WeightDtype.BF16, KvDtype.F32, 1000, 1, 0.8),       # one candidate: no draw, the state stays
+    (WeightDtype.BF16, KvDtype.F32, 1000, 5, 0.0),       # temperature 0: first candidate, no draw
+])
+def test_topk_run_on_device_equals_host_loop(wd, kv, vocab, k, T):
+    cfg = small_cfg(vocab)
+    w = synth.make_weights(cfg, seed=13, std=0.08, round_bf16=True)
+    a, b, lg = two_models(cfg, w, wd, kv, [3, 1, 4, 1, 5, 9, 2, 6])
+    first = int(np.argmax(lg))
+    steps, seed = 40, 0x1234567
+    got, state = a.decode_topk_sampled_run(first, k, T, seed, steps)
+    want, want_state = host_topk_loop(b, first, k, T, seed, steps)
+    np.testing.assert_array_equal(got, want)
+    assert state == want_state
+    assert a.len() == b.len() == 8 + steps
+    # a second run continues from where the first stopped, with the advanced state
+    got2, state2 = a.decode_topk_sampled_run(int(got[-1]), k, T, state, 7)
+    want2, want_state2 = host_topk_loop(b, int(want[-1]), k, T, want_state, 7)
+    np.testing.assert_array_equal(got2, want2)
+    assert state2 == want_state2
+    if k > 1 and T > 0:
+        assert state != seed and len(set(got.tolist())) > 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("wd,kv,vocab,T,softcap", [
+    (WeightDtype.BF16, KvDtype.BF16, 1000, 1.0, 0.0),
+    (WeightDtype.F32, KvDtype.F32, 8192, 0.7, 0.0),
+    (WeightDtype.BF16, KvDtype.F32, 320, 1.5, 2.5),      # softcap on the statistics and on the block
+    (WeightDtype.INT4_G128, KvDtype.BF16, 1000, 1.0, 0.0),
+])
+def test_fullvocab_run_on_device_equals_host_loop(wd, kv, vocab, T, softcap):
+    cfg = small_cfg(vocab)
+    w = synth.make_weights(cfg, seed=17, std=0.08, round_bf16=True)
+    a, b, lg = two_models(cfg, w, wd, kv, [2, 7, 1, 8, 2, 8, 1, 8])
+    first = int(np.argmax(lg))
+    steps, seed = 40, 99
+    got, state = a.decode_fullvocab_sampled_run(first, T, seed, steps, softcap=softcap)
+    want, want_state = host_fullvocab_loop(b, first, T, softcap, seed, steps)
+    np.testing.assert_array_equal(got, want)
+    assert state == want_state
+    assert len(set(got.tolist())) > 4                     # two draws per token took place
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("k,T,softcap", [(8, 0.8, 0.0), (0, 1.0, 0.0), (0, 0.9, 3.0)])
+def test_batched_run_on_device_equals_per_step_batch_calls(k, T, softcap):
+    cfg = small_cfg(1000)
+    w = synth.make_weights(cfg, seed=19, std=0.08, round_bf16=True)
+    a, b, lg = two_models(cfg, w, WeightDtype.BF16, KvDtype.BF16, [5, 6, 7, 8, 9, 10, 11, 12, 13])
+    R, steps = 5, 24
+    first = np.argsort(lg)[::-1][:R].astype(np.uint32)    # rows start from different tokens
+    seeds = np.arange(R, dtype=np.uint64) + np.uint64(21)
+    a.batch_begin(R)
+    b.batch_begin(R)
+    if k > 0:
+        got, states = a.decode_topk_sampled_run_batch(first, k, T, seeds, steps)
+    else:
+        got, states = a.decode_fullvocab_sampled_run_batch(first, T, seeds, steps, softcap=softcap)
+    rngs = [O.Rng(int(s)) for s in seeds]
+    cur = first.copy()
+    inv_t = float(np.float32(1.0) / np.float32(T))
+    for i in range(steps):
+        nxt = np.empty(R, np.uint32)
+        if k > 0:
+            vals, idxs = b.decode_token_topk_from_ids_batch(cur, k)
+            for r in range(R):
+                mv, mi = O.merge_topk(vals[r], idxs[r], k)
+                nxt[r] = O.lib().orc_sample_topk_candidates(O.PU(mi), O.P(mv), mi.size, T, rngs[r].ref)
+        else:
+            mx, sm = b.decode_token_block_stats_from_ids_batch(cur, inv_t, softcap)
+            for r in range(R):
+                mxr, smr = np.ascontiguousarray(mx[r]), np.ascontiguousarray(sm[r])
+                blk = int(O.lib().orc_sample_block_from_stats(O.P(mxr), O.P(smr), mxr.size, rngs[r].ref))
+                bl = b.materialize_current_logits_block_batch(r, blk, softcap)
+                nxt[r] = O.lib().orc_sample_block_logits(blk * 256, O.P(bl), bl.size, T, rngs[r].ref)
+        np.testing.assert_array_equal(got[i], nxt, err_msg="step %d" % i)
+        cur = nxt
+    np.testing.assert_array_equal(states, np.array([r.s.value for r in rngs], np.uint64))
+    assert a.batch_steps() == b.batch_steps() == steps
+    # the per-step calls continue an open batch after a run
+    np.testing.assert_array_equal(a.decode_token_argmax_from_ids_batch(cur), b.decode_token_argmax_from_ids_batch(cur))
+    a.batch_end()
+    b.batch_end()
+
+
+@pytest.mark.gpu
+def test_run_argument_errors_and_unsupported_softcap():
+    cfg = small_cfg(1000, seq=32)
+    w = synth.make_weights(cfg, seed=13, std=0.08, round_bf16=True)
+    m = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.F32)
+    m.prefill(np.array([1, 2, 3, 4], np.uint32))
+    with pytest.raises(hipdec.HipDecodeError) as e:
+        m.decode_topk_sampled_run(1, 8, 0.8, 1, 4, softcap=3.0)     # the host applies tanhf to the candidates
+    assert e.value.status == hipdec.ERR_UNSUPPORTED
+    for bad_k in (0, 33):
+        with pytest.raises(hipdec.HipDecodeError) as e:
+            m.decode_topk_sampled_run(1, bad_k, 0.8, 1, 4)
+        assert e.value.status == hipdec.ERR_ARG
+    with pytest.raises(hipdec.HipDecodeError) as e:
+        m.decode_fullvocab_sampled_run(1, 0.0, 1, 4)
+    assert e.value.status == hipdec.ERR_ARG
+    with pytest.raises(hipdec.HipDecodeError) as e:
+        m.decode_topk_sampled_run(1, 8, 0.8, 1, 29)                 # 4 + 29 > seq
+    assert e.value.status == hipdec.ERR_FULL
+    with pytest.raises(hipdec.HipDecodeError) as e:
+        m.decode_topk_sampled_run(5000, 8, 0.8, 1, 2)
+    assert e.value.status == hipdec.ERR_ARG
+    assert m.len() == 4                                             # nothing ran
+    toks, st = m.decode_topk_sampled_run(1, 8, 0.8, 1, 0)           # zero steps: no-op
+    assert toks.size == 0 and st == 1 and m.len() == 4
+    toks, _ = m.decode_topk_sampled_run(1, 8, 0.8, 1, 28)           # exactly to the end of the cache
+    assert toks.size == 28 and m.len() == 32
+
+
+# ------------------------------------------------------------------ the session picks the device runs
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,k,softcap,samples", [(0.8, 8, 0.0, 1), (1.0, 0, 0.0, 1), (1.0, 0, 2.5, 1), (0.8, 8, 0.0, 4),
+                                                 (1.0, 0, 0.0, 3), (0.8, 4, 3.0, 2)])
+def test_session_streams_are_the_same_with_device_and_host_draws(T, k, softcap, samples):
+    cfg = small_cfg(1000, seq=64)
+    prompt = [5, 6, 7, 8, 9, 10, 11, 12, 13]
+    w = synth.make_weights(cfg, seed=31, std=0.08, round_bf16=True)
+    req = E.GenerationRequest(E.DecodeBackendRequest.HIP, steps=30, temperature=T, top_k=k, samples=samples, seed=21)
+    dev = E.InferenceSession(cfg, w, prompt, softcap=softcap, weight_dtype=1).generate(req)
+    host = E.InferenceSession(cfg, w, prompt, softcap=softcap, weight_dtype=1, flags=0x200).generate(req)
+    assert len(dev.results) == len(host.results) == samples
+    for a, b in zip(dev.results, host.results):
+        np.testing.assert_array_equal(a.sampled, b.sampled)
+        np.testing.assert_array_equal(a.generated, b.generated)
+        assert a.seed == b.seed
+    # a second request on the same session repeats the streams (prompt cache intact, RNG re-seeded)
+    s = E.InferenceSession(cfg, w, prompt, softcap=softcap, weight_dtype=1)
+    r1, r2 = s.generate(req), s.generate(req)
+    for a, b in zip(r1.results, r2.results):
+        np.testing.assert_array_equal(a.sampled, b.sampled)
