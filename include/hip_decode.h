@@ -180,9 +180,9 @@ int hipdec_decode_greedy_run(hipdec_model *m, uint32_t token, size_t n_steps, ui
  * read at entry and advanced exactly as the host loop would advance it.  Equivalent to n_steps
  * rounds of hipdec_decode_token_topk_from_id + host merge + host draw (resp.
  * hipdec_decode_token_block_stats_from_id + block draw + hipdec_materialize_current_logits_block +
- * token draw).  The top-k form returns HIPDEC_ERR_UNSUPPORTED with softcap > 0 (the host applies
- * tanhf to the merged candidates; that function is not reproduced on the device): use the per-step
- * calls then.  Needs vocab <= 262144. */
+ * token draw); with softcap > 0 the top-k form applies cap * tanhf(v / cap) to the merged candidates
+ * as the host does (decode.rs:155-159), the host C library's tanhf reproduced bit for bit as well.
+ * Needs vocab <= 262144 (HIPDEC_ERR_UNSUPPORTED otherwise). */
 int hipdec_decode_topk_sampled_run(hipdec_model *m, uint32_t token, uint32_t top_k, float temperature, float softcap,
                                    uint64_t *rng_state, size_t n_steps, uint32_t *out_tokens);
 int hipdec_decode_fullvocab_sampled_run(hipdec_model *m, uint32_t token, float temperature, float softcap,
@@ -217,15 +217,17 @@ int hipdec_debug_step_profile(hipdec_model *m, uint32_t token, uint64_t *out, si
  * the known-size yardstick that hardware memory-traffic counters are scaled by. */
 int hipdec_debug_calibration_copy(size_t bytes, int reps);
 
-/* Verification of the exponential the on-device sampler uses (a restatement of the host C library's
- * expf): evaluate it for n inputs on the host (on_device = 0) or on the GPU; */
-int hipdec_debug_expf(const float *in, float *out, size_t n, int on_device);
+/* Verification of the two host C library functions the on-device sampler restates (fn 0: expf,
+ * fn 1: tanhf): evaluate the restatement for n inputs on the host (on_device = 0) or on the GPU; */
+int hipdec_debug_hostmath_eval(int fn, const float *in, float *out, size_t n, int on_device);
 /* an order-independent checksum of its results over `count` consecutive float bit patterns starting
  * at first_bits, computed on the host (with host_threads threads) or on the GPU: equal checksums
  * mean equal results; */
-int hipdec_debug_expf_checksum(uint32_t first_bits, uint64_t count, int on_device, int host_threads, uint64_t *out);
-/* and the number of those inputs for which the host evaluation differs from the C library's expf. */
-int hipdec_debug_expf_count_mismatch(uint32_t first_bits, uint64_t count, int host_threads, uint64_t *out_mismatches);
+int hipdec_debug_hostmath_checksum(int fn, uint32_t first_bits, uint64_t count, int on_device, int host_threads,
+                                   uint64_t *out);
+/* and the number of those inputs for which the host evaluation differs from the C library's function. */
+int hipdec_debug_hostmath_count_mismatch(int fn, uint32_t first_bits, uint64_t count, int host_threads,
+                                         uint64_t *out_mismatches);
 
 #ifdef __cplusplus
 }

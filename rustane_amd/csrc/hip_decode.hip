@@ -793,10 +793,9 @@ int sampled_args_ok(hipdec_model *m, bool topk, uint32_t top_k, float temperatur
                     const uint32_t *out_tokens) {
     if (!rng || !out_tokens) return fail(m, HIPDEC_ERR_ARG, "null buffer");
     if (m->blocks > SAMPLE_MAX_BLOCKS) return fail(m, HIPDEC_ERR_UNSUPPORTED, "on-device sampling serves up to 1024 vocab blocks");
+    (void)softcap;
     if (topk) {
         if (top_k == 0 || top_k > HIPDEC_MAX_GPU_TOPK) return fail(m, HIPDEC_ERR_ARG, "gpu top-k only supports k in 1..32");
-        if (softcap > 0.0f)
-            return fail(m, HIPDEC_ERR_UNSUPPORTED, "on-device top-k sampling does not reproduce the host's tanh: use the per-step calls with a softcap");
     } else if (!(temperature > 0.0f)) {
         return fail(m, HIPDEC_ERR_ARG, "full-vocab sampling needs a positive temperature");
     }
@@ -875,8 +874,8 @@ int batch_sampled_run(hipdec_model *m, int variant, const uint32_t *tokens, uint
     return HIPDEC_OK;
 }
 
-// expf_as_host on the host over consecutive bit patterns, split over threads
-template <typename F> void expf_host_range(uint32_t first_bits, uint64_t count, int threads, F &&per_chunk) {
+// a restated host function over consecutive bit patterns on the host, split over threads
+template <typename F> void hostmath_host_range(uint32_t first_bits, uint64_t count, int threads, F &&per_chunk) {
     if (threads < 1) threads = 1;
     if (threads > 64) threads = 64;
     std::vector<std::thread> pool;
@@ -1488,10 +1487,10 @@ int hipdec_decode_fullvocab_sampled_run_batch(hipdec_model *m, const uint32_t *t
     return batch_sampled_run(m, B_STATS_S, tokens, 1, temperature, softcap, rng_states, n_steps, out_tokens);
 }
 
-int hipdec_debug_expf(const float *in, float *out, size_t n, int on_device) {
-    if (!in || !out) return HIPDEC_ERR_ARG;
+int hipdec_debug_hostmath_eval(int fn, const float *in, float *out, size_t n, int on_device) {
+    if (!in || !out || (fn != HOSTMATH_EXPF && fn != HOSTMATH_TANHF)) return HIPDEC_ERR_ARG;
     if (!on_device) {
-        for (size_t i = 0; i < n; ++i) out[i] = expf_as_host(in[i]);
+        for (size_t i = 0; i < n; ++i) out[i] = hostmath_eval(fn, in[i]);
         return HIPDEC_OK;
     }
     if (n == 0) return HIPDEC_OK;
@@ -1500,23 +1499,25 @@ int hipdec_debug_expf(const float *in, float *out, size_t n, int on_device) {
     if (e == hipSuccess) e = hipMalloc((void **)&d_out, n * 4);
     if (e == hipSuccess) e = hipMemcpy(d_in, in, n * 4, hipMemcpyHostToDevice);
     if (e == hipSuccess) {
-        hipLaunchKernelGGL(k_expf_eval, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, nullptr, d_in, d_out, n);
+        hipLaunchKernelGGL(k_hostmath_eval, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, nullptr, fn, d_in, d_out, n);
         e = hipGetLastError();
     }
     if (e == hipSuccess) e = hipMemcpy(out, d_out, n * 4, hipMemcpyDeviceToHost);
     if (d_in) (void)hipFree(d_in);
     if (d_out) (void)hipFree(d_out);
-    if (e != hipSuccess) { g_create_error = std::string("hipdec_debug_expf: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+    if (e != hipSuccess) { g_create_error = std::string("hipdec_debug_hostmath_eval: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
     return HIPDEC_OK;
 }
 
-int hipdec_debug_expf_checksum(uint32_t first_bits, uint64_t count, int on_device, int host_threads, uint64_t *out) {
+int hipdec_debug_hostmath_checksum(int fn, uint32_t first_bits, uint64_t count, int on_device, int host_threads,
+                                   uint64_t *out) {
     if (!out || count > (1ull << 32) || (uint64_t)first_bits + count > (1ull << 32)) return HIPDEC_ERR_ARG;
+    if (fn != HOSTMATH_EXPF && fn != HOSTMATH_TANHF) return HIPDEC_ERR_ARG;
     if (!on_device) {
         uint64_t parts[64] = {};
-        expf_host_range(first_bits, count, host_threads, [&](int t, uint32_t lo, uint64_t n) {
+        hostmath_host_range(first_bits, count, host_threads, [&](int t, uint32_t lo, uint64_t n) {
             uint64_t acc = 0;
-            for (uint64_t i = 0; i < n; ++i) acc += sample_exp_mix(lo + (uint32_t)i);
+            for (uint64_t i = 0; i < n; ++i) acc += hostmath_mix(fn, lo + (uint32_t)i);
             parts[t] = acc;
         });
         uint64_t total = 0;
@@ -1528,26 +1529,28 @@ int hipdec_debug_expf_checksum(uint32_t first_bits, uint64_t count, int on_devic
     hipError_t e = hipMalloc((void **)&d_acc, 8);
     if (e == hipSuccess) e = hipMemset(d_acc, 0, 8);
     if (e == hipSuccess && count) {
-        hipLaunchKernelGGL(k_expf_checksum, dim3(4096), dim3(256), 0, nullptr, first_bits, count, d_acc);
+        hipLaunchKernelGGL(k_hostmath_checksum, dim3(4096), dim3(256), 0, nullptr, fn, first_bits, count, d_acc);
         e = hipGetLastError();
     }
     if (e == hipSuccess) e = hipMemcpy(&h_acc, d_acc, 8, hipMemcpyDeviceToHost);
     if (d_acc) (void)hipFree(d_acc);
-    if (e != hipSuccess) { g_create_error = std::string("hipdec_debug_expf_checksum: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+    if (e != hipSuccess) { g_create_error = std::string("hipdec_debug_hostmath_checksum: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
     *out = (uint64_t)h_acc;
     return HIPDEC_OK;
 }
 
-int hipdec_debug_expf_count_mismatch(uint32_t first_bits, uint64_t count, int host_threads, uint64_t *out_mismatches) {
+int hipdec_debug_hostmath_count_mismatch(int fn, uint32_t first_bits, uint64_t count, int host_threads,
+                                         uint64_t *out_mismatches) {
     if (!out_mismatches || count > (1ull << 32) || (uint64_t)first_bits + count > (1ull << 32)) return HIPDEC_ERR_ARG;
+    if (fn != HOSTMATH_EXPF && fn != HOSTMATH_TANHF) return HIPDEC_ERR_ARG;
     uint64_t parts[64] = {};
-    expf_host_range(first_bits, count, host_threads, [&](int t, uint32_t lo, uint64_t n) {
+    hostmath_host_range(first_bits, count, host_threads, [&](int t, uint32_t lo, uint64_t n) {
         uint64_t bad = 0;
         for (uint64_t i = 0; i < n; ++i) {
             const uint32_t bits = lo + (uint32_t)i;
             float x;
             memcpy(&x, &bits, 4);
-            const float a = expf(x), b = expf_as_host(x);
+            const float a = fn == HOSTMATH_TANHF ? tanhf(x) : expf(x), b = hostmath_eval(fn, x);
             uint32_t ab, bb;
             memcpy(&ab, &a, 4);
             memcpy(&bb, &b, 4);

@@ -12,8 +12,10 @@
 //   block draw from statistics engine/src/inference.rs:851-891
 //   draw inside the block      engine/src/inference.rs:893-921 (+ block_idx * 256, :613)
 //   uniform numbers            engine/src/inference.rs:759-768 (64-bit LCG, top 24 bits)
+//   softcap of the candidates  engine/src/decode.rs:155-159 (cap * tanhf(v / cap) on the host)
 // Sums run sequentially in one thread in the host's order; every float operation is written with
-// a single-rounding intrinsic so that the compiler cannot fuse a multiply into an add.
+// a single-rounding intrinsic (or compiled with contraction off) so that the compiler cannot fuse
+// a multiply into an add.
 #pragma once
 #include "hipdec_batch.h"
 #include "hipdec_kernels.h"
@@ -68,29 +70,136 @@ __host__ __device__ inline float expf_as_host(float x) {
     return (float)y;
 }
 
-// order-sensitive checksum of expf_as_host over `count` consecutive float bit patterns
-__host__ __device__ __forceinline__ uint64_t sample_exp_mix(uint32_t in_bits) {
-    const uint32_t out = __builtin_bit_cast(uint32_t, expf_as_host(__builtin_bit_cast(float, in_bits)));
+// ---------------------------------------------------------------- tanhf with the host's bits
+// The GNU C library's float tanh (through glibc 2.40) is the classic single-precision routine:
+// tanh(x) = 1 - 2/(expm1(2|x|) + 2) for |x| >= 1, -t/(t + 2) with t = expm1(-2|x|) below, x(1 + x)
+// for tiny x and 1 - 1e-30 from 22 up, on top of the single-precision expm1 (argument reduction by
+// ln2 in two pieces, a degree-5 polynomial in x^2/2, reconstruction by exponent arithmetic).  It is
+// plain float arithmetic with no fused operations, which is how both functions are written here;
+// the tests compare them with the C library for all 2^32 floats on the host and the device
+// against the host through checksums.
+__host__ __device__ inline float expm1f_as_host(float x) {
+#pragma clang fp contract(off)
+    const float one = 1.0f, huge = 1.0e+30f, tiny = 1.0e-30f, o_threshold = 8.8721679688e+01f,
+                ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f, invln2 = 1.4426950216e+00f,
+                q1 = -3.3333335072e-02f, q2 = 1.5873016091e-03f, q3 = -7.9365076090e-05f, q4 = 4.0082177293e-06f,
+                q5 = -2.0109921195e-07f;
+    float y, hi, lo, c = 0.0f, t, e;
+    int k;
+    uint32_t hx = __builtin_bit_cast(uint32_t, x);
+    const bool neg = (hx & 0x80000000u) != 0;
+    hx &= 0x7fffffffu;
+    if (hx >= 0x4195b844u) {                                     // |x| >= 27 ln2
+        if (hx >= 0x42b17218u) {                                 // |x| >= 88.72...
+            if (hx > 0x7f800000u) return x + x;
+            if (hx == 0x7f800000u) return neg ? -1.0f : x;
+            if (x > o_threshold) return huge * huge;
+        }
+        if (neg && x + tiny < 0.0f) return tiny - one;
+    }
+    if (hx > 0x3eb17218u) {                                      // |x| > 0.5 ln2
+        if (hx < 0x3f851592u) {                                  // and < 1.5 ln2
+            if (!neg) { hi = x - ln2_hi; lo = ln2_lo; k = 1; }
+            else { hi = x + ln2_hi; lo = -ln2_lo; k = -1; }
+        } else {
+            k = (int)(invln2 * x + (neg ? -0.5f : 0.5f));
+            t = (float)k;
+            hi = x - t * ln2_hi;
+            lo = t * ln2_lo;
+        }
+        x = hi - lo;
+        c = (hi - x) - lo;
+    } else if (hx < 0x33000000u) {                               // |x| < 2^-25
+        return x;
+    } else {
+        k = 0;
+    }
+    const float hfx = 0.5f * x;
+    const float hxs = x * hfx;
+    const float r1 = one + hxs * (q1 + hxs * (q2 + hxs * (q3 + hxs * (q4 + hxs * q5))));
+    t = 3.0f - r1 * hfx;
+    e = hxs * ((r1 - t) / (6.0f - x * t));
+    if (k == 0) return x - (x * e - hxs);
+    e = x * (e - c) - c;
+    e -= hxs;
+    if (k == -1) return 0.5f * (x - e) - 0.5f;
+    if (k == 1) {
+        if (x < -0.25f) return -2.0f * (e - (x + 0.5f));
+        return one + 2.0f * (x - e);
+    }
+    const uint32_t kexp = (uint32_t)k << 23;
+    if (k <= -2 || k > 56) {
+        y = one - (e - x);
+        y = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, y) + kexp);
+        return y - one;
+    }
+    if (k < 23) {
+        t = __builtin_bit_cast(float, 0x3f800000u - (0x1000000u >> k));      // 1 - 2^-k
+        y = t - (e - x);
+        y = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, y) + kexp);
+    } else {
+        t = __builtin_bit_cast(float, (uint32_t)(0x7f - k) << 23);            // 2^-k
+        y = x - (e + t);
+        y += one;
+        y = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, y) + kexp);
+    }
+    return y;
+}
+
+__host__ __device__ inline float tanhf_as_host(float x) {
+#pragma clang fp contract(off)
+    const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
+    const uint32_t xb = __builtin_bit_cast(uint32_t, x);
+    const bool neg = (xb & 0x80000000u) != 0;
+    const uint32_t ix = xb & 0x7fffffffu;
+    const float ax = __builtin_bit_cast(float, ix);
+    float z;
+    if (ix >= 0x7f800000u) return neg ? one / x - one : one / x + one;        // +-1 for inf, nan for nan
+    if (ix < 0x41b00000u) {                                      // |x| < 22
+        if (ix == 0) return x;
+        if (ix < 0x24000000u) return x * (one + x);              // |x| < 2^-55
+        if (ix >= 0x3f800000u) {
+            const float t = expm1f_as_host(two * ax);
+            z = one - two / (t + two);
+        } else {
+            const float t = expm1f_as_host(-two * ax);
+            z = -t / (t + two);
+        }
+    } else {
+        z = one - tiny;
+    }
+    return neg ? -z : z;
+}
+
+// which host function a verification call addresses
+enum { HOSTMATH_EXPF = 0, HOSTMATH_TANHF = 1 };
+__host__ __device__ __forceinline__ float hostmath_eval(int fn, float x) {
+    return fn == HOSTMATH_TANHF ? tanhf_as_host(x) : expf_as_host(x);
+}
+
+// order-independent checksum of a restated function over `count` consecutive float bit patterns
+__host__ __device__ __forceinline__ uint64_t hostmath_mix(int fn, uint32_t in_bits) {
+    const uint32_t out = __builtin_bit_cast(uint32_t, hostmath_eval(fn, __builtin_bit_cast(float, in_bits)));
     return ((uint64_t)out + 1ull) * (0x9e3779b97f4a7c15ull ^ ((uint64_t)in_bits << 17));
 }
 
-__global__ __launch_bounds__(256) void k_expf_checksum(uint32_t first_bits, uint64_t count,
-                                                       unsigned long long *__restrict__ out) {
+__global__ __launch_bounds__(256) void k_hostmath_checksum(int fn, uint32_t first_bits, uint64_t count,
+                                                           unsigned long long *__restrict__ out) {
     uint64_t acc = 0;
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (uint64_t)gridDim.x * blockDim.x)
-        acc += sample_exp_mix(first_bits + (uint32_t)i);
+        acc += hostmath_mix(fn, first_bits + (uint32_t)i);
     atomicAdd(out, (unsigned long long)acc);
 }
 
-__global__ void k_expf_eval(const float *__restrict__ in, float *__restrict__ out, size_t n) {
+__global__ void k_hostmath_eval(int fn, const float *__restrict__ in, float *__restrict__ out, size_t n) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = expf_as_host(in[i]);
+    if (i < n) out[i] = hostmath_eval(fn, in[i]);
 }
 
 // ---------------------------------------------------------------- run state
 struct SampleParams {        // device-resident; written by the host before a run
     float temperature;
-    float softcap;           // the block path re-applies it when it reads the chosen block
+    float softcap;           // top-k: applied to the merged candidates; block path: to the chosen block's logits
     int top_k;
     int step;                // ring slot of the step that is running
     int ring_cap;            // steps the ring holds
@@ -142,7 +251,7 @@ __global__ __launch_bounds__(256) void k_sample_topk(const float *__restrict__ v
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row = blockIdx.x, rows = gridDim.x;
     const int k = ss->top_k, step = ss->step;
-    const float temperature = ss->temperature;
+    const float temperature = ss->temperature, cap = ss->softcap;
     const float *v = vals + (size_t)row * blocks * k;
     const uint32_t *ix = idxs + (size_t)row * blocks * k;
     int ptr[4];
@@ -192,6 +301,8 @@ __global__ __launch_bounds__(256) void k_sample_topk(const float *__restrict__ v
         }
     }
     if (tid != 0) return;
+    if (cap > 0.0f)                                            // decode.rs:155-159
+        for (int i = 0; i < n; ++i) mv[i] = __fmul_rn(cap, tanhf_as_host(__fdiv_rn(mv[i], cap)));
     uint64_t s = rng[row];
     uint32_t tok = 0;
     if (n > 0) {

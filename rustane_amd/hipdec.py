@@ -30,8 +30,8 @@ EXPORTS = [
     "hipdec_decode_token_argmax_from_ids_batch", "hipdec_decode_token_topk_from_ids_batch",
     "hipdec_decode_token_block_stats_from_ids_batch", "hipdec_materialize_current_logits_block_batch",
     "hipdec_decode_topk_sampled_run", "hipdec_decode_fullvocab_sampled_run", "hipdec_decode_topk_sampled_run_batch",
-    "hipdec_decode_fullvocab_sampled_run_batch", "hipdec_debug_expf", "hipdec_debug_expf_checksum",
-    "hipdec_debug_expf_count_mismatch",
+    "hipdec_decode_fullvocab_sampled_run_batch", "hipdec_debug_hostmath_eval", "hipdec_debug_hostmath_checksum",
+    "hipdec_debug_hostmath_count_mismatch",
 ]
 
 
@@ -144,38 +144,43 @@ def load_library(path=None):
                                                          C.c_size_t, u32p]
     lib.hipdec_decode_fullvocab_sampled_run_batch.argtypes = [C.c_void_p, u32p, C.c_float, C.c_float, u64p, C.c_size_t,
                                                               u32p]
-    lib.hipdec_debug_expf.argtypes = [fp, fp, C.c_size_t, C.c_int]
-    lib.hipdec_debug_expf_checksum.argtypes = [C.c_uint32, C.c_uint64, C.c_int, C.c_int, u64p]
-    lib.hipdec_debug_expf_count_mismatch.argtypes = [C.c_uint32, C.c_uint64, C.c_int, u64p]
+    lib.hipdec_debug_hostmath_eval.argtypes = [C.c_int, fp, fp, C.c_size_t, C.c_int]
+    lib.hipdec_debug_hostmath_checksum.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int, C.c_int, u64p]
+    lib.hipdec_debug_hostmath_count_mismatch.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int, u64p]
     if path is None:
         _LIB = lib
     return lib
 
 
-def debug_expf(x, on_device=False):
-    """The sampler's exponential (the host C library's expf restated) on the host or on the GPU."""
+HOSTMATH_EXPF, HOSTMATH_TANHF = 0, 1
+
+
+def debug_hostmath(fn, x, on_device=False):
+    """The sampler's restatement of the host C library's expf (fn 0) or tanhf (fn 1), evaluated on
+    the host or on the GPU."""
     x = np.ascontiguousarray(x, dtype=np.float32)
     out = np.empty_like(x)
-    rc = load_library().hipdec_debug_expf(_fptr(x), _fptr(out), x.size, 1 if on_device else 0)
+    rc = load_library().hipdec_debug_hostmath_eval(fn, _fptr(x), _fptr(out), x.size, 1 if on_device else 0)
     if rc != OK:
-        raise HipDecodeError(rc, "hipdec_debug_expf failed")
+        raise HipDecodeError(rc, "hipdec_debug_hostmath_eval failed")
     return out
 
 
-def debug_expf_checksum(first_bits, count, on_device=False, host_threads=8):
+def debug_hostmath_checksum(fn, first_bits, count, on_device=False, host_threads=8):
     out = C.c_uint64()
-    rc = load_library().hipdec_debug_expf_checksum(first_bits, count, 1 if on_device else 0, host_threads, C.byref(out))
+    rc = load_library().hipdec_debug_hostmath_checksum(fn, first_bits, count, 1 if on_device else 0, host_threads,
+                                                       C.byref(out))
     if rc != OK:
-        raise HipDecodeError(rc, "hipdec_debug_expf_checksum failed")
+        raise HipDecodeError(rc, "hipdec_debug_hostmath_checksum failed")
     return out.value
 
 
-def debug_expf_count_mismatch(first_bits, count, host_threads=8):
-    """How many of `count` consecutive float bit patterns give a result different from libm's expf."""
+def debug_hostmath_count_mismatch(fn, first_bits, count, host_threads=8):
+    """How many of `count` consecutive float bit patterns give a result different from libm's function."""
     out = C.c_uint64()
-    rc = load_library().hipdec_debug_expf_count_mismatch(first_bits, count, host_threads, C.byref(out))
+    rc = load_library().hipdec_debug_hostmath_count_mismatch(fn, first_bits, count, host_threads, C.byref(out))
     if rc != OK:
-        raise HipDecodeError(rc, "hipdec_debug_expf_count_mismatch failed")
+        raise HipDecodeError(rc, "hipdec_debug_hostmath_count_mismatch failed")
     return out.value
 
 

@@ -3,10 +3,14 @@ engine/src/decode.rs:218-253 and the draws of engine/src/inference.rs:823-921 do
 give, token for token and with the same final RNG state, what the reference's loop gives when it
 reads the candidates / block statistics back and draws on the host (inference.rs:586-625).
 
-The draw needs exp() with the host C library's bits.  The restatement the kernels use is checked
-here (a) on the host against libm's expf for EVERY float <= 0 (the sampler's arguments are
-differences to a maximum, so never positive) and for 0..89, (b) against float64 exp, and (c) on the
-GPU against the host evaluation through checksums over the same ranges."""
+The draw needs exp() -- and the softcap of the merged candidates tanh() -- with the host C library's
+bits.  The restatements the kernels use are checked here (a) on the host against libm: expf for
+EVERY float <= 0 (the sampler's arguments are differences to a maximum, so never positive) and for
+0..89, tanhf for all 2^32 floats; (b) against float64 exp / tanh; and (c) on the GPU against the
+host evaluation through checksums over the same ranges."""
+import ctypes as C
+import ctypes.util
+
 import numpy as np
 import pytest
 
@@ -15,46 +19,84 @@ from rustane_amd import engine as E
 from rustane_amd import hipdec, synth
 from rustane_amd.hipdec import Config, HipDecodeModel, KvDtype, WeightDtype
 
+LIBM = C.CDLL(ctypes.util.find_library("m") or "libm.so.6")
+LIBM.tanhf.restype = C.c_float
+LIBM.tanhf.argtypes = [C.c_float]
+
 NEG_FIRST, NEG_COUNT = 0x80000000, 0xFF800000 - 0x80000000 + 1      # -0.0 .. -inf
 POS_FIRST, POS_COUNT = 0x00000000, 0x42B20000 + 1                   # +0.0 .. 89.0
 
 
 # ------------------------------------------------------------------ the exponential (CPU)
+EXPF, TANHF = hipdec.HOSTMATH_EXPF, hipdec.HOSTMATH_TANHF
+
+
 def test_restated_expf_equals_libm_for_every_non_positive_float():
-    assert hipdec.debug_expf_count_mismatch(NEG_FIRST, NEG_COUNT, host_threads=8) == 0
-    assert hipdec.debug_expf_count_mismatch(POS_FIRST, POS_COUNT, host_threads=8) == 0
+    assert hipdec.debug_hostmath_count_mismatch(EXPF, NEG_FIRST, NEG_COUNT, host_threads=8) == 0
+    assert hipdec.debug_hostmath_count_mismatch(EXPF, POS_FIRST, POS_COUNT, host_threads=8) == 0
+
+
+def test_restated_tanhf_equals_libm_for_every_float():
+    assert hipdec.debug_hostmath_count_mismatch(TANHF, 0, 1 << 32, host_threads=8) == 0
+
+
+def test_restated_tanhf_known_answers_and_float64_reference():
+    x = np.array([0.0, -0.0, np.inf, -np.inf, 30.0, -30.0, 1e-20, 0.5, -2.0], np.float32)
+    y = hipdec.debug_hostmath(TANHF, x)
+    assert y[0] == 0.0 and np.signbit(y[1]) and y[2] == 1.0 and y[3] == -1.0 and y[4] == 1.0 and y[5] == -1.0
+    assert y[6] == np.float32(1e-20)
+    assert np.isnan(hipdec.debug_hostmath(TANHF, np.array([np.nan], np.float32))[0])
+    rng = np.random.default_rng(6)
+    x = np.concatenate([(rng.random(200000) * 2 - 1) * 12.0, (rng.random(100000) * 2 - 1) * 0.3]).astype(np.float32)
+    y = hipdec.debug_hostmath(TANHF, x)
+    want = np.tanh(x.astype(np.float64))
+    ulp = np.spacing(np.abs(want).astype(np.float32)).astype(np.float64)
+    assert np.all(np.abs(y.astype(np.float64) - want) <= 2.5 * ulp)         # the classic routine is good to ~2 ulp
+    np.testing.assert_array_equal(hipdec.debug_hostmath(TANHF, -x), -y)    # odd
 
 
 def test_restated_expf_known_answers_and_float64_reference():
     x = np.array([0.0, -0.0, -np.inf, np.inf, -104.0, -200.0, 89.0, 1.0, -1.0], np.float32)
-    y = hipdec.debug_expf(x)
+    y = hipdec.debug_hostmath(EXPF, x)
     assert y[0] == 1.0 and y[1] == 1.0 and y[2] == 0.0 and np.isinf(y[3]) and y[4] == 0.0 and y[5] == 0.0
     assert np.isinf(y[6])                                            # exp(89) overflows float
     assert y[7] == np.float32(np.e) and y[8] == np.float32(1.0 / np.e)
-    assert np.isnan(hipdec.debug_expf(np.array([np.nan], np.float32))[0])
+    assert np.isnan(hipdec.debug_hostmath(EXPF, np.array([np.nan], np.float32))[0])
     rng = np.random.default_rng(5)
     x = np.concatenate([-rng.random(200000) * 104.0, rng.random(50000) * 88.0, -rng.random(50000) * 1e-3]).astype(np.float32)
-    y = hipdec.debug_expf(x)
+    y = hipdec.debug_hostmath(EXPF, x)
     want = np.exp(x.astype(np.float64))
     # the C library documents 0.502 units in the last place for this algorithm
     ulp = np.maximum(np.spacing(want.astype(np.float32)).astype(np.float64), 2.0 ** -149)
     assert np.all(np.abs(y.astype(np.float64) - want) <= 0.503 * ulp)
     # subnormal results are produced, not flushed
-    assert hipdec.debug_expf(np.array([-100.0], np.float32))[0] == np.float32(np.exp(-100.0))
+    assert hipdec.debug_hostmath(EXPF, np.array([-100.0], np.float32))[0] == np.float32(np.exp(-100.0))
 
 
 # ------------------------------------------------------------------ the exponential (GPU)
 @pytest.mark.gpu
 def test_device_expf_equals_host_expf_for_every_non_positive_float():
     for first, count in ((NEG_FIRST, NEG_COUNT), (POS_FIRST, POS_COUNT)):
-        host = hipdec.debug_expf_checksum(first, count, on_device=False, host_threads=16)
-        dev = hipdec.debug_expf_checksum(first, count, on_device=True)
+        host = hipdec.debug_hostmath_checksum(EXPF, first, count, on_device=False, host_threads=16)
+        dev = hipdec.debug_hostmath_checksum(EXPF, first, count, on_device=True)
         assert host == dev, (hex(first), hex(host), hex(dev))
     # element-wise on a sample, subnormal results and the special values included
     rng = np.random.default_rng(9)
     x = np.concatenate([-rng.random(100000) * 104.0, np.array([0.0, -0.0, -np.inf, -87.5, -88.0, -95.0, -103.9, -104.5])])
     x = x.astype(np.float32)
-    np.testing.assert_array_equal(hipdec.debug_expf(x, on_device=True).view(np.uint32), hipdec.debug_expf(x).view(np.uint32))
+    np.testing.assert_array_equal(hipdec.debug_hostmath(EXPF, x, on_device=True).view(np.uint32), hipdec.debug_hostmath(EXPF, x).view(np.uint32))
+
+
+@pytest.mark.gpu
+def test_device_tanhf_equals_host_tanhf_for_every_float():
+    host = hipdec.debug_hostmath_checksum(TANHF, 0, 1 << 32, on_device=False, host_threads=16)
+    dev = hipdec.debug_hostmath_checksum(TANHF, 0, 1 << 32, on_device=True)
+    assert host == dev, (hex(host), hex(dev))
+    rng = np.random.default_rng(10)
+    x = np.concatenate([(rng.random(100000) * 2 - 1) * 25.0, np.array([0.0, -0.0, np.inf, -np.inf, 1e-30, 0.3465, 1.0, 22.0])])
+    x = x.astype(np.float32)
+    np.testing.assert_array_equal(hipdec.debug_hostmath(TANHF, x, on_device=True).view(np.uint32),
+                                  hipdec.debug_hostmath(TANHF, x).view(np.uint32))
 
 
 # ------------------------------------------------------------------ runs against the host loop
@@ -71,13 +113,23 @@ def two_models(cfg, w, wd, kv, prompt):
     return a, b, la
 
 
-def host_topk_loop(dev, tok, k, T, seed, steps):
+def host_softcap(v, cap):
+    """decode.rs:155-159: cap * tanhf(v / cap) with the host C library's tanhf (float operations only)."""
+    if cap <= 0.0:
+        return v
+    cap = np.float32(cap)
+    t = np.array([LIBM.tanhf(C.c_float(float(np.float32(x) / cap))) for x in v], np.float32)
+    return (cap * t).astype(np.float32)
+
+
+def host_topk_loop(dev, tok, k, T, seed, steps, softcap=0.0):
     """inference.rs:586-599 with the oracle's merge and draw over the device's candidates."""
     rng = O.Rng(seed)
     out = []
     for _ in range(steps):
         vals, idxs = dev.decode_token_topk_from_id(tok, k)
         mv, mi = O.merge_topk(vals, idxs, k)
+        mv = host_softcap(mv, softcap)
         tok = int(O.lib().orc_sample_topk_candidates(O.PU(mi), O.P(mv), mi.size, T, rng.ref))
         out.append(tok)
     return np.array(out, np.uint32), rng.s.value
@@ -98,27 +150,29 @@ def host_fullvocab_loop(dev, tok, T, softcap, seed, steps):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("wd,kv,vocab,k,T", [
-    (WeightDtype.BF16, KvDtype.BF16, 1000, 8, 0.8),      # last block holds 232 rows
-    (WeightDtype.F32, KvDtype.F32, 8192, 4, 1.3),
-    (WeightDtype.FP8_E4M3, KvDtype.BF16, 320, 32, 0.5),  # k > rows of the last block (64): padded lists
-    (WeightDtype.BF16, KvDtype.F32, 1000, 1, 0.8),       # one candidate: no draw, the state stays
-    (WeightDtype.BF16, KvDtype.F32, 1000, 5, 0.0),       # temperature 0: first candidate, no draw
+@pytest.mark.parametrize("wd,kv,vocab,k,T,softcap", [
+    (WeightDtype.BF16, KvDtype.BF16, 1000, 8, 0.8, 0.0),      # last block holds 232 rows
+    (WeightDtype.F32, KvDtype.F32, 8192, 4, 1.3, 0.0),
+    (WeightDtype.FP8_E4M3, KvDtype.BF16, 320, 32, 0.5, 0.0),  # k > rows of the last block (64): padded lists
+    (WeightDtype.BF16, KvDtype.F32, 1000, 1, 0.8, 0.0),       # one candidate: no draw, the state stays
+    (WeightDtype.BF16, KvDtype.F32, 1000, 5, 0.0, 0.0),       # temperature 0: first candidate, no draw
+    (WeightDtype.BF16, KvDtype.BF16, 1000, 8, 0.8, 3.0),      # softcap on the merged candidates (host tanhf)
+    (WeightDtype.F32, KvDtype.F32, 8192, 16, 0.6, 0.75),
 ])
-def test_topk_run_on_device_equals_host_loop(wd, kv, vocab, k, T):
+def test_topk_run_on_device_equals_host_loop(wd, kv, vocab, k, T, softcap):
     cfg = small_cfg(vocab)
     w = synth.make_weights(cfg, seed=13, std=0.08, round_bf16=True)
     a, b, lg = two_models(cfg, w, wd, kv, [3, 1, 4, 1, 5, 9, 2, 6])
     first = int(np.argmax(lg))
     steps, seed = 40, 0x1234567
-    got, state = a.decode_topk_sampled_run(first, k, T, seed, steps)
-    want, want_state = host_topk_loop(b, first, k, T, seed, steps)
+    got, state = a.decode_topk_sampled_run(first, k, T, seed, steps, softcap=softcap)
+    want, want_state = host_topk_loop(b, first, k, T, seed, steps, softcap)
     np.testing.assert_array_equal(got, want)
     assert state == want_state
     assert a.len() == b.len() == 8 + steps
     # a second run continues from where the first stopped, with the advanced state
-    got2, state2 = a.decode_topk_sampled_run(int(got[-1]), k, T, state, 7)
-    want2, want_state2 = host_topk_loop(b, int(want[-1]), k, T, want_state, 7)
+    got2, state2 = a.decode_topk_sampled_run(int(got[-1]), k, T, state, 7, softcap=softcap)
+    want2, want_state2 = host_topk_loop(b, int(want[-1]), k, T, want_state, 7, softcap)
     np.testing.assert_array_equal(got2, want2)
     assert state2 == want_state2
     if k > 1 and T > 0:
@@ -146,7 +200,7 @@ def test_fullvocab_run_on_device_equals_host_loop(wd, kv, vocab, T, softcap):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("k,T,softcap", [(8, 0.8, 0.0), (0, 1.0, 0.0), (0, 0.9, 3.0)])
+@pytest.mark.parametrize("k,T,softcap", [(8, 0.8, 0.0), (0, 1.0, 0.0), (0, 0.9, 3.0), (6, 0.7, 2.0)])
 def test_batched_run_on_device_equals_per_step_batch_calls(k, T, softcap):
     cfg = small_cfg(1000)
     w = synth.make_weights(cfg, seed=19, std=0.08, round_bf16=True)
@@ -157,7 +211,7 @@ def test_batched_run_on_device_equals_per_step_batch_calls(k, T, softcap):
     a.batch_begin(R)
     b.batch_begin(R)
     if k > 0:
-        got, states = a.decode_topk_sampled_run_batch(first, k, T, seeds, steps)
+        got, states = a.decode_topk_sampled_run_batch(first, k, T, seeds, steps, softcap=softcap)
     else:
         got, states = a.decode_fullvocab_sampled_run_batch(first, T, seeds, steps, softcap=softcap)
     rngs = [O.Rng(int(s)) for s in seeds]
@@ -169,6 +223,7 @@ def test_batched_run_on_device_equals_per_step_batch_calls(k, T, softcap):
             vals, idxs = b.decode_token_topk_from_ids_batch(cur, k)
             for r in range(R):
                 mv, mi = O.merge_topk(vals[r], idxs[r], k)
+                mv = host_softcap(mv, softcap)
                 nxt[r] = O.lib().orc_sample_topk_candidates(O.PU(mi), O.P(mv), mi.size, T, rngs[r].ref)
         else:
             mx, sm = b.decode_token_block_stats_from_ids_batch(cur, inv_t, softcap)
@@ -188,14 +243,11 @@ def test_batched_run_on_device_equals_per_step_batch_calls(k, T, softcap):
 
 
 @pytest.mark.gpu
-def test_run_argument_errors_and_unsupported_softcap():
+def test_run_argument_errors():
     cfg = small_cfg(1000, seq=32)
     w = synth.make_weights(cfg, seed=13, std=0.08, round_bf16=True)
     m = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.F32)
     m.prefill(np.array([1, 2, 3, 4], np.uint32))
-    with pytest.raises(hipdec.HipDecodeError) as e:
-        m.decode_topk_sampled_run(1, 8, 0.8, 1, 4, softcap=3.0)     # the host applies tanhf to the candidates
-    assert e.value.status == hipdec.ERR_UNSUPPORTED
     for bad_k in (0, 33):
         with pytest.raises(hipdec.HipDecodeError) as e:
             m.decode_topk_sampled_run(1, bad_k, 0.8, 1, 4)
