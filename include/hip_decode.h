@@ -182,7 +182,8 @@ int hipdec_decode_greedy_run(hipdec_model *m, uint32_t token, size_t n_steps, ui
  * hipdec_decode_token_block_stats_from_id + block draw + hipdec_materialize_current_logits_block +
  * token draw); with softcap > 0 the top-k form applies cap * tanhf(v / cap) to the merged candidates
  * as the host does (decode.rs:155-159), the host C library's tanhf reproduced bit for bit as well.
- * Needs vocab <= 262144 (HIPDEC_ERR_UNSUPPORTED otherwise). */
+ * Needs vocab <= 262144, and a host C library whose expf and tanhf are the ones reproduced (probed
+ * once per process on 2^21 inputs); HIPDEC_ERR_UNSUPPORTED otherwise, and nothing has run. */
 int hipdec_decode_topk_sampled_run(hipdec_model *m, uint32_t token, uint32_t top_k, float temperature, float softcap,
                                    uint64_t *rng_state, size_t n_steps, uint32_t *out_tokens);
 int hipdec_decode_fullvocab_sampled_run(hipdec_model *m, uint32_t token, float temperature, float softcap,
@@ -217,6 +218,9 @@ int hipdec_debug_step_profile(hipdec_model *m, uint32_t token, uint64_t *out, si
  * the known-size yardstick that hardware memory-traffic counters are scaled by. */
 int hipdec_debug_calibration_copy(size_t bytes, int reps);
 
+/* 1 when this host's C library computes expf and tanhf as the on-device sampler reproduces them
+ * (the probe the sampled runs consult), else 0. */
+int hipdec_debug_hostmath_probe(void);
 /* Verification of the two host C library functions the on-device sampler restates (fn 0: expf,
  * fn 1: tanhf): evaluate the restatement for n inputs on the host (on_device = 0) or on the GPU; */
 int hipdec_debug_hostmath_eval(int fn, const float *in, float *out, size_t n, int on_device);

@@ -789,10 +789,39 @@ float sample_inv_temperature(float temperature) {              // engine/src/dec
     return 1.0f / (temperature > tiny ? temperature : tiny);
 }
 
+// The device draws are only offered where the restated expf/tanhf equal THIS host's C library (a
+// different libm would make device runs and per-step host draws disagree in rare last-bit cases):
+// checked once per process on 2^20 inputs each, spread over the whole range, plus the one input
+// known to separate the C library's fused and unfused expf variants.
+bool hostmath_matches_libm() {
+    static const bool ok = [] {
+        auto same = [](float a, float b) {
+            uint32_t ab, bb;
+            memcpy(&ab, &a, 4);
+            memcpy(&bb, &b, 4);
+            return ab == bb || (a != a && b != b);
+        };
+        auto at = [](uint32_t bits) { float x; memcpy(&x, &bits, 4); return x; };
+        volatile uint32_t special = 0xc27c65d9u;                   // volatile: the C library must run, not the compiler's folder
+        const float xs = at(special);
+        if (!same(expf(xs), expf_as_host(xs))) return false;
+        for (uint32_t i = 0; i < (1u << 20); ++i) {
+            const float xe = at(0x80000000u + i * 2039u);          // -0.0 .. about -1e38
+            if (!same(expf(xe), expf_as_host(xe))) return false;
+            const float xt = at(i * 4093u + 7u);                   // all signs and magnitudes
+            if (!same(tanhf(xt), tanhf_as_host(xt))) return false;
+        }
+        return true;
+    }();
+    return ok;
+}
+
 int sampled_args_ok(hipdec_model *m, bool topk, uint32_t top_k, float temperature, float softcap, const uint64_t *rng,
                     const uint32_t *out_tokens) {
     if (!rng || !out_tokens) return fail(m, HIPDEC_ERR_ARG, "null buffer");
     if (m->blocks > SAMPLE_MAX_BLOCKS) return fail(m, HIPDEC_ERR_UNSUPPORTED, "on-device sampling serves up to 1024 vocab blocks");
+    if (!hostmath_matches_libm())
+        return fail(m, HIPDEC_ERR_UNSUPPORTED, "this host's expf/tanhf differ from the ones the device sampler reproduces: use the per-step calls");
     (void)softcap;
     if (topk) {
         if (top_k == 0 || top_k > HIPDEC_MAX_GPU_TOPK) return fail(m, HIPDEC_ERR_ARG, "gpu top-k only supports k in 1..32");
@@ -1486,6 +1515,8 @@ int hipdec_decode_fullvocab_sampled_run_batch(hipdec_model *m, const uint32_t *t
                                               uint64_t *rng_states, size_t n_steps, uint32_t *out_tokens) {
     return batch_sampled_run(m, B_STATS_S, tokens, 1, temperature, softcap, rng_states, n_steps, out_tokens);
 }
+
+int hipdec_debug_hostmath_probe(void) { return hostmath_matches_libm() ? 1 : 0; }
 
 int hipdec_debug_hostmath_eval(int fn, const float *in, float *out, size_t n, int on_device) {
     if (!in || !out || (fn != HOSTMATH_EXPF && fn != HOSTMATH_TANHF)) return HIPDEC_ERR_ARG;

@@ -31,7 +31,7 @@ EXPORTS = [
     "hipdec_decode_token_block_stats_from_ids_batch", "hipdec_materialize_current_logits_block_batch",
     "hipdec_decode_topk_sampled_run", "hipdec_decode_fullvocab_sampled_run", "hipdec_decode_topk_sampled_run_batch",
     "hipdec_decode_fullvocab_sampled_run_batch", "hipdec_debug_hostmath_eval", "hipdec_debug_hostmath_checksum",
-    "hipdec_debug_hostmath_count_mismatch",
+    "hipdec_debug_hostmath_count_mismatch", "hipdec_debug_hostmath_probe",
 ]
 
 

@@ -36,6 +36,11 @@ def test_restated_expf_equals_libm_for_every_non_positive_float():
     assert hipdec.debug_hostmath_count_mismatch(EXPF, POS_FIRST, POS_COUNT, host_threads=8) == 0
 
 
+def test_library_probe_accepts_this_hosts_libm():
+    # the sampled runs answer UNSUPPORTED where this is 0; here it must hold (the two exhaustive tests say so)
+    assert hipdec.load_library().hipdec_debug_hostmath_probe() == 1
+
+
 def test_restated_tanhf_equals_libm_for_every_float():
     assert hipdec.debug_hostmath_count_mismatch(TANHF, 0, 1 << 32, host_threads=8) == 0
 
