@@ -101,7 +101,7 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
                 for (int e = 0; e < EPL; ++e) p = fmaf(wf[e], xv[e], p);
                 if (WT == WT_INT4) {
                     const uint16_t *sc = (const uint16_t *)a.scales + (size_t)rowi[r] * (K / 128);
-                    p *= bf16_to_f32(sc[(c * EPL) / 128]);
+                    p *= bf16_to_f32(sc[(c * EPL) / 128]) * WS<WT_INT4>::SCALE_MUL;
                 }
                 acc[r] += p;
             }

@@ -593,7 +593,10 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                                 float p0 = 0.0f, p1 = 0.0f;
 #pragma unroll
                                 for (int e = 0; e < EPL; ++e) { p0 = fmaf(w0[e], xv[e], p0); p1 = fmaf(w1[e], xv[e], p1); }
-                                if (WT == WT_INT4) { p0 *= bf16_to_f32(st[s].sc[0][j]); p1 *= bf16_to_f32(st[s].sc[1][j]); }
+                                if (WT == WT_INT4) {
+                                    p0 *= bf16_to_f32(st[s].sc[0][j]) * WS<WT_INT4>::SCALE_MUL;
+                                    p1 *= bf16_to_f32(st[s].sc[1][j]) * WS<WT_INT4>::SCALE_MUL;
+                                }
                                 acc[s][0] += p0; acc[s][1] += p1;
                             }
                         }
