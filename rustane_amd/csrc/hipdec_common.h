@@ -58,6 +58,16 @@ __device__ __forceinline__ void wave_argbest(float &v, uint32_t &i) {
     }
 }
 
+// 16-byte load of data that is used once per step (the weight stream of the persistent decode
+// kernel): the non-temporal hint keeps it from displacing what the caches should hold (600M step
+// 0.730 -> 0.708 ms, 5B 3.10 -> 2.89 ms).  Not for the multi-row streaming GEMM, where neighbouring
+// lanes' 32-byte pieces share cache lines across instructions: there the hint costs 15 %.
+typedef uint32_t stream_u4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 ld_stream_u4(const void *p) {
+    const stream_u4 v = __builtin_nontemporal_load((const __attribute__((address_space(1))) stream_u4 *)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 // ---------------------------------------------------------------- weight stream decoders
 // Every weight matrix is stored out-major: row = output channel, reduction axis contiguous, so
 // one 128-bit load gives a lane EPL consecutive reduction elements of one output row.

@@ -331,7 +331,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                     if (piece < p_pieces) {
 #pragma unroll
                         for (int r = 0; r < 2; ++r) {
-                            st[s].w[r][j] = ldg_u4(p_W + (row + r) * p_rb + (size_t)piece * 16);
+                            st[s].w[r][j] = ld_stream_u4(p_W + (row + r) * p_rb + (size_t)piece * 16);
                             if (WT == WT_INT4) st[s].sc[r][j] = ldg_u16(p_SC + (row + r) * p_kg + (piece >> 2));   // 4-bit models keep the head outside
                         }
                     }
