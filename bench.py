@@ -41,7 +41,7 @@ C3_SAMPLES, C3_TEMPERATURE, C3_TOP_K = 8, 0.8, 8
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, each
 # scaled by what the same counter reads for a plain copy of known size): measured separately with
 # rocprofv3 --pmc and recorded in profiles/k_mega_c2_600m_bf16_bs1.md; a benchmark run cannot collect it itself.
-MEASURED_TRAFFIC_BYTES = {"c2_600m_bf16_bs1": 1.512e9}
+MEASURED_TRAFFIC_BYTES = {"c2_600m_bf16_bs1": 1.509e9}
 
 
 def run_c3(args, cfg, weights, n_prompt):
