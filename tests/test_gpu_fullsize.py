@@ -75,6 +75,60 @@ def test_600m_chained_greedy_run_equals_single_calls(w600):
     assert dev.len() == 168
 
 
+def test_600m_sampled_runs_on_the_device_equal_the_host_loop(w600):
+    """The two sampled workloads at the benchmark model's size (128 vocab blocks): tokens drawn on the
+    device (hipdec_decode_*_sampled_run*) against the reference's loop -- candidates / statistics
+    read back each step, the oracle's merge and draws on the host (inference.rs:586-625)."""
+    cfg, w = w600
+    a = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.BF16)
+    b = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.BF16)
+    ids = synth.make_prompt(7, cfg.vocab, 256)
+    lg = a.prefill(ids)
+    np.testing.assert_array_equal(lg, b.prefill(ids))
+    first = int(np.argmax(lg))
+    steps = 24
+    # top-k 8 at T 0.8 (one draw per token)
+    got, state = a.decode_topk_sampled_run(first, 8, 0.8, 1234, steps)
+    rng, tok, want = O.Rng(1234), first, []
+    for _ in range(steps):
+        vals, idxs = b.decode_token_topk_from_id(tok, 8)
+        mv, mi = O.merge_topk(vals, idxs, 8)
+        tok = int(O.lib().orc_sample_topk_candidates(O.PU(mi), O.P(mv), mi.size, 0.8, rng.ref))
+        want.append(tok)
+    np.testing.assert_array_equal(got, np.array(want, np.uint32))
+    assert state == rng.s.value
+    # full vocabulary at T 1.0 (block draw, then token draw), continuing both models
+    got, state = a.decode_fullvocab_sampled_run(int(got[-1]), 1.0, 99, steps)
+    rng, want = O.Rng(99), []
+    for _ in range(steps):
+        mx, sm = b.decode_token_block_stats_from_id(tok, 1.0, 0.0)
+        blk = int(O.lib().orc_sample_block_from_stats(O.P(mx), O.P(sm), mx.size, rng.ref))
+        bl = b.materialize_current_logits_block(blk, 0.0)
+        tok = int(O.lib().orc_sample_block_logits(blk * 256, O.P(bl), bl.size, 1.0, rng.ref))
+        want.append(tok)
+    np.testing.assert_array_equal(got, np.array(want, np.uint32))
+    assert state == rng.s.value
+    # 8 rows stepped together, top-k 8: every row against its own host loop over the batched candidates
+    rows = 8
+    a.batch_begin(rows)
+    b.batch_begin(rows)
+    starts = np.argsort(-lg, kind="stable")[:rows].astype(np.uint32)
+    seeds = np.arange(rows, dtype=np.uint64) + np.uint64(5)
+    got, states = a.decode_topk_sampled_run_batch(starts, 8, 0.8, seeds, steps)
+    rngs, cur = [O.Rng(int(x)) for x in seeds], starts.copy()
+    for i in range(steps):
+        vals, idxs = b.decode_token_topk_from_ids_batch(cur, 8)
+        nxt = np.empty(rows, np.uint32)
+        for r in range(rows):
+            mv, mi = O.merge_topk(vals[r], idxs[r], 8)
+            nxt[r] = O.lib().orc_sample_topk_candidates(O.PU(mi), O.P(mv), mi.size, 0.8, rngs[r].ref)
+        np.testing.assert_array_equal(got[i], nxt, err_msg="step %d" % i)
+        cur = nxt
+    np.testing.assert_array_equal(states, np.array([x.s.value for x in rngs], np.uint64))
+    a.batch_end()
+    b.batch_end()
+
+
 @pytest.mark.parametrize("kvdt,tol", [(KvDtype.F32, 2e-4), (KvDtype.BF16, 2e-2)])
 def test_5b_bf16_short_prompt_against_the_oracle(w5b, kvdt, tol):
     # fp32 cache: the fp32-path bound (1e-4 at the reference's tiny test shapes, crates/engine/tests/
