@@ -108,6 +108,9 @@ int main(int argc, char **argv) {
             if (!parse_decode_backend(raw, &req.decode_backend))
                 fail("--decode-backend must be one of: auto, naive, hip; got " + raw);
         } else if (a == "--help" || a == "-h") { usage(); return 0; }
+        else if (a == "--prompt" || a == "--tokenizer" || a == "--add-special-tokens" || a == "--no-skip-special-tokens")
+            // generate.rs:173-188: text goes through the tokenizers crate there; this engine works on ids
+            fail(a + " needs a tokenizer, which this build does not carry: pass the prompt as --prompt-ids");
         else fail("unknown argument " + a);
     }
     if (req.samples == 0) fail("samples must be >= 1");

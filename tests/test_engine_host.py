@@ -163,3 +163,19 @@ def test_validate_token_ids_message_and_window():
     out = np.full(16, 9, np.uint32)
     assert L.rs_fill_input_window(gen.ctypes.data_as(u32p), 10, 16, out.ctypes.data_as(u32p)) == 10
     assert out.tolist() == list(range(1, 11)) + [0] * 6
+
+
+def test_generate_cli_refuses_text_flags_with_a_clear_message():
+    # generate.rs:173-188 takes text through a tokenizer; this build works on token ids only
+    import os
+    import subprocess
+    from rustane_amd import build as B
+    if not os.path.exists(B.GENERATE_BIN):
+        pytest.skip("generate binary not built")
+    for flag in ("--prompt", "--tokenizer"):
+        res = subprocess.run([B.GENERATE_BIN, "--model", "tiny", flag, "x"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                             text=True)
+        assert res.returncode != 0
+        assert "needs a tokenizer" in res.stdout and "--prompt-ids" in res.stdout
+    res = subprocess.run([B.GENERATE_BIN, "--frobnicate"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert res.returncode != 0 and "unknown argument --frobnicate" in res.stdout
