@@ -288,3 +288,43 @@ def test_error_codes_replace_panics():
     dev.set_len(cfg.seq - 1)
     dev.decode_token_argmax_from_id(1)     # the last slot is usable
     assert dev.len() == cfg.seq
+
+
+@pytest.mark.parametrize("wdt,kvdt", [(WeightDtype.F32, KvDtype.F32), (WeightDtype.BF16, KvDtype.BF16),
+                                      (WeightDtype.FP8_E4M3, KvDtype.BF16)])
+def test_graph_replay_equals_eager_launch_and_runs_repeat_bit_for_bit(wdt, kvdt):
+    """The reference checks its reordered schedules against the straightforward ones with tolerance 0.0
+    (its auto_*.rs tests).  Here: the captured-graph step against eager launches of the same kernels,
+    and a run against its own repetition -- every reduction has a fixed order, so the bits must agree.
+    Covers single steps, the chained greedy run and the multi-row step."""
+    cfg = tiny_cfg(1000)
+    w = synth.make_weights(cfg, seed=23, std=0.08, round_bf16=True)
+    graph = HipDecodeModel(cfg, w, weight_dtype=wdt, kv_dtype=kvdt)
+    eager = HipDecodeModel(cfg, w, weight_dtype=wdt, kv_dtype=kvdt, flags=1)
+    ids = np.array([7, 1, 9, 4, 4, 2, 8, 3, 5, 6], np.uint32)
+
+    def run(dev):
+        dev.set_len(0)
+        out = [dev.prefill(ids)]
+        tok = int(np.argmax(out[0]))
+        for _ in range(5):
+            out.append(dev.decode_logits_from_id(tok))
+            tok = int(np.argmax(out[-1]))
+        out.append(dev.decode_greedy_run(tok, 6).astype(np.float32))
+        vals, idxs = dev.decode_token_topk_from_id(int(out[-1][-1]), 4)
+        out += [vals, idxs.astype(np.float32)]
+        if wdt != WeightDtype.F32:                               # the multi-row step needs 16-bit or 8-bit weights
+            dev.batch_begin(3)
+            toks = np.array([1, 2, 3], np.uint32)
+            for _ in range(3):
+                lg = dev.decode_logits_from_ids_batch(toks)
+                out.append(lg)
+                toks = np.argmax(lg, axis=1).astype(np.uint32)
+            dev.batch_end()
+        return out
+
+    a, b, c = run(graph), run(eager), run(graph)
+    assert len(a) == len(b) == len(c)
+    for x, y, z in zip(a, b, c):
+        np.testing.assert_array_equal(x.view(np.uint32), y.view(np.uint32))
+        np.testing.assert_array_equal(x.view(np.uint32), z.view(np.uint32))
