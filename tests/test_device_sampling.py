@@ -205,6 +205,30 @@ def test_fullvocab_run_on_device_equals_host_loop(wd, kv, vocab, T, softcap):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("flags", [1, 2, 3])      # eager launches, one kernel per product, both
+@pytest.mark.parametrize("k", [6, 0])
+def test_runs_on_device_without_graph_and_without_the_persistent_kernel(flags, k):
+    """The draw kernels follow whatever produced the candidates / statistics: the same runs with the
+    step launched eagerly (HIPDEC_FLAG_NO_GRAPH) and as one kernel per product (HIPDEC_FLAG_NO_MEGA)."""
+    cfg = small_cfg(1000)
+    w = synth.make_weights(cfg, seed=29, std=0.08, round_bf16=True)
+    a = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.BF16, flags=flags)
+    b = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.BF16, flags=flags)
+    prompt = np.array([4, 8, 15, 16, 23, 42], np.uint32)
+    lg = a.prefill(prompt)
+    b.prefill(prompt)
+    first, steps, seed = int(np.argmax(lg)), 20, 77
+    if k > 0:
+        got, state = a.decode_topk_sampled_run(first, k, 0.9, seed, steps, softcap=1.5)
+        want, want_state = host_topk_loop(b, first, k, 0.9, seed, steps, 1.5)
+    else:
+        got, state = a.decode_fullvocab_sampled_run(first, 1.1, seed, steps)
+        want, want_state = host_fullvocab_loop(b, first, 1.1, 0.0, seed, steps)
+    np.testing.assert_array_equal(got, want)
+    assert state == want_state and a.len() == b.len() == 6 + steps
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("k,T,softcap", [(8, 0.8, 0.0), (0, 1.0, 0.0), (0, 0.9, 3.0), (6, 0.7, 2.0)])
 def test_batched_run_on_device_equals_per_step_batch_calls(k, T, softcap):
     cfg = small_cfg(1000)
