@@ -218,6 +218,15 @@ int hipdec_debug_step_profile(hipdec_model *m, uint32_t token, uint64_t *out, si
  * the known-size yardstick that hardware memory-traffic counters are scaled by. */
 int hipdec_debug_calibration_copy(size_t bytes, int reps);
 
+/* Verification: the draw kernels of the sampled runs on caller-supplied inputs (one row).  top-k: the
+ * per-block candidate lists vals/idxs[blocks * top_k] as hipdec_decode_token_topk_from_id returns them
+ * (engine/src/decode.rs:218-253 merge, engine/src/inference.rs:823-849 draw); full vocabulary: raw
+ * logits[vocab] with their block statistics maxes/sums[ceil(vocab / 256)] (inference.rs:851-921).
+ * *rng_state in and out, *out_token = the drawn token. */
+int hipdec_debug_sample_topk(const float *vals, const uint32_t *idxs, size_t blocks, uint32_t top_k, float temperature,
+                             float softcap, uint64_t *rng_state, uint32_t *out_token);
+int hipdec_debug_sample_fullvocab(const float *logits, size_t vocab, const float *maxes, const float *sums,
+                                  float temperature, float softcap, uint64_t *rng_state, uint32_t *out_token);
 /* 1 when this host's C library computes expf and tanhf as the on-device sampler reproduces them
  * (the probe the sampled runs consult), else 0. */
 int hipdec_debug_hostmath_probe(void);

@@ -940,6 +940,19 @@ int batch_sampled_run(hipdec_model *m, int variant, const uint32_t *tokens, uint
     return HIPDEC_OK;
 }
 
+// the draw kernels on caller-supplied inputs: one row, device buffers of exactly the sizes the kernels index
+struct DebugDraw {
+    std::vector<void *> bufs;
+    ~DebugDraw() { for (void *p : bufs) (void)hipFree(p); }
+    template <typename T> T *up(const T *host, size_t n, hipError_t *e) {
+        void *d = nullptr;
+        if (*e == hipSuccess) *e = hipMalloc(&d, n ? n * sizeof(T) : sizeof(T));
+        if (*e == hipSuccess) bufs.push_back(d);
+        if (*e == hipSuccess && n && host) *e = hipMemcpy(d, host, n * sizeof(T), hipMemcpyHostToDevice);
+        return (T *)d;
+    }
+};
+
 // a restated host function over consecutive bit patterns on the host, split over threads
 template <typename F> void hostmath_host_range(uint32_t first_bits, uint64_t count, int threads, F &&per_chunk) {
     if (threads < 1) threads = 1;
@@ -1570,6 +1583,56 @@ int hipdec_decode_fullvocab_sampled_run_batch(hipdec_model *m, const uint32_t *t
 }
 
 int hipdec_debug_hostmath_probe(void) { return hostmath_matches_libm() ? 1 : 0; }
+
+int hipdec_debug_sample_topk(const float *vals, const uint32_t *idxs, size_t blocks, uint32_t top_k, float temperature,
+                             float softcap, uint64_t *rng_state, uint32_t *out_token) {
+    if (!vals || !idxs || !rng_state || !out_token || blocks == 0 || blocks > SAMPLE_MAX_BLOCKS || top_k == 0 ||
+        top_k > HIPDEC_MAX_GPU_TOPK)
+        return HIPDEC_ERR_ARG;
+    hipError_t e = hipSuccess;
+    DebugDraw d;
+    const SampleParams sp{temperature, softcap, (int)top_k, 0, 1, 0u};
+    const uint32_t zero = 0;
+    float *dv = d.up(vals, blocks * top_k, &e);
+    uint32_t *di = d.up(idxs, blocks * top_k, &e);
+    SampleParams *dsp = d.up(&sp, 1, &e);
+    uint64_t *drng = d.up(rng_state, 1, &e);
+    uint32_t *dtok = d.up(&zero, 1, &e), *dring = d.up(&zero, 1, &e);
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(k_sample_topk, dim3(1), dim3(256), 0, nullptr, dv, di, (int)blocks, dsp, drng, dtok, dring,
+                           (BatchParams *)nullptr);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpy(out_token, dtok, 4, hipMemcpyDeviceToHost);
+    if (e == hipSuccess) e = hipMemcpy(rng_state, drng, 8, hipMemcpyDeviceToHost);
+    if (e != hipSuccess) { g_create_error = std::string("hipdec_debug_sample_topk: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+    return HIPDEC_OK;
+}
+
+int hipdec_debug_sample_fullvocab(const float *logits, size_t vocab, const float *maxes, const float *sums, float temperature,
+                                  float softcap, uint64_t *rng_state, uint32_t *out_token) {
+    const size_t blocks = (vocab + HIPDEC_HEAD_BLOCK - 1) / HIPDEC_HEAD_BLOCK;
+    if (!logits || !maxes || !sums || !rng_state || !out_token || vocab == 0 || blocks > SAMPLE_MAX_BLOCKS ||
+        !(temperature > 0.0f))
+        return HIPDEC_ERR_ARG;
+    hipError_t e = hipSuccess;
+    DebugDraw d;
+    const SampleParams sp{temperature, softcap, 1, 0, 1, 0u};
+    const uint32_t zero = 0;
+    float *dl = d.up(logits, vocab, &e), *dm = d.up(maxes, blocks, &e), *ds = d.up(sums, blocks, &e);
+    SampleParams *dsp = d.up(&sp, 1, &e);
+    uint64_t *drng = d.up(rng_state, 1, &e);
+    uint32_t *dtok = d.up(&zero, 1, &e), *dring = d.up(&zero, 1, &e);
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(k_sample_fullvocab, dim3(1), dim3(256), 0, nullptr, dl, (int)vocab, dm, ds, (int)blocks, dsp, drng,
+                           dtok, dring, (BatchParams *)nullptr);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpy(out_token, dtok, 4, hipMemcpyDeviceToHost);
+    if (e == hipSuccess) e = hipMemcpy(rng_state, drng, 8, hipMemcpyDeviceToHost);
+    if (e != hipSuccess) { g_create_error = std::string("hipdec_debug_sample_fullvocab: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+    return HIPDEC_OK;
+}
 
 int hipdec_debug_hostmath_eval(int fn, const float *in, float *out, size_t n, int on_device) {
     if (!in || !out || (fn != HOSTMATH_EXPF && fn != HOSTMATH_TANHF)) return HIPDEC_ERR_ARG;

@@ -31,7 +31,8 @@ EXPORTS = [
     "hipdec_decode_token_block_stats_from_ids_batch", "hipdec_materialize_current_logits_block_batch",
     "hipdec_decode_topk_sampled_run", "hipdec_decode_fullvocab_sampled_run", "hipdec_decode_topk_sampled_run_batch",
     "hipdec_decode_fullvocab_sampled_run_batch", "hipdec_debug_hostmath_eval", "hipdec_debug_hostmath_checksum",
-    "hipdec_debug_hostmath_count_mismatch", "hipdec_debug_hostmath_probe",
+    "hipdec_debug_hostmath_count_mismatch", "hipdec_debug_hostmath_probe", "hipdec_debug_sample_topk",
+    "hipdec_debug_sample_fullvocab",
 ]
 
 
@@ -147,6 +148,8 @@ def load_library(path=None):
     lib.hipdec_debug_hostmath_eval.argtypes = [C.c_int, fp, fp, C.c_size_t, C.c_int]
     lib.hipdec_debug_hostmath_checksum.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int, C.c_int, u64p]
     lib.hipdec_debug_hostmath_count_mismatch.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int, u64p]
+    lib.hipdec_debug_sample_topk.argtypes = [fp, u32p, C.c_size_t, C.c_uint32, C.c_float, C.c_float, u64p, u32p]
+    lib.hipdec_debug_sample_fullvocab.argtypes = [fp, C.c_size_t, fp, fp, C.c_float, C.c_float, u64p, u32p]
     if path is None:
         _LIB = lib
     return lib
@@ -182,6 +185,29 @@ def debug_hostmath_count_mismatch(fn, first_bits, count, host_threads=8):
     if rc != OK:
         raise HipDecodeError(rc, "hipdec_debug_hostmath_count_mismatch failed")
     return out.value
+
+
+def debug_sample_topk(vals, idxs, top_k, temperature, rng_state, softcap=0.0):
+    """The on-device merge + draw over per-block candidate lists [blocks * top_k]; returns (token, new state)."""
+    v = np.ascontiguousarray(vals, dtype=np.float32)
+    i = np.ascontiguousarray(idxs, dtype=np.uint32)
+    st, tok = C.c_uint64(int(rng_state) & 0xFFFFFFFFFFFFFFFF), C.c_uint32()
+    rc = load_library().hipdec_debug_sample_topk(_fptr(v), i.ctypes.data_as(C.POINTER(C.c_uint32)), v.size // top_k, top_k,
+                                                 temperature, softcap, C.byref(st), C.byref(tok))
+    if rc != OK:
+        raise HipDecodeError(rc, "hipdec_debug_sample_topk failed")
+    return tok.value, st.value
+
+
+def debug_sample_fullvocab(logits, maxes, sums, temperature, rng_state, softcap=0.0):
+    """The on-device block draw + token draw over raw logits and their block statistics; returns (token, new state)."""
+    lg, mx, sm = (np.ascontiguousarray(a, dtype=np.float32) for a in (logits, maxes, sums))
+    st, tok = C.c_uint64(int(rng_state) & 0xFFFFFFFFFFFFFFFF), C.c_uint32()
+    rc = load_library().hipdec_debug_sample_fullvocab(_fptr(lg), lg.size, _fptr(mx), _fptr(sm), temperature, softcap,
+                                                      C.byref(st), C.byref(tok))
+    if rc != OK:
+        raise HipDecodeError(rc, "hipdec_debug_sample_fullvocab failed")
+    return tok.value, st.value
 
 
 def calibration_copy(nbytes, reps=1):

@@ -104,6 +104,93 @@ def test_device_tanhf_equals_host_tanhf_for_every_float():
                                   hipdec.debug_hostmath(TANHF, x).view(np.uint32))
 
 
+# ------------------------------------------------------------------ the draw kernels on crafted inputs
+def oracle_topk_draw(vals, idxs, k, T, seed, softcap=0.0):
+    mv, mi = O.merge_topk(vals, idxs, k)
+    mv = host_softcap(mv, softcap)
+    rng = O.Rng(seed)
+    tok = int(O.lib().orc_sample_topk_candidates(O.PU(mi), O.P(mv), mi.size, T, rng.ref)) if mi.size else 0
+    if mi.size == 0:
+        tok = 0                                   # inference.rs:829-831: no candidate, token 0, no draw
+    return tok, rng.s.value
+
+
+@pytest.mark.gpu
+def test_topk_draw_kernel_on_crafted_candidate_lists():
+    """Ties across blocks (lower index first), padded lists (index u32::MAX, value -inf), +inf / NaN
+    values (dropped as the host merge drops them, decode.rs:229-231), fewer valid candidates than k,
+    no valid candidate at all, weights that underflow: device merge + draw == oracle merge + draw."""
+    MAXI = 0xFFFFFFFF
+    rng = np.random.default_rng(3)
+    cases = []
+    for blocks, k in ((4, 8), (128, 8), (300, 32), (1024, 3), (1, 1), (2, 32)):
+        vals = -np.sort(-rng.standard_normal((blocks, k)).astype(np.float32) * 3.0, axis=1)
+        idxs = (np.arange(blocks)[:, None] * 256 + np.argsort(rng.random((blocks, 256)), axis=1)[:, :k]).astype(np.uint32)
+        cases.append((vals.copy(), idxs.copy(), k))
+        # ties: the same value at the head of several blocks
+        v2, i2 = vals.copy(), idxs.copy()
+        v2[:, 0] = np.float32(9.5)
+        cases.append((v2, i2, k))
+        # padding and non-finite entries
+        v3, i3 = vals.copy(), idxs.copy()
+        if k > 1:
+            v3[::2, k // 2:] = -np.inf
+            i3[::2, k // 2:] = MAXI
+        v3[0, 0] = np.inf
+        if blocks > 1:
+            v3[1, 0] = np.nan
+        cases.append((v3, i3, k))
+        # hardly anything valid, and nothing valid
+        v4, i4 = np.full_like(vals, -np.inf), np.full_like(idxs, MAXI)
+        cases.append((v4.copy(), i4.copy(), k))
+        v4[blocks - 1, 0], i4[blocks - 1, 0] = 1.25, 7
+        cases.append((v4, i4, k))
+        # a spread wide enough for zero and subnormal weights
+        v5 = vals.copy()
+        v5[0, 0] = 120.0
+        cases.append((v5, idxs.copy(), k))
+    seed = 1
+    for n, (vals, idxs, k) in enumerate(cases):
+        for T, cap in ((0.8, 0.0), (0.05, 0.0), (1.7, 2.0), (0.0, 0.0)):
+            seed += 1
+            got = hipdec.debug_sample_topk(vals.ravel(), idxs.ravel(), k, T, seed, softcap=cap)
+            want = oracle_topk_draw(vals.ravel(), idxs.ravel(), k, T, seed, cap)
+            assert got == want, (n, k, T, cap, got, want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("vocab", [1000, 256, 257, 8192])
+def test_fullvocab_draw_kernel_on_crafted_logits(vocab):
+    """Block draw from the statistics, token draw inside the block (the last block may be short):
+    ordinary logits, blocks that are entirely -inf (weight 0), statistics with non-finite entries,
+    and the all-non-finite case with its fallbacks (block 0, last maximal element)."""
+    rng = np.random.default_rng(vocab)
+    B = (vocab + 255) // 256
+    base = (rng.standard_normal(vocab) * 4.0).astype(np.float32)
+    variants = [base]
+    v = base.copy(); v[:min(256, vocab)] = -np.inf; variants.append(v)          # a dead first block
+    v = base.copy(); v[vocab - 1] = 50.0; variants.append(v)                    # nearly all mass in the last row
+    v = np.full(vocab, -np.inf, np.float32); variants.append(v)                 # nothing finite anywhere
+    seed = 10
+    for n, lg in enumerate(variants):
+        for T in (1.0, 0.3, 2.5):
+            seed += 1
+            inv_t = float(np.float32(1.0) / np.float32(T))
+            with np.errstate(invalid="ignore"):
+                mx, sm = O.block_stats(lg, inv_t, 0.0)
+            for tweak in range(2):
+                if tweak and B > 1:
+                    mx, sm = mx.copy(), sm.copy()
+                    sm[B // 2] = np.nan                                          # ignored block (inference.rs:861-866)
+                    mx[0] = np.inf
+                got = hipdec.debug_sample_fullvocab(lg, mx, sm, T, seed)
+                r = O.Rng(seed)
+                blk = int(O.lib().orc_sample_block_from_stats(O.P(mx), O.P(sm), mx.size, r.ref))
+                bl = O.materialize_block(lg, blk, 0.0)
+                tok = int(O.lib().orc_sample_block_logits(blk * 256, O.P(bl), bl.size, T, r.ref))
+                assert got == (tok, r.s.value), (n, T, tweak, got, (tok, r.s.value))
+
+
 # ------------------------------------------------------------------ runs against the host loop
 def small_cfg(vocab=1000, seq=96):
     return Config.make(dim=256, hidden=640, heads=2, hd=128, seq=seq, nlayers=2, vocab=vocab)
