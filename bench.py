@@ -40,8 +40,11 @@ C3_SAMPLES, C3_TEMPERATURE, C3_TOP_K = 8, 0.8, 8
 
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, each
 # scaled by what the same counter reads for a plain copy of known size): measured separately with
-# rocprofv3 --pmc and recorded in profiles/k_mega_c2_600m_bf16_bs1.md; a benchmark run cannot collect it itself.
-MEASURED_TRAFFIC_BYTES = {"c2_600m_bf16_bs1": 1.509e9}
+# rocprofv3 --pmc and recorded in profiles/k_mega_c2_600m_bf16_bs1.md and profiles/k_mega_hbm_traffic_c1_c4_c5.md
+# (per step, i.e. the LM-head GEMV included where it is a launch of its own, at the KV length of the
+# profiled run); a benchmark run cannot collect it itself.
+MEASURED_TRAFFIC_BYTES = {"c1_tiny_fp32": 1.265e8, "c2_600m_bf16_bs1": 1.509e9, "c4_5b_bf16_bs1": 1.3868e10,
+                          "c5_5b_fp8_bs1": 7.123e9, "c5_5b_int4_bs1": 3.973e9}
 
 
 def run_c3(args, cfg, weights, n_prompt):
@@ -167,7 +170,8 @@ def run_c4_sampled(args, cfg, dev, kvdt, prompt_logits, n_prompt, gen_steps, pre
                              "frac": prefill_flops / (prefill_dev_ms * 1e-3) / mfma_peak},
         "device_ms_per_step": dev_ms / K,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "bytes_per_step": bytes_per_step},
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "bytes_per_step": bytes_per_step},
         "sampled_head": [int(t) for t in toks[:4]],
     }
 
