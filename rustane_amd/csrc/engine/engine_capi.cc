@@ -10,6 +10,7 @@
 #include "checkpoint.h"
 #include "inference.h"
 #include "jsonl_session.h"
+#include "session_cache.h"
 
 using namespace rustane;
 
@@ -185,6 +186,93 @@ void rs_session_result_copy(const rs_session *s, size_t i, int which, uint32_t *
 }
 double rs_session_result_decode_s(const rs_session *s, size_t i) { return s->last.results[i].decode_elapsed; }
 uint64_t rs_session_result_seed(const rs_session *s, size_t i) { return s->last.results[i].seed; }
+
+// ---- the server's session cache (bin/serve.rs:225-471)
+struct rs_session_cache {
+    ModelConfig cfg;
+    std::unique_ptr<SessionCache> c;
+    CacheGeneration last;
+};
+rs_session_cache *rs_session_cache_new(const rs_config *c, const rs_weights *w, float softcap, size_t max_entries,
+                                       uint32_t weight_dtype, uint32_t kv_dtype, uint32_t flags) {
+    SessionOptions o;
+    o.weight_dtype = (WeightDtype)weight_dtype;
+    o.kv_dtype = (KvDtype)kv_dtype;
+    o.flags = flags & 0xffu;
+    o.batch_samples = !(flags & 0x100u);
+    o.device_sampling = !(flags & 0x200u);
+    rs_session_cache *sc = new rs_session_cache();
+    sc->cfg = to_cfg(c);
+    sc->c.reset(new SessionCache(sc->cfg, w->w, softcap, max_entries, o));     // w must outlive the cache
+    return sc;
+}
+void rs_session_cache_free(rs_session_cache *sc) { delete sc; }
+uint64_t rs_session_cache_len(const rs_session_cache *sc) { return sc->c->len(); }
+uint64_t rs_session_cache_max_entries(const rs_session_cache *sc) { return sc->c->max_entries(); }
+uint64_t rs_session_cache_entry_prompt(const rs_session_cache *sc, size_t i, uint32_t *out, size_t cap) {
+    const std::vector<uint32_t> &p = sc->c->entry_prompt(i);
+    if (out && cap >= p.size()) memcpy(out, p.data(), p.size() * sizeof(uint32_t));
+    return p.size();
+}
+uint64_t rs_session_cache_normalize(const rs_session_cache *sc, const uint32_t *prompt, size_t n, uint32_t *out, size_t cap) {
+    const std::vector<uint32_t> p = sc->c->normalize_prompt_ids(std::vector<uint32_t>(prompt, prompt + n));
+    if (out && cap >= p.size()) memcpy(out, p.data(), p.size() * sizeof(uint32_t));
+    return p.size();
+}
+int64_t rs_session_cache_find(const rs_session_cache *sc, const uint32_t *prompt, size_t n, int longest_prefix) {
+    const std::vector<uint32_t> p(prompt, prompt + n);
+    return longest_prefix ? sc->c->find_longest_prefix(p) : sc->c->find_exact(p);
+}
+int64_t rs_session_cache_insert(rs_session_cache *sc, const uint32_t *prompt, size_t n, char *err, size_t errcap) {
+    std::string e;
+    const long idx = sc->c->insert(std::vector<uint32_t>(prompt, prompt + n), &e);
+    if (idx < 0) put_err(err, errcap, e);
+    return idx;
+}
+// cache_info: effective prompt tokens, prompt truncated (0/1), prompt tokens found in a cached session
+int rs_session_cache_generate(rs_session_cache *sc, const uint32_t *prompt, size_t n, const rs_request *r, int stream,
+                              uint64_t abort_after, rs_batch_info *info, uint64_t *cache_info, char *err, size_t errcap) {
+    GenerationRequest req;
+    req.decode_backend = r->backend == 1 ? DecodeBackendRequest::Naive
+                         : r->backend == 2 ? DecodeBackendRequest::Hip : DecodeBackendRequest::Auto;
+    req.steps = r->steps; req.temperature = r->temperature; req.top_k = r->top_k; req.samples = r->samples;
+    req.seed = r->seed;
+    const std::vector<uint32_t> p(prompt, prompt + n);
+    std::string e;
+    bool ok;
+    if (stream) {
+        StreamCallback cb = [&](uint32_t, const std::vector<uint32_t> &sampled, const std::vector<uint32_t> &) {
+            if (abort_after && sampled.size() >= abort_after) return std::string("callback asked to stop");
+            return std::string();
+        };
+        ok = sc->c->stream_generate(p, req, cb, &sc->last, &e);
+    } else {
+        ok = sc->c->generate(p, req, &sc->last, &e);
+    }
+    if (!ok) { put_err(err, errcap, e); return 1; }
+    const GenerationBatch &b = sc->last.batch;
+    info->mode = (uint32_t)b.decode_selection.mode;
+    info->fallback_reason = b.decode_selection.fallback_reason;
+    info->auto_reason = b.decode_selection.auto_reason;
+    info->base_prefill_s = b.base_prefill_elapsed; info->request_prefill_s = b.request_prefill_elapsed;
+    info->prefill_s = b.prefill_elapsed; info->total_decode_s = b.total_decode_elapsed;
+    info->avg_decode_s = b.avg_decode_elapsed; info->total_s = b.total_elapsed;
+    info->n_results = b.results.size();
+    cache_info[0] = sc->last.effective_prompt_tokens;
+    cache_info[1] = sc->last.prompt_truncated ? 1 : 0;
+    cache_info[2] = sc->last.cache_prefix_tokens;
+    return 0;
+}
+uint64_t rs_session_cache_result_len(const rs_session_cache *sc, size_t i, int which) {
+    const SampleResult &r = sc->last.batch.results[i];
+    return which ? r.generated.size() : r.sampled.size();
+}
+void rs_session_cache_result_copy(const rs_session_cache *sc, size_t i, int which, uint32_t *out) {
+    const SampleResult &r = sc->last.batch.results[i];
+    const std::vector<uint32_t> &v = which ? r.generated : r.sampled;
+    memcpy(out, v.data(), v.size() * sizeof(uint32_t));
+}
+uint64_t rs_session_cache_result_seed(const rs_session_cache *sc, size_t i) { return sc->last.batch.results[i].seed; }
 
 void rs_select_decode_mode(const rs_config *c, uint32_t requested, uint64_t ctx_len, uint64_t steps, uint32_t *mode,
                            const char **fallback_reason, const char **auto_reason) {

@@ -96,6 +96,29 @@ def lib():
         L.rs_session_result_decode_s.argtypes = [C.c_void_p, C.c_size_t]
         L.rs_session_result_seed.restype = C.c_uint64
         L.rs_session_result_seed.argtypes = [C.c_void_p, C.c_size_t]
+        L.rs_session_cache_new.restype = C.c_void_p
+        L.rs_session_cache_new.argtypes = [C.POINTER(RsConfig), C.c_void_p, C.c_float, C.c_size_t, C.c_uint32, C.c_uint32,
+                                           C.c_uint32]
+        L.rs_session_cache_free.argtypes = [C.c_void_p]
+        L.rs_session_cache_len.restype = C.c_uint64
+        L.rs_session_cache_len.argtypes = [C.c_void_p]
+        L.rs_session_cache_max_entries.restype = C.c_uint64
+        L.rs_session_cache_max_entries.argtypes = [C.c_void_p]
+        L.rs_session_cache_entry_prompt.restype = C.c_uint64
+        L.rs_session_cache_entry_prompt.argtypes = [C.c_void_p, C.c_size_t, u32p, C.c_size_t]
+        L.rs_session_cache_normalize.restype = C.c_uint64
+        L.rs_session_cache_normalize.argtypes = [C.c_void_p, u32p, C.c_size_t, u32p, C.c_size_t]
+        L.rs_session_cache_find.restype = C.c_int64
+        L.rs_session_cache_find.argtypes = [C.c_void_p, u32p, C.c_size_t, C.c_int]
+        L.rs_session_cache_insert.restype = C.c_int64
+        L.rs_session_cache_insert.argtypes = [C.c_void_p, u32p, C.c_size_t, C.c_char_p, C.c_size_t]
+        L.rs_session_cache_generate.argtypes = [C.c_void_p, u32p, C.c_size_t, C.POINTER(RsRequest), C.c_int, C.c_uint64,
+                                                C.POINTER(RsBatchInfo), u64p, C.c_char_p, C.c_size_t]
+        L.rs_session_cache_result_len.restype = C.c_uint64
+        L.rs_session_cache_result_len.argtypes = [C.c_void_p, C.c_size_t, C.c_int]
+        L.rs_session_cache_result_copy.argtypes = [C.c_void_p, C.c_size_t, C.c_int, u32p]
+        L.rs_session_cache_result_seed.restype = C.c_uint64
+        L.rs_session_cache_result_seed.argtypes = [C.c_void_p, C.c_size_t]
         L.rs_select_decode_mode.argtypes = [C.POINTER(RsConfig), C.c_uint32, C.c_uint64, C.c_uint64, u32p,
                                             C.POINTER(C.c_char_p), C.POINTER(C.c_char_p)]
         L.rs_parse_decode_backend.argtypes = [C.c_char_p, u32p]
@@ -272,6 +295,105 @@ class InferenceSession:
 
     def stream_count(self):
         return int(self._L.rs_session_stream_count(self._s))
+
+
+# ---------------------------------------------------------------- the server's session cache (bin/serve.rs:225-471)
+class CacheGeneration:
+    """serve.rs:241-246"""
+
+    def __init__(self, batch, effective_prompt_tokens, prompt_truncated, cache_prefix_tokens):
+        self.batch = batch
+        self.effective_prompt_tokens = effective_prompt_tokens
+        self.prompt_truncated = prompt_truncated
+        self.cache_prefix_tokens = cache_prefix_tokens
+
+
+class SessionCache:
+    """LRU set of sessions keyed by prompt: exact hit, longest cached prefix + suffix prefill, or a new session."""
+
+    def __init__(self, cfg, weights, softcap=0.0, max_entries=4, weight_dtype=0, kv_dtype=0, flags=0, ffn_activation=0):
+        L = lib()
+        self._L = L
+        self.cfg = cfg
+        rc = RsConfig.of(cfg, ffn_activation)
+        keep, ptrs = [], (fp * (9 * cfg.nlayers))()
+        for l, lw in enumerate(weights["layers"]):
+            for k, nme in enumerate(_TENSORS):
+                a = np.ascontiguousarray(lw[nme], np.float32)
+                keep.append(a)
+                ptrs[l * 9 + k] = a.ctypes.data_as(fp)
+        gf = np.ascontiguousarray(weights["gamma_final"], np.float32)
+        em = np.ascontiguousarray(weights["embed"], np.float32)
+        self._w = C.c_void_p(L.rs_weights_from_arrays(C.byref(rc), ptrs, gf.ctypes.data_as(fp), em.ctypes.data_as(fp)))
+        self._c = C.c_void_p(L.rs_session_cache_new(C.byref(rc), self._w, softcap, max_entries, int(weight_dtype),
+                                                    int(kv_dtype), flags))
+
+    def close(self):
+        if getattr(self, "_c", None) and self._c.value:
+            self._L.rs_session_cache_free(self._c)
+            self._c = C.c_void_p()
+        if getattr(self, "_w", None):
+            self._L.rs_weights_free(self._w)
+            self._w = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def __len__(self):
+        return int(self._L.rs_session_cache_len(self._c))
+
+    def max_entries(self):
+        return int(self._L.rs_session_cache_max_entries(self._c))
+
+    def entry_prompt(self, i):
+        n = self._L.rs_session_cache_entry_prompt(self._c, i, None, 0)
+        out = np.empty(max(n, 1), np.uint32)
+        self._L.rs_session_cache_entry_prompt(self._c, i, out.ctypes.data_as(u32p), out.size)
+        return out[:n]
+
+    def normalize_prompt_ids(self, prompt_ids):
+        p = np.ascontiguousarray(prompt_ids, np.uint32)
+        out = np.empty(max(p.size, 1), np.uint32)
+        n = self._L.rs_session_cache_normalize(self._c, p.ctypes.data_as(u32p), p.size, out.ctypes.data_as(u32p), out.size)
+        return out[:n]
+
+    def find_exact(self, prompt_ids):
+        p = np.ascontiguousarray(prompt_ids, np.uint32)
+        return int(self._L.rs_session_cache_find(self._c, p.ctypes.data_as(u32p), p.size, 0))
+
+    def find_longest_prefix(self, prompt_ids):
+        p = np.ascontiguousarray(prompt_ids, np.uint32)
+        return int(self._L.rs_session_cache_find(self._c, p.ctypes.data_as(u32p), p.size, 1))
+
+    def insert(self, prompt_ids):
+        p = np.ascontiguousarray(prompt_ids, np.uint32)
+        err = C.create_string_buffer(512)
+        idx = int(self._L.rs_session_cache_insert(self._c, p.ctypes.data_as(u32p), p.size, err, 512))
+        if idx < 0:
+            raise SessionError(err.value.decode())
+        return idx
+
+    def generate(self, prompt_ids, req, stream=False, abort_after=0):
+        p = np.ascontiguousarray(prompt_ids, np.uint32)
+        info, cinfo = RsBatchInfo(), (C.c_uint64 * 3)()
+        err = C.create_string_buffer(512)
+        rc = self._L.rs_session_cache_generate(self._c, p.ctypes.data_as(u32p), p.size, C.byref(req._c()), int(stream),
+                                               abort_after, C.byref(info), cinfo, err, 512)
+        if rc:
+            raise SessionError(err.value.decode())
+        results = []
+        for i in range(info.n_results):
+            arrs = []
+            for which in (0, 1):
+                n = self._L.rs_session_cache_result_len(self._c, i, which)
+                a = np.empty(max(n, 1), np.uint32)
+                self._L.rs_session_cache_result_copy(self._c, i, which, a.ctypes.data_as(u32p))
+                arrs.append(a[:n])
+            results.append(SampleResult(self._L.rs_session_cache_result_seed(self._c, i), arrs[1], arrs[0], 0.0))
+        return CacheGeneration(GenerationBatch(info, results), int(cinfo[0]), bool(cinfo[1]), int(cinfo[2]))
 
 
 # ---------------------------------------------------------------- RSTK checkpoints (crates/engine/src/checkpoint.rs)
