@@ -11,7 +11,10 @@ scale 0.05 with an fp32 KV cache (the stream keeps moving; with a bf16 cache a 1
 cached value flips its rounding and a stream this sensitive is not a stable known answer).
 
 Each vector holds the 32 largest prompt logits (index, value), the whole-vocabulary logit checksum
-and the greedy stream.  Run from the repository root:  python tests/golden/make_fullsize_vectors.py
+and the greedy stream; the fp32-cache case also holds two sampled streams of the reference's cached
+loop (crates/engine/src/inference.rs:586-625): top-k 8 at temperature 0.8 and full-vocabulary block
+sampling at temperature 1.0, each with its LCG seed.
+Run from the repository root:  python tests/golden/make_fullsize_vectors.py
 """
 import json
 import os
@@ -35,6 +38,9 @@ CASES = [
 ]
 
 
+SAMPLED = [(0.8, 8, 21), (1.0, 0, 22)]      # temperature, top_k, seed
+
+
 def main():
     for name, factory, std, wseed, pseed, n_prompt, steps, kv_bf16 in CASES:
         t0 = time.time()
@@ -46,6 +52,13 @@ def main():
         lg = lg[0]
         top = np.lexsort((np.arange(lg.size), -lg))[:32]
         sampled, _ = orc.run_cached_sample(ids, lg, steps)
+        streams = []
+        if not kv_bf16:
+            for temperature, top_k, seed in SAMPLED:
+                o2 = O.Oracle(cfg, w, kv_round_bf16=kv_bf16)
+                o2.forward_window(ids)
+                st, _ = o2.run_cached_sample(ids, lg, steps, temperature, top_k, seed=seed)
+                streams.append({"temperature": temperature, "top_k": top_k, "seed": seed, "stream": [int(t) for t in st]})
         out = {
             "workload": name, "config": factory, "weight_std": std, "weight_seed": wseed, "prompt_seed": pseed,
             "prompt_tokens": n_prompt, "weights": "bf16-rounded", "kv_cache": "bf16" if kv_bf16 else "f32",
@@ -56,6 +69,8 @@ def main():
             "logit_abs_max": float(np.abs(lg).max()),
             "greedy_stream": [int(t) for t in sampled],
         }
+        if streams:
+            out["sampled_streams"] = streams
         with open(os.path.join(HERE, name + ".json"), "w") as f:
             json.dump(out, f, indent=1)
         print(name, "done in %.1f s" % (time.time() - t0), out["greedy_stream"][:8], flush=True)

@@ -49,6 +49,11 @@ def test_oracle_reproduces_the_fullsize_vector():
     check_logits(g, lg[0], 1e-5)
     sampled, _ = orc.run_cached_sample(ids, lg[0], len(g["greedy_stream"]))
     assert [int(t) for t in sampled] == g["greedy_stream"]
+    for st in g["sampled_streams"]:
+        o2 = O.Oracle(cfg, w, kv_round_bf16=False)
+        o2.forward_window(ids)
+        got, _ = o2.run_cached_sample(ids, lg[0], len(st["stream"]), st["temperature"], st["top_k"], seed=st["seed"])
+        assert [int(t) for t in got] == st["stream"]
 
 
 @pytest.mark.gpu
@@ -68,3 +73,21 @@ def test_hip_backend_matches_the_fullsize_vector(name, prefill_steps):
     assert first == want[0]
     got = dev.decode_greedy_run(first, len(want) - 1)
     assert [int(t) for t in got] == want[1:]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("device_draws", [True, False])
+def test_session_reproduces_the_fullsize_sampled_streams(device_draws):
+    """The oracle's sampled streams of the 600M-class model (top-k 8 at T 0.8; full-vocabulary block
+    sampling at T 1.0) through the session API, with the draws on the device and with the draws on the
+    host (flag 0x200): the same tokens as the CPU restatement of the reference's loop."""
+    from rustane_amd import engine as E
+    g = load("c2_600m_bf16_std005_kvf32")
+    cfg, w, ids = model_inputs(g)
+    s = E.InferenceSession(cfg, w, ids, weight_dtype=1, kv_dtype=0, flags=0 if device_draws else 0x200)
+    for st in g["sampled_streams"]:
+        req = E.GenerationRequest(E.DecodeBackendRequest.HIP, steps=len(st["stream"]), temperature=st["temperature"],
+                                  top_k=st["top_k"], samples=1, seed=st["seed"])
+        got = s.generate(req)
+        assert got.decode_selection.mode == E.DecodeMode.KV_CACHE_HIP
+        assert [int(t) for t in got.results[0].sampled] == st["stream"], (st["top_k"], device_draws)
