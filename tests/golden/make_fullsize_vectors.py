@@ -13,7 +13,7 @@ cached value flips its rounding and a stream this sensitive is not a stable know
 Each vector holds the 32 largest prompt logits (index, value), the whole-vocabulary logit checksum
 and the greedy stream; the fp32-cache case also holds two sampled streams of the reference's cached
 loop (crates/engine/src/inference.rs:586-625): top-k 8 at temperature 0.8 and full-vocabulary block
-sampling at temperature 1.0, each with its LCG seed.
+sampling at temperature 1.0, each with its LCG seed, and the 8 streams of one 8-sample top-k request.
 Run from the repository root:  python tests/golden/make_fullsize_vectors.py
 """
 import json
@@ -39,6 +39,7 @@ CASES = [
 
 
 SAMPLED = [(0.8, 8, 21), (1.0, 0, 22)]      # temperature, top_k, seed
+BATCH = (0.8, 8, 30, 8, 12)                 # temperature, top_k, first seed, samples, steps
 
 
 def main():
@@ -71,6 +72,15 @@ def main():
         }
         if streams:
             out["sampled_streams"] = streams
+            # the multi-sample workload's shape: 8 samples of one request, seeds seed .. seed + 7 (inference.rs:256)
+            temperature, top_k, seed, samples, bsteps = BATCH
+            rows = []
+            for i in range(samples):
+                o2 = O.Oracle(cfg, w, kv_round_bf16=kv_bf16)
+                o2.forward_window(ids)
+                st, _ = o2.run_cached_sample(ids, lg, bsteps, temperature, top_k, seed=seed + i)
+                rows.append([int(t) for t in st])
+            out["batch_sampled"] = {"temperature": temperature, "top_k": top_k, "seed": seed, "samples": samples, "streams": rows}
         with open(os.path.join(HERE, name + ".json"), "w") as f:
             json.dump(out, f, indent=1)
         print(name, "done in %.1f s" % (time.time() - t0), out["greedy_stream"][:8], flush=True)

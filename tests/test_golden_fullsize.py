@@ -54,6 +54,11 @@ def test_oracle_reproduces_the_fullsize_vector():
         o2.forward_window(ids)
         got, _ = o2.run_cached_sample(ids, lg[0], len(st["stream"]), st["temperature"], st["top_k"], seed=st["seed"])
         assert [int(t) for t in got] == st["stream"]
+    b = g["batch_sampled"]                      # one of the 8 rows (each costs a window forward on the CPU)
+    o2 = O.Oracle(cfg, w, kv_round_bf16=False)
+    o2.forward_window(ids)
+    got, _ = o2.run_cached_sample(ids, lg[0], len(b["streams"][3]), b["temperature"], b["top_k"], seed=b["seed"] + 3)
+    assert [int(t) for t in got] == b["streams"][3]
 
 
 @pytest.mark.gpu
@@ -91,3 +96,22 @@ def test_session_reproduces_the_fullsize_sampled_streams(device_draws):
         got = s.generate(req)
         assert got.decode_selection.mode == E.DecodeMode.KV_CACHE_HIP
         assert [int(t) for t in got.results[0].sampled] == st["stream"], (st["top_k"], device_draws)
+
+
+@pytest.mark.gpu
+def test_session_reproduces_the_fullsize_eight_sample_request():
+    """The multi-sample workload's shape at full size: one request, 8 samples (seeds seed .. seed + 7),
+    top-k 8 at T 0.8, stepped together on the device with the draws on the device -- against the 8
+    streams the CPU restatement of the reference's loop gives one after the other."""
+    from rustane_amd import engine as E
+    g = load("c2_600m_bf16_std005_kvf32")
+    cfg, w, ids = model_inputs(g)
+    b = g["batch_sampled"]
+    s = E.InferenceSession(cfg, w, ids, weight_dtype=1, kv_dtype=0)
+    req = E.GenerationRequest(E.DecodeBackendRequest.HIP, steps=len(b["streams"][0]), temperature=b["temperature"],
+                              top_k=b["top_k"], samples=b["samples"], seed=b["seed"])
+    got = s.generate(req)
+    assert len(got.results) == b["samples"]
+    for i, (r, want) in enumerate(zip(got.results, b["streams"])):
+        assert r.seed == b["seed"] + i
+        assert [int(t) for t in r.sampled] == want, i
