@@ -118,11 +118,14 @@ template <> struct WS<WT_INT4> {
         const uint32_t u[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const uint32_t lo = u[i] ^ 0x88888888u, hi = lo >> 4;
+            const uint32_t lo = u[i] ^ 0x88888888u;
+            uint32_t hi = lo >> 4;
+            asm volatile("" : "+v"(hi));      // keeps `hi` a register of its own (otherwise its bytes are re-extracted from `lo` with one bit-field op each)
 #pragma unroll
             for (int b = 0; b < 4; ++b) {
-                f[8 * i + 2 * b] = __builtin_amdgcn_cvt_off_f32_i4((int)(lo >> (8 * b)));
-                f[8 * i + 2 * b + 1] = __builtin_amdgcn_cvt_off_f32_i4((int)(hi >> (8 * b)));
+                // (written as byte extractions so that they fold into the instruction's byte select)
+                f[8 * i + 2 * b] = __builtin_amdgcn_cvt_off_f32_i4(b == 0 ? (int)lo : (int)((lo >> (8 * b)) & 0xffu));
+                f[8 * i + 2 * b + 1] = __builtin_amdgcn_cvt_off_f32_i4((int)((hi >> (8 * b)) & 0xffu));
             }
         }
     }

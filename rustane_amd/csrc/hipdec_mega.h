@@ -110,6 +110,23 @@ __device__ __forceinline__ bool repoll16(mega_u4 &v, __amdgpu_buffer_rsrc_t r, i
     return true;
 }
 
+// Layout of a staged input vector in LDS.  The multiply reads it one 16-byte chunk per lane and
+// instruction, lane l holding piece l of a segment (a piece = the EPL inputs of one 16-byte weight
+// load).  With pieces of 64 or 128 bytes, eight neighbouring lanes of such a read meet in a quarter
+// or an eighth of the 32 LDS banks.  The chunks of a piece are therefore stored rotated by the
+// piece's index (counted in 128-byte bank rows), which spreads every read over all banks.
+// MEGA_SWZ_MIN_EPL: smallest piece (in inputs) stored this way.
+#ifndef MEGA_SWZ_MIN_EPL
+#define MEGA_SWZ_MIN_EPL 16
+#endif
+__device__ __forceinline__ int xs_chunk_pos(int chunk, int epl) {     // epl: 0 (plain order), 8, 16 or 32
+    if (epl == 0) return chunk;
+    const int cpl = epl == 32 ? 3 : epl == 16 ? 2 : 1;                // log2(chunks per piece)
+    const int piece = chunk >> cpl, c = chunk & ((1 << cpl) - 1);
+    return (piece << cpl) | ((c + (piece >> (3 - cpl))) & ((1 << cpl) - 1));
+}
+__device__ __forceinline__ int xs_pos(int i, int epl) { return (xs_chunk_pos(i >> 2, epl) << 2) | (i & 3); }
+
 // Polls n stamped floats (n % 4 == 0, src 16-byte aligned) with the polling waves (thread pt of
 // MEGA_PT) into dst (LDS): dst[i] = src[i] * (gamma ? gamma[i] : 1); elements with index in
 // [r0, r0 + nres) are also copied raw to res[i - r0].  Returns this thread's sum of squares of
@@ -120,6 +137,7 @@ __device__ __forceinline__ bool repoll16(mega_u4 &v, __amdgpu_buffer_rsrc_t r, i
 // return in order, so the polled values could not be seen before those anyway.
 #define MEGA_P0 (MEGA_POLLERS ? MEGA_SW * 64 : 0)   // first polling thread
 #define MEGA_PT (MEGA_THREADS - MEGA_P0)            // polling threads
+template <int SWZ_EPL>      // layout of dst: 0 plain order, else xs_chunk_pos(., SWZ_EPL)
 __device__ __noinline__ float mega_poll_vec(const float *src, int n, unsigned par, unsigned *abortf, float *dst,
                                             const float *gamma, float *res, int r0, int nres, int pt) {
     const int n4 = n >> 2;
@@ -152,7 +170,7 @@ __device__ __noinline__ float mega_poll_vec(const float *src, int n, unsigned pa
                 float4 o;
                 const float4 gm = make_float4(__uint_as_float(g[b].x), __uint_as_float(g[b].y), __uint_as_float(g[b].z), __uint_as_float(g[b].w));
                 o.x = x[0] * gm.x; o.y = x[1] * gm.y; o.z = x[2] * gm.z; o.w = x[3] * gm.w;
-                *(float4 *)(dst + 4 * i) = o;
+                *(float4 *)(dst + 4 * xs_chunk_pos(i, SWZ_EPL)) = o;
                 ss += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -214,6 +232,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     constexpr int SLOTS = MEGA_THREADS / LPR;    // cache rows per pass
     constexpr int PRE = 4;                       // passes prefetched
     constexpr int REC = HD + MEGA_PREC;          // floats per attention partial record
+    constexpr int XSWZ = EPL >= MEGA_SWZ_MIN_EPL ? EPL : 0;   // chunk rotation of the staged vectors (0: plain order)
     extern __shared__ __align__(16) float smem[];
     __shared__ MegaKind kinds[MK_KINDS];
     __shared__ float s_red[2][MEGA_WAVES];       // per-wave sums of squares, by phase parity
@@ -501,7 +520,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                 if (use_x_in) v = a.x_in[i];
                 else if (WT == WT_F32) v = ((const float *)a.embed)[(size_t)tok * D + i];
                 else v = bf16_to_f32(((const uint16_t *)a.embed)[(size_t)tok * D + i]);
-                xs[i] = v * g1[i];
+                xs[xs_pos(i, XSWZ)] = v * g1[i];
                 ss += v * v;
                 if (i >= wo_row0 && i < wo_row0 + wo_rows) xres_w[i - wo_row0] = v;
             }
@@ -514,7 +533,8 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             const unsigned pr = kind == MK_QKV ? (par ^ 1u) : kind == MK_HEAD ? ((ep_layer + (unsigned)L) & 1u) : par;
             const int nres = (kind == MK_QKV || kind == MK_W13) ? wo_rows : 0;
             if (polls) {
-                ss = mega_poll_vec(src, n, pr, abortf, dst, gm, xres_w, wo_row0, nres, pt);
+                if (XSWZ == 0 || kind == MK_WO) ss = mega_poll_vec<0>(src, n, pr, abortf, dst, gm, xres_w, wo_row0, nres, pt);
+                else ss = mega_poll_vec<XSWZ>(src, n, pr, abortf, dst, gm, xres_w, wo_row0, nres, pt);
                 if (ss < 0.0f) { ok = false; ss = 0.0f; }
             }
         }
@@ -542,7 +562,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                 const float *hp2 = stage + h * REC;
                 float A = 0.0f;
                 for (int s = 0; s < NS; ++s) A = fmaf(hp2[s * sstride + j], hp2[s * sstride + HD + 2], A);
-                xs[i] = A;
+                xs[xs_pos(i, XSWZ)] = A;
             }
             lds_barrier();
             mark();
@@ -582,9 +602,11 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                             const int piece = sg * MEGA_SEG_PIECES + j * 64 + lane;
                             if (piece < k.pieces) {
                                 float xv[EPL];
+                                constexpr int CPP = EPL / 4;                              // chunks per piece
+                                const int rot = XSWZ ? piece >> (EPL == 32 ? 0 : EPL == 16 ? 1 : 2) : 0;
 #pragma unroll
                                 for (int e = 0; e < EPL; e += 4) {
-                                    float4 tq = *(const float4 *)(xs + piece * EPL + e);
+                                    float4 tq = *(const float4 *)(xs + piece * EPL + 4 * ((e / 4 + rot) & (CPP - 1)));
                                     xv[e] = tq.x; xv[e + 1] = tq.y; xv[e + 2] = tq.z; xv[e + 3] = tq.w;
                                 }
                                 float w0[EPL], w1[EPL];
