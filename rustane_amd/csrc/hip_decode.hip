@@ -104,6 +104,7 @@ struct hipdec_model {
     MegaArgs mega{};
     int mega_grid = 0;
     size_t mega_lds = 0;
+    int mega_slots = 0;               // cache rows one attention pass of the persistent kernel covers
     unsigned *d_epochs = nullptr;
     void *xslab = nullptr;                            // uncached slab holding the exchange buffers (uncached_take)
     size_t xslab_cap = 0;
@@ -260,10 +261,17 @@ void launch_attn(hipdec_model *m, const DevLayer &L) {
 
 template <int WT> void launch_mega_t(hipdec_model *m, const MegaArgs &a) {
     dim3 grid(m->mega_grid), block(MEGA_THREADS);
-#define MEGA(KVB, HD) hipLaunchKernelGGL((k_mega<WT, KVB, HD>), grid, block, m->mega_lds, m->stream, a)
+#define MEGA2(KVB, HD, BP) hipLaunchKernelGGL((k_mega<WT, KVB, HD, BP>), grid, block, m->mega_lds, m->stream, a)
+    // the kernel's split count at this position (positions of steps enqueued behind this one are
+    // not known here: a run keeps the variant its first step chose; both give the same results)
+    const int n_att = (int)m->len + 1;
+    const int ns = std::max(1, std::min((n_att + m->mega_slots * MEGA_ATT_PRE - 1) / (m->mega_slots * MEGA_ATT_PRE), a.ns_max));
+    const bool bigpart = (size_t)a.heads * ns * (a.hd + MEGA_PREC) / 4 > (size_t)2048;
+#define MEGA(KVB, HD) do { if (bigpart) MEGA2(KVB, HD, 1); else MEGA2(KVB, HD, 0); } while (0)
     if (m->kvbf16) { if (m->cfg.hd == 64) MEGA(1, 64); else MEGA(1, 128); }
     else { if (m->cfg.hd == 64) MEGA(0, 64); else MEGA(0, 128); }
 #undef MEGA
+#undef MEGA2
 }
 void launch_mega(hipdec_model *m, int do_head, int advance) {
     MegaArgs a = m->mega;
@@ -280,8 +288,13 @@ void launch_mega(hipdec_model *m, int do_head, int advance) {
 template <int WT> hipError_t mega_set_lds_t(hipdec_model *m) {
     hipError_t e = hipSuccess;
 #define MEGA_ATTR(KVB, HD)                                                                                       \
-    e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mega<WT, KVB, HD>),                                 \
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)m->mega_lds)
+    do {                                                                                                          \
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mega<WT, KVB, HD, 0>),                          \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)m->mega_lds);                    \
+        if (e == hipSuccess)                                                                                      \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mega<WT, KVB, HD, 1>),                      \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)m->mega_lds);                \
+    } while (0)
     if (m->kvbf16) { if (m->cfg.hd == 64) MEGA_ATTR(1, 64); else MEGA_ATTR(1, 128); }
     else { if (m->cfg.hd == 64) MEGA_ATTR(0, 64); else MEGA_ATTR(0, 128); }
 #undef MEGA_ATTR
@@ -1115,6 +1128,7 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
         const size_t stage_floats = std::max((size_t)c.heads * (ns_max > 0 ? ns_max : 1) * (c.hd + MEGA_PREC),
                                              (size_t)slots * (c.hd + MEGA_PREC) + 3 * c.hd);
         m->mega_lds = fixed_lds + stage_floats * 4;
+        m->mega_slots = slots;
         const char *env = getenv("HIPDEC_NO_MEGA");
         bool want = !(m->opt.flags & HIPDEC_FLAG_NO_MEGA) && !(env && env[0] == '1');
         bool fits = ns_max >= 1 && m->mega_lds <= lds_cap && (V % 2 == 0) && (int)c.heads <= G &&

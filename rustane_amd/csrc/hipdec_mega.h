@@ -33,6 +33,7 @@
 #define MEGA_SW (MEGA_WAVES - MEGA_POLLERS)   // waves that stream weight rows
 #define MEGA_PREC 4             // attention partial record = HD + 4 floats (acc[HD], max, sum, 0, 0)
 #define MEGA_PROF_SLOTS 32      // timestamps per layer when profiling
+#define MEGA_ATT_PRE 4          // attention: cache-row passes a thread requests ahead
 #define MEGA_LPTR 12            // pointers per layer in the LDS copy of the layer table
 
 enum { MK_QKV = 0, MK_WO = 1, MK_W13 = 2, MK_W2 = 3, MK_HEAD = 4, MK_KINDS = 5 };
@@ -135,26 +136,30 @@ __device__ __forceinline__ int xs_pos(int i, int epl) { return (xs_chunk_pos(i >
 // to its use and the loads of one thread stop overlapping.  The price is that a called function
 // starts by waiting for every outstanding load of the wave, the requested weights included; loads
 // return in order, so the polled values could not be seen before those anyway.
+#ifndef MEGA_PART_NB
+#define MEGA_PART_NB 11
+#endif
 #define MEGA_P0 (MEGA_POLLERS ? MEGA_SW * 64 : 0)   // first polling thread
 #define MEGA_PT (MEGA_THREADS - MEGA_P0)            // polling threads
-template <int SWZ_EPL>      // layout of dst: 0 plain order, else xs_chunk_pos(., SWZ_EPL)
+// SWZ_EPL: layout of dst (0 plain order, else xs_chunk_pos(., SWZ_EPL)); NB: slots a thread requests
+// before it looks at the first one (every further group of NB costs another round trip).
+template <int SWZ_EPL, int NB = 2048 / MEGA_PT, bool GAMMA = true>     // GAMMA false: gamma is null, no registers for it
 __device__ __noinline__ float mega_poll_vec(const float *src, int n, unsigned par, unsigned *abortf, float *dst,
                                             const float *gamma, float *res, int r0, int nres, int pt) {
     const int n4 = n >> 2;
-    constexpr int NB = 2048 / MEGA_PT;
     const __amdgpu_buffer_rsrc_t r = make_rsrc(src, n * 4);
     const unsigned pm = par ? 0xffffffffu : 0u;
     float ss = 0.0f;
     bool good = true;
     for (int base = 0; base < n4 && good; base += MEGA_PT * NB) {
-        mega_u4 v[NB], g[NB];
+        mega_u4 v[NB], g[GAMMA ? NB : 1];
         // the norm weights do not depend on the exchange: request them first so that they are
         // there when the stamped values arrive
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             const int i = base + b * MEGA_PT + pt;
-            g[b] = mega_u4{0x3f800000u, 0x3f800000u, 0x3f800000u, 0x3f800000u};
-            if (gamma && i < n4) g[b] = *(const __attribute__((address_space(1))) mega_u4 *)(gamma + 4 * i);
+            g[GAMMA ? b : 0] = mega_u4{0x3f800000u, 0x3f800000u, 0x3f800000u, 0x3f800000u};
+            if (GAMMA && gamma && i < n4) g[GAMMA ? b : 0] = *(const __attribute__((address_space(1))) mega_u4 *)(gamma + 4 * i);
         }
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
@@ -168,7 +173,8 @@ __device__ __noinline__ float mega_poll_vec(const float *src, int n, unsigned pa
                 good = repoll16(v[b], r, i * 16, pm, abortf);
                 float x[4] = {__uint_as_float(v[b].x), __uint_as_float(v[b].y), __uint_as_float(v[b].z), __uint_as_float(v[b].w)};
                 float4 o;
-                const float4 gm = make_float4(__uint_as_float(g[b].x), __uint_as_float(g[b].y), __uint_as_float(g[b].z), __uint_as_float(g[b].w));
+                const mega_u4 gb = g[GAMMA ? b : 0];
+                const float4 gm = make_float4(__uint_as_float(gb.x), __uint_as_float(gb.y), __uint_as_float(gb.z), __uint_as_float(gb.w));
                 o.x = x[0] * gm.x; o.y = x[1] * gm.y; o.z = x[2] * gm.z; o.w = x[3] * gm.w;
                 *(float4 *)(dst + 4 * xs_chunk_pos(i, SWZ_EPL)) = o;
                 ss += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
@@ -223,14 +229,19 @@ template <int WT> struct MegaStage {
     uint32_t sc[2][2];       // int4 group scales (bf16 bits)
 };
 
-template <int WT, int KVBF16, int HD>
+// BIGPART: the attention partials (heads x splits records) are more than one request group of the
+// ordinary poll: wait for them with MEGA_PART_NB slots per thread in flight instead (5B: one round
+// trip instead of three, 2.79 -> 2.74 ms per token).  A template parameter, chosen by the host per
+// launch from heads x splits at the current position, because the poll routine's register footprint and a further call site shift the
+// code of the small models (600M: -0.4 % with the wide poll, -3 % with a run-time choice).
+template <int WT, int KVBF16, int HD, int BIGPART>
 __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     constexpr int EPL = WS<WT>::EPL;
     constexpr int KESZ = KVBF16 ? 2 : 4;
     constexpr int KEPL = 16 / KESZ;
     constexpr int LPR = HD / KEPL;               // lanes per cache row
     constexpr int SLOTS = MEGA_THREADS / LPR;    // cache rows per pass
-    constexpr int PRE = 4;                       // passes prefetched
+    constexpr int PRE = MEGA_ATT_PRE;            // passes prefetched
     constexpr int REC = HD + MEGA_PREC;          // floats per attention partial record
     constexpr int XSWZ = EPL >= MEGA_SWZ_MIN_EPL ? EPL : 0;   // chunk rotation of the staged vectors (0: plain order)
     extern __shared__ __align__(16) float smem[];
@@ -533,7 +544,8 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             const unsigned pr = kind == MK_QKV ? (par ^ 1u) : kind == MK_HEAD ? ((ep_layer + (unsigned)L) & 1u) : par;
             const int nres = (kind == MK_QKV || kind == MK_W13) ? wo_rows : 0;
             if (polls) {
-                if (XSWZ == 0 || kind == MK_WO) ss = mega_poll_vec<0>(src, n, pr, abortf, dst, gm, xres_w, wo_row0, nres, pt);
+                if (BIGPART && kind == MK_WO) ss = mega_poll_vec<0, MEGA_PART_NB, false>(src, n, pr, abortf, dst, gm, xres_w, wo_row0, nres, pt);
+                else if (XSWZ == 0 || kind == MK_WO) ss = mega_poll_vec<0>(src, n, pr, abortf, dst, gm, xres_w, wo_row0, nres, pt);
                 else ss = mega_poll_vec<XSWZ>(src, n, pr, abortf, dst, gm, xres_w, wo_row0, nres, pt);
                 if (ss < 0.0f) { ok = false; ss = 0.0f; }
             }
