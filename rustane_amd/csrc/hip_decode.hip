@@ -267,7 +267,8 @@ template <int WT> void launch_mega_t(hipdec_model *m, const MegaArgs &a) {
     const int n_att = (int)m->len + 1;
     const int ns = std::max(1, std::min((n_att + m->mega_slots * MEGA_ATT_PRE - 1) / (m->mega_slots * MEGA_ATT_PRE), a.ns_max));
     const bool bigpart = (size_t)a.heads * ns * (a.hd + MEGA_PREC) / 4 > (size_t)2048;
-#define MEGA(KVB, HD) do { if (bigpart) MEGA2(KVB, HD, 1); else MEGA2(KVB, HD, 0); } while (0)
+#define MEGA(KVB, HD) do { if (bigpart) MEGA2(KVB, HD, MEGA_VAR_BIGPART); else if (a.prof) MEGA2(KVB, HD, MEGA_VAR_STAMPS); \
+                            else MEGA2(KVB, HD, MEGA_VAR_PLAIN); } while (0)
     if (m->kvbf16) { if (m->cfg.hd == 64) MEGA(1, 64); else MEGA(1, 128); }
     else { if (m->cfg.hd == 64) MEGA(0, 64); else MEGA(0, 128); }
 #undef MEGA
@@ -289,10 +290,13 @@ template <int WT> hipError_t mega_set_lds_t(hipdec_model *m) {
     hipError_t e = hipSuccess;
 #define MEGA_ATTR(KVB, HD)                                                                                       \
     do {                                                                                                          \
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mega<WT, KVB, HD, 0>),                          \
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mega<WT, KVB, HD, MEGA_VAR_PLAIN>),             \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)m->mega_lds);                    \
         if (e == hipSuccess)                                                                                      \
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mega<WT, KVB, HD, 1>),                      \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mega<WT, KVB, HD, MEGA_VAR_STAMPS>),        \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)m->mega_lds);                \
+        if (e == hipSuccess)                                                                                      \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mega<WT, KVB, HD, MEGA_VAR_BIGPART>),       \
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)m->mega_lds);                \
     } while (0)
     if (m->kvbf16) { if (m->cfg.hd == 64) MEGA_ATTR(1, 64); else MEGA_ATTR(1, 128); }

@@ -234,8 +234,14 @@ template <int WT> struct MegaStage {
 // trip instead of three, 2.79 -> 2.74 ms per token).  A template parameter, chosen by the host per
 // launch from heads x splits at the current position, because the poll routine's register footprint and a further call site shift the
 // code of the small models (600M: -0.4 % with the wide poll, -3 % with a run-time choice).
-template <int WT, int KVBF16, int HD, int BIGPART>
+// VAR selects one of three builds of the kernel: MEGA_VAR_PLAIN (ordinary partials poll, no time
+// stamps: the stamp code, although never executed without a profile buffer, costs the 600M step 1.7 %
+// in registers and branches), MEGA_VAR_STAMPS (the same with time stamps, for the step profile) and
+// MEGA_VAR_BIGPART (wide partials poll; keeps the stamp code, which there costs nothing measurable).
+enum { MEGA_VAR_PLAIN = 0, MEGA_VAR_STAMPS = 1, MEGA_VAR_BIGPART = 2 };
+template <int WT, int KVBF16, int HD, int VAR>
 __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
+    constexpr int BIGPART = VAR == MEGA_VAR_BIGPART;
     constexpr int EPL = WS<WT>::EPL;
     constexpr int KESZ = KVBF16 ? 2 : 4;
     constexpr int KEPL = 16 / KESZ;
@@ -311,7 +317,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         }
     }
 
-    unsigned long long *prof = (a.prof && b == 0 && tid == 0) ? a.prof : nullptr;
+    unsigned long long *const prof = (VAR != MEGA_VAR_PLAIN && a.prof && b == 0 && tid == 0) ? a.prof : nullptr;
     int prof_n = 0;
     auto mark = [&]() { if (prof) prof[prof_n++] = wall_clock64(); };
 
