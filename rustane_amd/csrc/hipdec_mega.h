@@ -325,9 +325,9 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     // the local pairs w, w+MEGA_SW, ... and walks each pair's segments in order, so both the
     // streaming side and the prefetch side advance with two counters and no division.  The last
     // MEGA_POLLERS waves stream nothing: they wait for and stage the exchanged vectors.
-    const bool streams = wave < MEGA_SW;
+    const bool streams = MEGA_POLLERS ? wave < MEGA_SW : true;      // (without polling waves both are constants)
     const int pt = tid - MEGA_P0;                            // index among the polling threads (negative: not one)
-    const bool polls = pt >= 0;
+    const bool polls = MEGA_POLLERS ? pt >= 0 : true;
     auto n_mine = [&](int kind) {
         const int npl = kinds[kind].npl;
         return (streams && npl > wave) ? ((npl - wave + MEGA_SW - 1) / MEGA_SW) * kinds[kind].segs : 0;
