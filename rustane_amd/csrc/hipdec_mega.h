@@ -556,8 +556,8 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                 if (ss < 0.0f) { ok = false; ss = 0.0f; }
             }
         }
-        ss = wave_sum(ss);
-        if (lane == 0) s_red[ph & 1][wave] = ss;
+        ss = wave_sum_dpp(ss);                    // (no LDS round trips; total in lane 63)
+        if (lane == 63) s_red[ph & 1][wave] = ss;
         if (!ok) s_bad = 1;
         lds_barrier();
         if (s_bad) return;
