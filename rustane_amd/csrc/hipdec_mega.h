@@ -613,8 +613,8 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             lds_barrier();
             mark();
         }
-        float inv;
-        {
+        float inv = 0.0f;
+        if (kind != MK_WO && kind != MK_W2) {     // (the projections back into the residual stream take no norm)
             float t = 0.0f;
 #pragma unroll
             for (int w = 0; w < MEGA_WAVES; ++w) t += s_red[ph & 1][w];
