@@ -37,17 +37,23 @@ WORKLOADS = {
     "c3_600m_bf16_8samples": ("config_600m", "BF16", "BF16", 512, 256),
 }
 C3_SAMPLES, C3_TEMPERATURE, C3_TOP_K = 8, 0.8, 8
+ALL_CONFIG_ORDER = ["c1_tiny_fp32", "c2_600m_bf16_bs1", "c3_600m_bf16_8samples", "c4_5b_bf16_bs1", "c5_5b_fp8_bs1",
+                    "c5_5b_int4_bs1"]
+# timed steps of the short runs behind the all_configs entries (generated steps - 1 of the workload, capped)
+ALL_CONFIG_STEPS = {"c1_tiny_fp32": 31, "c2_600m_bf16_bs1": 255, "c3_600m_bf16_8samples": 64, "c4_5b_bf16_bs1": 32,
+                    "c5_5b_fp8_bs1": 64, "c5_5b_int4_bs1": 64}
 
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, each
 # scaled by what the same counter reads for a plain copy of known size): measured separately with
 # rocprofv3 --pmc and recorded in profiles/k_mega_c2_600m_bf16_bs1.md and profiles/k_mega_hbm_traffic_c1_c4_c5.md
 # (per step, i.e. the LM-head GEMV included where it is a launch of its own, at the KV length of the
 # profiled run); a benchmark run cannot collect it itself.
+TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries under profiles/, not measured in this run"
 MEASURED_TRAFFIC_BYTES = {"c1_tiny_fp32": 1.265e8, "c2_600m_bf16_bs1": 1.509e9, "c4_5b_bf16_bs1": 1.3868e10,
                           "c5_5b_fp8_bs1": 7.123e9, "c5_5b_int4_bs1": 3.973e9}
 
 
-def run_c3(args, cfg, weights, n_prompt):
+def run_c3(args, workload, cfg, weights, n_prompt):
     """Multi-sample workload through the session layer: a step is one pass of the weights that
     advances all 8 samples by one token (per-block top-k candidates, their merge and the reference's
     draw, all on the device: the whole request is one enqueued run); value = sampled tokens per
@@ -80,7 +86,7 @@ def run_c3(args, cfg, weights, n_prompt):
         "value": C3_SAMPLES * K / decode_s, "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": decode_s * 1e3 / K, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": args.workload, "prompt_tokens": n_prompt, "batch": C3_SAMPLES, "kv_dtype": "bf16",
+        "config": {"workload": workload, "prompt_tokens": n_prompt, "batch": C3_SAMPLES, "kv_dtype": "bf16",
                    "temperature": C3_TEMPERATURE, "top_k": C3_TOP_K, "params": cfg.param_count(), "mean_kv_len": mean_kv},
         "prefill_ms": s.prefill_elapsed() * 1e3, "request_wall_ms": wall * 1e3,
         "device_ms_per_step": dev_ms / K,
@@ -128,7 +134,7 @@ def cpu_baseline(cfg, weights, kv_bf16, prompt=None, gpu_stream=None, budget_s=2
     return out
 
 
-def run_c4_sampled(args, cfg, dev, kvdt, prompt_logits, n_prompt, gen_steps, prefill_dev_ms, prefill_wall_ms,
+def run_c4_sampled(args, workload, cfg, dev, kvdt, prompt_logits, n_prompt, gen_steps, prefill_dev_ms, prefill_wall_ms,
                    prefill_flops, mfma_peak):
     """The 5B workload as defined: full-vocabulary sampling at temperature 1.0 through the exact
     block-stats path (crates/engine/src/inference.rs:600-625) -- per token one decode step that
@@ -162,7 +168,7 @@ def run_c4_sampled(args, cfg, dev, kvdt, prompt_logits, n_prompt, gen_steps, pre
         "metric": "decode tok/s @600M bf16 bs1; % of HBM peak GB/s; prefill ms",
         "value": K / wall, "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": wall * 1e3 / K,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": args.workload, "prompt_tokens": n_prompt, "batch": 1, "kv_dtype": kvdt.name.lower(),
+        "config": {"workload": workload, "prompt_tokens": n_prompt, "batch": 1, "kv_dtype": kvdt.name.lower(),
                    "sampler": "full-vocab block stats, temperature 1.0", "params": cfg.param_count(), "mean_kv_len": mean_kv},
         "prefill_ms": prefill_dev_ms, "prefill_wall_ms": prefill_wall_ms,
         "prefill_roofline": {"bound": "mfma", "achieved": prefill_flops / (prefill_dev_ms * 1e-3) / 1e12,
@@ -170,38 +176,38 @@ def run_c4_sampled(args, cfg, dev, kvdt, prompt_logits, n_prompt, gen_steps, pre
                              "frac": prefill_flops / (prefill_dev_ms * 1e-3) / mfma_peak},
         "device_ms_per_step": dev_ms / K,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                     "bytes_per_step": bytes_per_step},
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(workload),
+                     "traffic_source": TRAFFIC_SOURCE, "bytes_per_step": bytes_per_step},
         "sampled_head": [int(t) for t in toks[:4]],
     }
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=255)
-    ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--workload", default="c2_600m_bf16_bs1", choices=sorted(WORKLOADS))
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--seed", type=int, default=1234)
-    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
-                    help="also run 4 launches of a plain copy kernel of this size (for scaling traffic counters)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this decode path runs on one GPU (no sharding); --gpus %d is not supported" % args.gpus,
-              file=sys.stderr)
-        sys.exit(2)
+_WEIGHTS = {}
 
+
+def cached_weights(cfg_name, cfg, seed, round_bf16):
+    """Synthetic N(0, 0.02) weights of a configuration; the latest set is kept, since consecutive
+    workloads share their model (the 5B fp32 master copy is 26 GB of host memory)."""
+    from rustane_amd import synth
+    key = (cfg_name, seed, round_bf16)
+    if key not in _WEIGHTS:
+        _WEIGHTS.clear()
+        _WEIGHTS[key] = synth.make_weights(cfg, seed=seed, std=0.02, round_bf16=round_bf16)
+    return _WEIGHTS[key]
+
+
+def measure(args, workload, with_cpu_baseline):
+    """One workload, start to finish: weights, prefill (reported), the timed decode region; returns the
+    result object (the keys of the benchmark line)."""
     from rustane_amd import synth
     from rustane_amd.hipdec import HipDecodeModel, KvDtype, WeightDtype
 
-    cfg_name, wdt, kvdt, n_prompt, gen_steps = WORKLOADS[args.workload]
+    cfg_name, wdt, kvdt, n_prompt, gen_steps = WORKLOADS[workload]
     cfg = getattr(synth, cfg_name)()
     wdt, kvdt = WeightDtype[wdt], KvDtype[kvdt]
-    weights = synth.make_weights(cfg, seed=args.seed, std=0.02, round_bf16=(wdt != WeightDtype.F32))
-    if args.workload == "c3_600m_bf16_8samples":
-        print(json.dumps(run_c3(args, cfg, weights, n_prompt)))
-        return
+    weights = cached_weights(cfg_name, cfg, args.seed, wdt != WeightDtype.F32)
+    if workload == "c3_600m_bf16_8samples":
+        return run_c3(args, workload, cfg, weights, n_prompt)
     dev = HipDecodeModel(cfg, weights, weight_dtype=wdt, kv_dtype=kvdt)
     prompt = synth.make_prompt(7, cfg.vocab, n_prompt)
 
@@ -222,10 +228,9 @@ def main():
 
     room = cfg.seq - n_prompt
     K, W = args.steps, args.warmup
-    if args.workload == "c4_5b_bf16_bs1":
-        print(json.dumps(run_c4_sampled(args, cfg, dev, kvdt, logits, n_prompt, gen_steps, prefill_dev_ms, prefill_wall_ms,
-                                        prefill_flops, mfma_peak)))
-        return
+    if workload == "c4_5b_bf16_bs1":
+        return run_c4_sampled(args, workload, cfg, dev, kvdt, logits, n_prompt, gen_steps, prefill_dev_ms, prefill_wall_ms,
+                              prefill_flops, mfma_peak)
     if W > 0:
         dev.decode_greedy_run(first, min(W, room))
     # timed region: exactly K greedy steps, in runs that restart at the end of the prompt so every
@@ -263,7 +268,7 @@ def main():
         "vs_baseline": None,
         "dtype": {"F32": "f32", "BF16": "bf16", "FP8_E4M3": "fp8_e4m3", "INT4_G128": "int4"}[wdt.name],
         "data": "synthetic",
-        "config": {"workload": args.workload, "prompt_tokens": n_prompt, "batch": 1, "kv_dtype": kvdt.name.lower(),
+        "config": {"workload": workload, "prompt_tokens": n_prompt, "batch": 1, "kv_dtype": kvdt.name.lower(),
                    "params": cfg.param_count(), "mean_kv_len": mean_kv},
         "prefill_ms": prefill_dev_ms,
         "prefill_wall_ms": prefill_wall_ms,
@@ -272,13 +277,61 @@ def main():
                              "frac": prefill_flops / (prefill_dev_ms * 1e-3) / mfma_peak},
         "device_ms_per_step": dev_ms / K,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                     "bytes_per_step": bytes_per_step},
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(workload),
+                     "traffic_source": TRAFFIC_SOURCE, "bytes_per_step": bytes_per_step},
     }
-    if not args.no_cpu_baseline:
-        replay = args.workload in ("c1_tiny_fp32", "c2_600m_bf16_bs1")      # the oracle can afford the prompt here
+    if with_cpu_baseline:
+        replay = workload in ("c1_tiny_fp32", "c2_600m_bf16_bs1")      # the oracle can afford the prompt here
         out["cpu_baseline"] = cpu_baseline(cfg, weights, kvdt == KvDtype.BF16, prompt if replay else None,
                                            gpu_stream if replay else None)
+    return out
+
+
+def summary(r):
+    """What the all_configs entry of the benchmark line keeps of a workload's result."""
+    e = {"dtype": r["dtype"], "kv_dtype": r["config"]["kv_dtype"], "batch": r["config"]["batch"],
+         "prompt_tokens": r["config"]["prompt_tokens"], "steps": r["steps"], "tok_s": r["value"],
+         "ms_per_step": r["ms_per_step"], "device_ms_per_step": r["device_ms_per_step"], "prefill_ms": r["prefill_ms"],
+         "roofline_frac": r["roofline"]["frac"], "achieved_GBps": r["roofline"]["achieved"],
+         "bytes_per_step": r["roofline"]["bytes_per_step"]}
+    if "prefill_roofline" in r:
+        e["prefill_mfma_frac"] = r["prefill_roofline"]["frac"]
+    if "mfma_roofline" in r:
+        e["step_mfma_frac"] = r["mfma_roofline"]["frac"]
+    return e
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=255)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--workload", default="c2_600m_bf16_bs1", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-all-configs", action="store_true",
+                    help="only the selected workload (by default the line also carries a short run of every other one)")
+    ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="also run 4 launches of a plain copy kernel of this size (for scaling traffic counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this decode path runs on one GPU (no sharding); --gpus %d is not supported" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    out = measure(args, args.workload, not args.no_cpu_baseline)
+    if not args.no_all_configs:
+        # the other workloads of the benchmark definition, each over its own prompt and a bounded
+        # number of steps, in the same process (their full-length runs: --workload NAME)
+        allc = {args.workload: summary(out)}
+        short = argparse.Namespace(**vars(args))
+        short.calibrate_copy = 0
+        for name in ALL_CONFIG_ORDER:
+            if name == args.workload:
+                continue
+            short.steps, short.warmup = ALL_CONFIG_STEPS[name], 4
+            allc[name] = summary(measure(short, name, False))
+        out["all_configs"] = allc
     print(json.dumps(out))
 
 

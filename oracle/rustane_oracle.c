@@ -22,7 +22,10 @@
  *                           test regime, layer.rs:706-709)
  *   heads (argmax/top-k/    integer-exact against a sort with (value desc, index asc); the
  *    merge/block stats)     log-sum-exp identity; materialised block == slice of full logits
- *   RNG / samplers          hand-computed LCG known answers; inverse-CDF brute force
+ *   RNG / samplers          hand-computed LCG known answers; inverse-CDF brute force; the block draw
+ *                           (orc_sample_block_from_stats) against its float64 definition on either side
+ *                           of every threshold, with overflowing / underflowing maxima, dead blocks and
+ *                           a short last block; block-then-token draws against softmax(logits / T)
  *   ANE fp16-internal numerics and MPS accumulation order: parity unpinned (not reachable
  *   off Apple hardware); this oracle is fp32, the precision of the reference's Metal path.
  */

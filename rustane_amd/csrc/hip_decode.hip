@@ -459,8 +459,23 @@ int sync_checked(hipdec_model *m) {
         unsigned flag = 0;
         HCHK(hipMemcpy(&flag, m->d_epochs + 2, 4, hipMemcpyDeviceToHost));
         if (flag) {
-            HCHK(hipMemset(m->d_epochs + 2, 0, 4));
-            m->err = "persistent decode kernel: a wait on another workgroup timed out (grid not co-resident?)";
+            // The aborted step left a mix of old and new stamps in the exchange buffers and did not
+            // advance the epochs, so a later step could accept its values: clear all of it and let
+            // every later step take the one-kernel-per-product path (its captured graphs hold
+            // persistent launches and go too).
+            const hipdec_config &c = m->cfg;
+            const MegaArgs &a = m->mega;
+            HCHK(hipMemset(a.QKV, 0, (size_t)(c.q_dim + 2 * c.kv_dim) * 4));
+            HCHK(hipMemset(a.PART, 0, (size_t)c.heads * a.ns_max * (c.hd + MEGA_PREC) * 4));
+            HCHK(hipMemset(a.X2, 0, (size_t)c.dim * 4));
+            HCHK(hipMemset(a.GATE, 0, (size_t)c.hidden * 4));
+            HCHK(hipMemset(a.CAND, 0, (size_t)m->mega_grid * 8));
+            HCHK(hipMemset(m->x_a, 0, (size_t)c.dim * 4));
+            HCHK(hipMemset(m->d_epochs, 0, 16));
+            m->mega_ok = false;
+            for (auto &g : m->graphs) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
+            m->err = "persistent decode kernel: a wait on another workgroup timed out (the grid needs the whole GPU to "
+                     "itself); later steps use one kernel per product";
             return HIPDEC_ERR_HIP;
         }
     }

@@ -18,7 +18,8 @@
 //    (a loop over phases with a small switch per phase), which keeps the loop body inside the
 //    instruction cache.
 //
-// All reductions run in a fixed order, so a step is bit-reproducible.  Every wait is bounded:
+// All reductions run in a fixed order and the stamp bit is cleared from every value before it is
+// used, so a step is bit-reproducible whatever the epoch.  Every wait is bounded:
 // a workgroup that spins too long raises an abort flag that makes every other workgroup leave too.
 #pragma once
 #include "hipdec_kernels.h"
@@ -171,7 +172,9 @@ __device__ __noinline__ float mega_poll_vec(const float *src, int n, unsigned pa
             const int i = base + b * MEGA_PT + pt;
             if (i < n4 && good) {
                 good = repoll16(v[b], r, i * 16, pm, abortf);
-                float x[4] = {__uint_as_float(v[b].x), __uint_as_float(v[b].y), __uint_as_float(v[b].z), __uint_as_float(v[b].w)};
+                // the stamp bit is cleared before use, so a value does not depend on the epoch it travelled in
+                float x[4] = {__uint_as_float(v[b].x & ~1u), __uint_as_float(v[b].y & ~1u), __uint_as_float(v[b].z & ~1u),
+                              __uint_as_float(v[b].w & ~1u)};
                 float4 o;
                 const mega_u4 gb = g[GAMMA ? b : 0];
                 const float4 gm = make_float4(__uint_as_float(gb.x), __uint_as_float(gb.y), __uint_as_float(gb.z), __uint_as_float(gb.w));
@@ -438,8 +441,8 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                     const __amdgpu_buffer_rsrc_t r = make_rsrc(src, HD * 4);
                     mega_u4 v = ld16_coherent(r, i4 * 16);
                     ok = repoll16(v, r, i4 * 16, par ? 0xffffffffu : 0u, abortf);
-                    dst[4 * i4] = __uint_as_float(v.x) * mul; dst[4 * i4 + 1] = __uint_as_float(v.y) * mul;
-                    dst[4 * i4 + 2] = __uint_as_float(v.z) * mul; dst[4 * i4 + 3] = __uint_as_float(v.w) * mul;
+                    dst[4 * i4] = __uint_as_float(v.x & ~1u) * mul; dst[4 * i4 + 1] = __uint_as_float(v.y & ~1u) * mul;
+                    dst[4 * i4 + 2] = __uint_as_float(v.z & ~1u) * mul; dst[4 * i4 + 3] = __uint_as_float(v.w & ~1u) * mul;
                 }
                 if (!streams) kv_first();
                 if (!ok) s_bad = 1;
@@ -526,6 +529,15 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             }
             lds_barrier();
             mark();
+        } else if (kind == MK_WO && b < a.heads * a.ns_max) {
+            // A split record that no workgroup fills at this position still takes this layer's stamp
+            // (an empty partial: maximum -1e30, sum 0).  Consumers only read the first NS splits, but the
+            // split count grows with the position: a record that had skipped launches would carry a
+            // stamp of unknown age, which a consumer could take for the current one.
+            if (tid < REC) {
+                float *pp = a.PART + (size_t)b * REC;              // record (split b / heads, head b % heads)
+                st_stamped(pp + tid, tid == HD ? -1e30f : 0.0f, par);
+            }
         }
 
         // ================= stage this phase's input vector in xs
@@ -704,6 +716,9 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                             cp[0] = eb; cp[1] = ob;
                             s0 = bf16_to_f32(eb); s1 = bf16_to_f32(ob);
                         } else {
+                            // the cache keeps what the exchange delivers (stamp bit cleared), so this step and
+                            // every later one attend over the same key / value bits
+                            s0 = __uint_as_float(__float_as_uint(s0) & ~1u); s1 = __uint_as_float(__float_as_uint(s1) & ~1u);
                             float *cp = (float *)cache + (size_t)pos * KV + rr;
                             cp[0] = s0; cp[1] = s1;
                         }

@@ -47,8 +47,9 @@ def test_oracle_reproduces_the_fullsize_vector():
     orc = O.Oracle(cfg, w, kv_round_bf16=(g["kv_cache"] == "bf16"))
     lg, _, _ = orc.forward_window(ids)
     check_logits(g, lg[0], 1e-5)
-    sampled, _ = orc.run_cached_sample(ids, lg[0], len(g["greedy_stream"]))
-    assert [int(t) for t in sampled] == g["greedy_stream"]
+    assert len(g["greedy_stream"]) == 256 and g["greedy_min_top2_gap"] > 50 * 1e-4 * g["logit_abs_max"]
+    sampled, _ = orc.run_cached_sample(ids, lg[0], 40)          # a prefix here; the GPU suite checks all 256 steps
+    assert [int(t) for t in sampled] == g["greedy_stream"][:40]
     for st in g["sampled_streams"]:
         o2 = O.Oracle(cfg, w, kv_round_bf16=False)
         o2.forward_window(ids)
@@ -59,6 +60,28 @@ def test_oracle_reproduces_the_fullsize_vector():
     o2.forward_window(ids)
     got, _ = o2.run_cached_sample(ids, lg[0], len(b["streams"][3]), b["temperature"], b["top_k"], seed=b["seed"] + 3)
     assert [int(t) for t in got] == b["streams"][3]
+
+
+def test_oracle_reproduces_the_multi_sample_fixture():
+    """tests/golden/c3_600m_bf16_8samples.npz (512-token prompt, bf16 cache, 8 samples): prompt logits,
+    and for one row the first steps' tokens and merged candidates, recomputed by the oracle."""
+    z = np.load(os.path.join(GOLDEN, "c3_600m_bf16_8samples.npz"))
+    meta = json.loads(str(z["meta"]))
+    cfg = getattr(synth, meta["config"])()
+    w = synth.make_weights(cfg, seed=meta["weight_seed"], std=meta["weight_std"], round_bf16=True)
+    ids = synth.make_prompt(meta["prompt_seed"], cfg.vocab, meta["prompt_tokens"])
+    assert z["streams"].shape == (meta["samples"], meta["steps"]) and meta["steps"] == 256 and meta["prompt_tokens"] == 512
+    orc = O.Oracle(cfg, w, kv_round_bf16=True)
+    lg, _, _ = orc.forward_window(ids)
+    assert np.abs(lg[0][z["top_logit_indices"]] - z["top_logit_values"]).max() <= 1e-5 * meta["logit_abs_max"]
+    row = 5
+    got, _ = orc.run_cached_sample(ids, lg[0], 6, meta["temperature"], meta["top_k"], seed=meta["seed"] + row)
+    assert [int(t) for t in got] == [int(t) for t in z["streams"][row, :6]]
+    orc.set_len(meta["prompt_tokens"])
+    raw = orc.decode_logits_from_id(int(z["streams"][row, 0]))
+    ci, cv = O.topk_candidates(raw, meta["top_k"], 0.0)
+    np.testing.assert_array_equal(ci, z["cand_ids"][row, 0])
+    np.testing.assert_array_equal(cv, z["cand_vals"][row, 0])
 
 
 @pytest.mark.gpu

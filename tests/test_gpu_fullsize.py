@@ -172,3 +172,60 @@ def test_5b_quantised_prefill_paths_and_chained_run_agree(w5b, wdt):
         tok = a.decode_token_argmax_from_id(tok)
         single.append(tok)
     np.testing.assert_array_equal(run, single)
+
+
+def test_5b_bf16_workload_prefill_paths_and_fullvocab_sampled_run(w5b):
+    """The 5B bf16 workload at its own shape: 1024-token prompt, bf16 cache, then full-vocabulary
+    sampling at temperature 1.0 through the block-statistics path.  (i) The chunked matrix-core
+    prefill against one token step per prompt row (the persistent kernel, which moves to its
+    many-partials build on the way: 32 heads x 3 splits from position 256).  (ii) 24 steps of
+    hipdec_decode_fullvocab_sampled_run against the reference's loop built from the per-step calls
+    and the oracle's two draws (inference.rs:600-625), tokens and RNG state."""
+    cfg, w = w5b
+    ids = synth.make_prompt(7, cfg.vocab, 1024)
+    a = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.BF16)
+    b = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.BF16)
+    c = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.BF16, flags=FLAG_PREFILL_STEPS)
+    la = a.prefill(ids)
+    np.testing.assert_array_equal(la, b.prefill(ids))
+    lc = c.prefill(ids)
+    assert rel_err(la, lc) < 2e-2          # the bf16 bound: cached values may round differently on the two paths
+    del c
+    first = int(np.argmax(la))
+    steps = 24
+    got, state = a.decode_fullvocab_sampled_run(first, 1.0, 1, steps)
+    rng, tok, want = O.Rng(1), first, []
+    for _ in range(steps):
+        mx, sm = b.decode_token_block_stats_from_id(tok, 1.0, 0.0)
+        blk = int(O.lib().orc_sample_block_from_stats(O.P(mx), O.P(sm), mx.size, rng.ref))
+        bl = b.materialize_current_logits_block(blk, 0.0)
+        tok = int(O.lib().orc_sample_block_logits(blk * 256, O.P(bl), bl.size, 1.0, rng.ref))
+        want.append(tok)
+    np.testing.assert_array_equal(got, np.array(want, np.uint32))
+    assert state == rng.s.value
+    assert a.len() == 1024 + steps
+
+
+@pytest.mark.parametrize("wdt", [WeightDtype.FP8_E4M3, WeightDtype.INT4_G128])
+def test_5b_quantised_workload_bf16_cache_512_token_prompt(w5b, wdt):
+    """The quantised 5B workloads at their own shape: 512-token prompt, bf16 cache, greedy decode.
+    Chunked prefill against token-step prefill (5e-2, the bound for 8-bit / 4-bit weights), a
+    device-chained greedy run against the same steps taken one call at a time, and the step logits of
+    the two models against each other."""
+    cfg, w = w5b
+    ids = synth.make_prompt(7, cfg.vocab, 512)
+    a = HipDecodeModel(cfg, w, weight_dtype=wdt, kv_dtype=KvDtype.BF16)
+    b = HipDecodeModel(cfg, w, weight_dtype=wdt, kv_dtype=KvDtype.BF16, flags=FLAG_PREFILL_STEPS)
+    la, lb = a.prefill(ids), b.prefill(ids)
+    assert rel_err(la, lb) < 5e-2
+    first = int(np.argmax(la))
+    run = a.decode_greedy_run(first, 16)
+    a.set_len(512)
+    tok, single = first, []
+    for _ in range(16):
+        tok = a.decode_token_argmax_from_id(tok)
+        single.append(tok)
+    np.testing.assert_array_equal(run, single)
+    a.set_len(512)
+    b.set_len(512)
+    assert rel_err(a.decode_logits_from_id(first), b.decode_logits_from_id(first)) < 5e-2

@@ -420,6 +420,91 @@ def test_sampler_degenerate_cases():
     assert L.orc_sample_block_from_stats(O.P(mx), O.P(sm), 2, r.ref) == 0          # inference.rs:861-863
 
 
+def _block_draw_expected(maxes, sums, u):
+    """The block inference.rs:851-891 must choose for the uniform u, in float64 from the definition:
+    weights exp(max_b - gmax) * sum_b (0 where max or sum is not finite or sum <= 0), inverse CDF in
+    block order.  Returns (block, margin) with margin = relative distance of u * total to the nearest
+    cumulative threshold (draws closer than float32 round-off to a threshold are not decidable)."""
+    mx, sm = np.asarray(maxes, np.float64), np.asarray(sums, np.float64)
+    fin = np.isfinite(mx)
+    g = mx[fin].max()
+    ok = fin & np.isfinite(sm) & (sm > 0)
+    w = np.where(ok, np.exp(np.where(ok, mx, g) - g) * np.where(ok, sm, 0.0), 0.0)
+    cum = np.cumsum(w)
+    x = float(u) * cum[-1]
+    blk = int(np.searchsorted(cum, x, side="left"))
+    live = cum[np.concatenate([[True], np.diff(cum) > 0])]
+    return min(blk, len(w) - 1), float(np.abs(live - x).min() / cum[-1])
+
+
+@pytest.mark.parametrize("case", ["plain", "huge_maxes", "tiny_maxes", "dead_blocks", "short_last_block"])
+def test_block_draw_from_stats_inverse_cdf_against_float64(case):
+    """orc_sample_block_from_stats (inference.rs:851-891) against the float64 definition, for uniforms on
+    either side of every threshold.  The cases are chosen so that a dropped `* sum_b`, a dropped
+    `- gmax` (overflow / underflow of exp), a block order other than 0..B-1 or a weight for a block
+    with non-finite statistics each pick a different block."""
+    if case == "plain":
+        mx, sm = [1.0, 0.2, 1.5, -0.3, 0.9, 1.4], [40.0, 200.0, 3.0, 120.0, 77.0, 9.0]
+    elif case == "huge_maxes":           # exp(max) overflows float32 without the shift by gmax
+        mx, sm = [95.0, 99.5, 97.0, 100.0, 98.0], [30.0, 2.0, 50.0, 1.5, 20.0]
+    elif case == "tiny_maxes":           # exp(max) underflows to 0 without the shift
+        mx, sm = [-200.0, -201.0, -199.5, -203.0], [10.0, 60.0, 5.0, 250.0]
+    elif case == "dead_blocks":          # non-finite max / sum and sum <= 0 carry no weight (inference.rs:861-866)
+        mx = [0.5, np.inf, 1.0, -np.inf, 0.8, 0.1, np.nan, 0.7, 0.3]
+        sm = [12.0, 5.0, np.nan, 9.0, 0.0, 30.0, 4.0, -25.0, 8.0]
+    else:                                # a last block of few rows: its sum is what keeps it rare
+        mx, sm = [2.0, 2.1, 1.9, 2.05], [180.0, 190.0, 170.0, 3.0]
+    mxa, sma = O.f32(mx), O.f32(sm)
+    hit = np.zeros(len(mx), int)
+    decided = 0
+    for seed in range(3000):
+        u = O.Rng(seed).next_f32()
+        want, margin = _block_draw_expected(mxa, sma, u)
+        if margin < 1e-5:
+            continue
+        r = O.Rng(seed)
+        got = L.orc_sample_block_from_stats(O.P(mxa), O.P(sma), len(mx), r.ref)
+        assert got == want, (case, seed, u, got, want)
+        assert r.s.value == (seed * 6364136223846793005 + 1442695040888963407) % (1 << 64)     # exactly one draw
+        hit[got] += 1
+        decided += 1
+    assert decided > 2900
+    mx64, sm64 = np.asarray(mxa, np.float64), np.asarray(sma, np.float64)
+    live = np.isfinite(mx64) & np.isfinite(sm64) & (sm64 > 0)
+    assert np.all(hit[live] > 0) and np.all(hit[~live] == 0)        # both sides of every threshold were visited
+
+
+def test_block_then_token_sampling_reproduces_the_softmax_distribution():
+    """The two draws of the cached full-vocabulary path (block from the statistics, inference.rs:851-891,
+    then the token inside the block, :893-921) must together sample softmax(logits / T): block marginals
+    and token probabilities over 40 000 draws at V = 777 (three full blocks and one of 9 rows)."""
+    rng = np.random.default_rng(21)
+    V, T = 777, 0.8
+    logits = (rng.standard_normal(V) * 1.5).astype(np.float32)
+    logits[770:] += 2.0                                    # the short block is not negligible
+    p = np.exp((logits.astype(np.float64) - logits.max()) / T); p /= p.sum()
+    inv_t = float(np.float32(1.0) / np.float32(T))
+    mx, sm = O.block_stats(logits, inv_t, 0.0)
+    B = len(mx)
+    r = O.Rng(2024)
+    N = 40000
+    counts = np.zeros(V)
+    for _ in range(N):
+        b = L.orc_sample_block_from_stats(O.P(mx), O.P(sm), B, r.ref)
+        blk = O.materialize_block(logits, b, 0.0)
+        counts[L.orc_sample_block_logits(b * 256, O.P(blk), blk.size, T, r.ref)] += 1
+    pb = np.array([p[b * 256:(b + 1) * 256].sum() for b in range(B)])
+    cb = np.array([counts[b * 256:(b + 1) * 256].sum() for b in range(B)])
+    assert np.abs(cb / N - pb).max() < 4.0 * np.sqrt(0.25 / N)                 # 4 sigma of a block frequency
+    # token level: chi-square of the observed counts against softmax (cells with expectation >= 5)
+    e = p * N
+    cells = e >= 5.0
+    chi2 = float((((counts - e) ** 2) / e)[cells].sum()) + (counts[~cells].sum() - e[~cells].sum()) ** 2 / max(e[~cells].sum(), 1.0)
+    dof = int(cells.sum())
+    assert chi2 < dof + 5.0 * np.sqrt(2.0 * dof), (chi2, dof)
+    assert np.abs(counts / N - p).max() < 0.01
+
+
 def test_fullvocab_cached_path_draws_twice_per_token():
     # inference.rs:602-617 (block, then token inside the block) against :786-788 (one draw)
     cfg = tiny_cfg(vocab=320)
