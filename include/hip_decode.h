@@ -227,6 +227,19 @@ int hipdec_debug_sample_topk(const float *vals, const uint32_t *idxs, size_t blo
                              float softcap, uint64_t *rng_state, uint32_t *out_token);
 int hipdec_debug_sample_fullvocab(const float *logits, size_t vocab, const float *maxes, const float *sums,
                                   float temperature, float softcap, uint64_t *rng_state, uint32_t *out_token);
+/* The full-vocabulary draw for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.
+ * Same draw as hipdec_debug_sample_fullvocab (block from the statistics, then the token inside the
+ * block; engine/src/inference.rs:851-921 on the device), but every buffer is DEVICE memory of the
+ * current device -- d_logits[vocab] raw logits, d_maxes/d_sums[ceil(vocab / 256)], *d_rng_state in and
+ * out, *d_out_token out -- and the two kernels are enqueued on `stream` (a hipStream_t, NULL = the
+ * default stream) without waiting for them.  Calls no hipMalloc / hipFree: the kernels' run state lives
+ * in a 256-byte array the library holds on every GPU it runs on, reset by the call itself.  Every call
+ * on a GPU shares that array, so calls that overlap on one GPU (two streams, two threads) race.
+ * vocab <= 262144 (1024 blocks), else HIPDEC_ERR_ARG; errors are reported through hipdec_last_error(NULL). */
+int hipdec_sample_fullvocab_noalloc(const float *d_logits, size_t vocab, const float *d_maxes, const float *d_sums,
+                                    float temperature, float softcap, uint64_t *d_rng_state, uint32_t *d_out_token,
+                                    void *stream);
 /* 1 when this host's C library computes expf and tanhf as the on-device sampler reproduces them
  * (the probe the sampled runs consult), else 0. */
 int hipdec_debug_hostmath_probe(void);

@@ -1667,6 +1667,64 @@ int hipdec_debug_sample_fullvocab(const float *logits, size_t vocab, const float
     return HIPDEC_OK;
 }
 
+// ---- the full-vocabulary draw for callers that may not allocate (see include/hip_decode.h)
+// Run state of the draw kernel (SampleParams with its arrival counter at byte 0, the one-slot token
+// ring at byte 64).  Every GPU the library runs on holds its own copy of this array until the process
+// ends; host code reaches it only through the address hipGetSymbolAddress returns for the current device.
+#define NOALLOC_SCRATCH_BYTES 256
+#define NOALLOC_MAX_VOCAB ((size_t)SAMPLE_MAX_BLOCKS * HIPDEC_HEAD_BLOCK)
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
+// (a kernel, not hipMemsetAsync: the call may be recorded into a graph)
+__global__ void k_noalloc_reset(SampleParams *ss, uint32_t *ring, float temperature, float softcap) {
+    ss->temperature = temperature; ss->softcap = softcap; ss->top_k = 1; ss->step = 0; ss->ring_cap = 1; ss->done = 0u;
+    *ring = 0u;
+}
+
+static std::mutex g_scratch_mu;
+static void *g_scratch_ptr[64] = {};      // by device ordinal
+
+int hipdec_sample_fullvocab_noalloc(const float *d_logits, size_t vocab, const float *d_maxes, const float *d_sums,
+                                    float temperature, float softcap, uint64_t *d_rng_state, uint32_t *d_out_token,
+                                    void *stream) {
+    if (!d_logits || !d_maxes || !d_sums || !d_rng_state || !d_out_token || vocab == 0 || !(temperature > 0.0f)) {
+        g_create_error = "hipdec_sample_fullvocab_noalloc: null buffer, empty vocabulary or non-positive temperature";
+        return HIPDEC_ERR_ARG;
+    }
+    if (vocab > NOALLOC_MAX_VOCAB) {
+        g_create_error = "hipdec_sample_fullvocab_noalloc: vocab exceeds the 262144 rows (1024 blocks of 256) this entry point serves";
+        return HIPDEC_ERR_ARG;
+    }
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    void *base = nullptr;
+    if (e == hipSuccess && (dev < 0 || dev >= 64)) {
+        g_create_error = "hipdec_sample_fullvocab_noalloc: device ordinal out of range";
+        return HIPDEC_ERR_UNSUPPORTED;
+    }
+    if (e == hipSuccess) {
+        std::lock_guard<std::mutex> lock(g_scratch_mu);
+        if (!g_scratch_ptr[dev]) {
+            void *p = nullptr;
+            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));      // this device's copy of the array
+            if (e == hipSuccess) g_scratch_ptr[dev] = p;
+        }
+        base = g_scratch_ptr[dev];
+    }
+    if (e == hipSuccess) {
+        SampleParams *ss = (SampleParams *)base;
+        uint32_t *ring = (uint32_t *)((unsigned char *)base + 64);
+        const int blocks = (int)((vocab + HIPDEC_HEAD_BLOCK - 1) / HIPDEC_HEAD_BLOCK);
+        hipStream_t s = (hipStream_t)stream;
+        hipLaunchKernelGGL(k_noalloc_reset, dim3(1), dim3(1), 0, s, ss, ring, temperature, softcap);
+        hipLaunchKernelGGL(k_sample_fullvocab, dim3(1), dim3(256), 0, s, d_logits, (int)vocab, d_maxes, d_sums, blocks, ss,
+                           d_rng_state, d_out_token, ring, (BatchParams *)nullptr);
+        e = hipGetLastError();
+    }
+    if (e != hipSuccess) { g_create_error = std::string("hipdec_sample_fullvocab_noalloc: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+    return HIPDEC_OK;
+}
+
 int hipdec_debug_hostmath_eval(int fn, const float *in, float *out, size_t n, int on_device) {
     if (!in || !out || (fn != HOSTMATH_EXPF && fn != HOSTMATH_TANHF)) return HIPDEC_ERR_ARG;
     if (!on_device) {

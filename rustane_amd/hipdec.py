@@ -32,7 +32,7 @@ EXPORTS = [
     "hipdec_decode_topk_sampled_run", "hipdec_decode_fullvocab_sampled_run", "hipdec_decode_topk_sampled_run_batch",
     "hipdec_decode_fullvocab_sampled_run_batch", "hipdec_debug_hostmath_eval", "hipdec_debug_hostmath_checksum",
     "hipdec_debug_hostmath_count_mismatch", "hipdec_debug_hostmath_probe", "hipdec_debug_sample_topk",
-    "hipdec_debug_sample_fullvocab",
+    "hipdec_debug_sample_fullvocab", "hipdec_sample_fullvocab_noalloc",
 ]
 
 
@@ -150,6 +150,8 @@ def load_library(path=None):
     lib.hipdec_debug_hostmath_count_mismatch.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int, u64p]
     lib.hipdec_debug_sample_topk.argtypes = [fp, u32p, C.c_size_t, C.c_uint32, C.c_float, C.c_float, u64p, u32p]
     lib.hipdec_debug_sample_fullvocab.argtypes = [fp, C.c_size_t, fp, fp, C.c_float, C.c_float, u64p, u32p]
+    lib.hipdec_sample_fullvocab_noalloc.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_float, C.c_float,
+                                                    C.c_void_p, C.c_void_p, C.c_void_p]
     if path is None:
         _LIB = lib
     return lib
@@ -208,6 +210,16 @@ def debug_sample_fullvocab(logits, maxes, sums, temperature, rng_state, softcap=
     if rc != OK:
         raise HipDecodeError(rc, "hipdec_debug_sample_fullvocab failed")
     return tok.value, st.value
+
+
+def sample_fullvocab_noalloc(d_logits, vocab, d_maxes, d_sums, temperature, d_rng_state, d_out_token, softcap=0.0,
+                             stream=None):
+    """hipdec_sample_fullvocab_noalloc: every pointer is a device address (an int); enqueues on `stream`
+    (a hipStream_t as an int, None = default stream) and returns without waiting."""
+    rc = load_library().hipdec_sample_fullvocab_noalloc(d_logits, vocab, d_maxes, d_sums, temperature, softcap,
+                                                        d_rng_state, d_out_token, stream)
+    if rc != OK:
+        raise HipDecodeError(rc, (load_library().hipdec_last_error(None) or b"").decode())
 
 
 def calibration_copy(nbytes, reps=1):
