@@ -26,12 +26,12 @@
 
 #define MEGA_THREADS 512
 #define MEGA_WAVES 8
-#define MEGA_DEPTH 4            // tasks per round (16 loads of 16 bytes in flight per lane)
+#define MEGA_DEPTH 4            // tasks per round of the even phases (16 loads of 16 bytes in flight per lane)
+#ifndef MEGA_DEPTH_B
+#define MEGA_DEPTH_B 2          // tasks per round of the odd phases (wo, w2: few rows per workgroup)
+#endif
 #define MEGA_SEG_PIECES 128     // 16-byte pieces of one row per task: 2 per lane
 #define MEGA_SPIN_LIMIT (1u << 22)
-#define MEGA_POLLERS 0          // waves that only wait for and stage exchanged vectors (they request no weights,
-                                // so their loads are never queued behind a round of weight loads)
-#define MEGA_SW (MEGA_WAVES - MEGA_POLLERS)   // waves that stream weight rows
 #define MEGA_PREC 4             // attention partial record = HD + 4 floats (acc[HD], max, sum, 0, 0)
 #define MEGA_PROF_SLOTS 32      // timestamps per layer when profiling
 #define MEGA_ATT_PRE 4          // attention: cache-row passes a thread requests ahead
@@ -140,8 +140,7 @@ __device__ __forceinline__ int xs_pos(int i, int epl) { return (xs_chunk_pos(i >
 #ifndef MEGA_PART_NB
 #define MEGA_PART_NB 11
 #endif
-#define MEGA_P0 (MEGA_POLLERS ? MEGA_SW * 64 : 0)   // first polling thread
-#define MEGA_PT (MEGA_THREADS - MEGA_P0)            // polling threads
+#define MEGA_PT MEGA_THREADS                        // polling threads
 // SWZ_EPL: layout of dst (0 plain order, else xs_chunk_pos(., SWZ_EPL)); NB: slots a thread requests
 // before it looks at the first one (every further group of NB costs another round trip).
 template <int SWZ_EPL, int NB = 2048 / MEGA_PT, bool GAMMA = true>     // GAMMA false: gamma is null, no registers for it
@@ -324,59 +323,123 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     int prof_n = 0;
     auto mark = [&]() { if (prof) prof[prof_n++] = wall_clock64(); };
 
-    // Tasks of a GEMV phase: (row pair, segment of MEGA_SEG_PIECES pieces).  Streaming wave w owns
-    // the local pairs w, w+MEGA_SW, ... and walks each pair's segments in order, so both the
-    // streaming side and the prefetch side advance with two counters and no division.  The last
-    // MEGA_POLLERS waves stream nothing: they wait for and stage the exchanged vectors.
-    const bool streams = MEGA_POLLERS ? wave < MEGA_SW : true;      // (without polling waves both are constants)
-    const int pt = tid - MEGA_P0;                            // index among the polling threads (negative: not one)
-    const bool polls = MEGA_POLLERS ? pt >= 0 : true;
-    auto n_mine = [&](int kind) {
+    // The GEMV phases run in the order l*4 + kind (qkv, wo, w13, w2 of layer l), then the head.  Even
+    // phases (qkv, w13, head: many rows, reduction over D) and odd phases (wo, w2: D rows shared by all
+    // workgroups, long reductions) alternate, and each kind of phase has a register set of its own for
+    // the weights it streams:
+    //  * set A, MEGA_DEPTH tasks per round.  A task is (row pair, segment of MEGA_SEG_PIECES pieces);
+    //    wave w owns the local pairs w, w + 8, ... and walks each pair's segments in order, keeps per-lane
+    //    sums across the segments, reduces them across lanes once, and its last lane finishes and
+    //    publishes the two outputs, so the waves never wait for each other after staging;
+    //  * set B, MEGA_DEPTH_B tasks per round.  An odd phase has only a few row pairs per workgroup, so
+    //    its (pair, segment) tasks are dealt to the waves one by one (task t to wave t % 8); the per-task
+    //    sums meet in LDS and the first threads of the workgroup finish the rows.
+    // The first round of a phase is requested when the input of the phase BEFORE it has been seen, into
+    // the set that phase does not use: it streams while that phase multiplies and publishes and while
+    // the exchange travels.  Inside a phase the next round follows the current one into the same set.
+    // Each set is written at fixed places of the loop body, always after its last use, so the loads
+    // land in the registers the multiply reads (a set refilled on only one of two merging paths is
+    // copied register by register at the merge, which waits for the loads).
+    const int pt = tid;                                      // every thread polls
+    const int last_ph = a.do_head ? 4 * L : 4 * L - 1;
+    MegaStage<WT> stA[MEGA_DEPTH], stB[MEGA_DEPTH_B];
+    int e_left = 0, e_pl = 0, e_sg = 0;                      // cursor of set A: tasks left in its phase, next (local pair, segment)
+    int o_left = 0, o_pl = 0, o_sg = 0;                      // cursor of set B
+    // Lanes past the end of a row and padding tasks issue nothing (a skipped load is not free if it
+    // is issued anyway: it still occupies the address unit) and are ignored when the round is consumed.
+    auto start_even = [&](int ph) {
+        const int kind = ph == 4 * L ? MK_HEAD : (ph & 3);
         const int npl = kinds[kind].npl;
-        return (streams && npl > wave) ? ((npl - wave + MEGA_SW - 1) / MEGA_SW) * kinds[kind].segs : 0;
+        e_left = npl > wave ? ((npl - wave + MEGA_WAVES - 1) / MEGA_WAVES) * kinds[kind].segs : 0;
+        e_pl = wave; e_sg = 0;
     };
-    const int last_ph = a.do_head ? 4 * L : 4 * L - 1;       // GEMV phase sequence: l*4 + kind, then the head
-
-    // ---- weight prefetch: one register set holding the next round of MEGA_DEPTH tasks
-    MegaStage<WT> st[MEGA_DEPTH];
-    int p_ph = -1, p_left = 0, p_pl = 0, p_sg = 0;           // prefetch cursor
-    int p_pieces = 1, p_segs = 1, p_pair0 = 0, p_kg = 0;
-    size_t p_rb = 0;
-    const char *p_W = (const char *)a.embed;
-    const uint16_t *p_SC = nullptr;
-    // Requests the next round of this wave (a round never mixes phases).  Lanes past the end of
-    // a row and padding tasks re-read a valid address (served from cache) and are ignored when
-    // the round is consumed.
-    auto issue_round = [&]() {
-        while (p_left == 0 && p_ph < last_ph) {
-            ++p_ph;
-            const int kind = p_ph == 4 * L ? MK_HEAD : (p_ph & 3);
-            const MegaKind &k = kinds[kind];
-            p_left = n_mine(kind);
-            p_pieces = k.pieces; p_segs = k.segs; p_pair0 = k.pair0; p_rb = k.row_bytes; p_kg = k.K / 128;
-            p_pl = wave; p_sg = 0;
-            if (kind == MK_HEAD) { p_W = (const char *)a.embed; p_SC = nullptr; }
-            else { p_W = (const char *)lptr[(p_ph >> 2) * MEGA_LPTR + kind]; p_SC = (const uint16_t *)lptr[(p_ph >> 2) * MEGA_LPTR + 4 + kind]; }
-        }
-        // a skipped load is not free if it is issued anyway (it still occupies the address unit),
-        // so padding tasks and lanes past the row end issue nothing
+    auto issue_even = [&](int ph) {
+        const int kind = ph == 4 * L ? MK_HEAD : (ph & 3);
+        const MegaKind &k = kinds[kind];
+        const int p_pieces = k.pieces, p_segs = k.segs, p_pair0 = k.pair0, p_kg = k.K / 128;
+        const size_t p_rb = k.row_bytes;
+        const char *p_W = kind == MK_HEAD ? (const char *)a.embed : (const char *)lptr[(ph >> 2) * MEGA_LPTR + kind];
+        const uint16_t *p_SC = kind == MK_HEAD ? nullptr : (const uint16_t *)lptr[(ph >> 2) * MEGA_LPTR + 4 + kind];
 #pragma unroll
         for (int s = 0; s < MEGA_DEPTH; ++s) {
-            if (p_left > 0) {
-                const size_t row = (size_t)2 * (p_pair0 + p_pl);
+            if (e_left > 0) {
+                const size_t row = (size_t)2 * (p_pair0 + e_pl);
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
-                    const int piece = p_sg * MEGA_SEG_PIECES + j * 64 + lane;
+                    const int piece = e_sg * MEGA_SEG_PIECES + j * 64 + lane;
                     if (piece < p_pieces) {
 #pragma unroll
                         for (int r = 0; r < 2; ++r) {
-                            st[s].w[r][j] = ld_stream_u4(p_W + (row + r) * p_rb + (size_t)piece * 16);
-                            if (WT == WT_INT4) st[s].sc[r][j] = ldg_u16(p_SC + (row + r) * p_kg + (piece >> 2));   // 4-bit models keep the head outside
+                            stA[s].w[r][j] = ld_stream_u4(p_W + (row + r) * p_rb + (size_t)piece * 16);
+                            if (WT == WT_INT4) stA[s].sc[r][j] = ldg_u16(p_SC + (row + r) * p_kg + (piece >> 2));   // 4-bit models keep the head outside
                         }
                     }
                 }
-                --p_left;
-                if (++p_sg == p_segs) { p_sg = 0; p_pl += MEGA_SW; }
+                --e_left;
+                if (++e_sg == p_segs) { e_sg = 0; e_pl += MEGA_WAVES; }
+            }
+        }
+    };
+    auto start_odd = [&](int ph) {
+        const MegaKind &k = kinds[ph & 3];
+        o_left = k.ntasks > wave ? (k.ntasks - wave + MEGA_WAVES - 1) / MEGA_WAVES : 0;
+        o_pl = 0; o_sg = wave;
+        while (o_sg >= k.segs) { o_sg -= k.segs; ++o_pl; }
+    };
+    auto issue_odd = [&](int ph) {
+        const int kind = ph & 3;
+        const MegaKind &k = kinds[kind];
+        const int p_pieces = k.pieces, p_segs = k.segs, p_pair0 = k.pair0, p_kg = k.K / 128;
+        const size_t p_rb = k.row_bytes;
+        const char *p_W = (const char *)lptr[(ph >> 2) * MEGA_LPTR + kind];
+        const uint16_t *p_SC = (const uint16_t *)lptr[(ph >> 2) * MEGA_LPTR + 4 + kind];
+#pragma unroll
+        for (int s = 0; s < MEGA_DEPTH_B; ++s) {
+            if (o_left > 0) {
+                const size_t row = (size_t)2 * (p_pair0 + o_pl);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int piece = o_sg * MEGA_SEG_PIECES + j * 64 + lane;
+                    if (piece < p_pieces) {
+#pragma unroll
+                        for (int r = 0; r < 2; ++r) {
+                            stB[s].w[r][j] = ld_stream_u4(p_W + (row + r) * p_rb + (size_t)piece * 16);
+                            if (WT == WT_INT4) stB[s].sc[r][j] = ldg_u16(p_SC + (row + r) * p_kg + (piece >> 2));
+                        }
+                    }
+                }
+                --o_left;
+                o_sg += MEGA_WAVES;
+                while (o_sg >= p_segs) { o_sg -= p_segs; ++o_pl; }
+            }
+        }
+    };
+    // one task: both rows of a pair times the staged vector over one segment
+    auto mul_task = [&](const MegaStage<WT> &t, const float *xs, const int sg, const int pieces, float &o0, float &o1) {
+        o0 = 0.0f; o1 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int piece = sg * MEGA_SEG_PIECES + j * 64 + lane;
+            if (piece < pieces) {
+                float xv[EPL];
+                constexpr int CPP = EPL / 4;                              // chunks per piece
+                const int rot = XSWZ ? piece >> (EPL == 32 ? 0 : EPL == 16 ? 1 : 2) : 0;
+#pragma unroll
+                for (int e = 0; e < EPL; e += 4) {
+                    float4 tq = *(const float4 *)(xs + piece * EPL + 4 * ((e / 4 + rot) & (CPP - 1)));
+                    xv[e] = tq.x; xv[e + 1] = tq.y; xv[e + 2] = tq.z; xv[e + 3] = tq.w;
+                }
+                float w0[EPL], w1[EPL];
+                WS<WT>::decode(t.w[0][j], w0);
+                WS<WT>::decode(t.w[1][j], w1);
+                float p0 = 0.0f, p1 = 0.0f;
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) { p0 = fmaf(w0[e], xv[e], p0); p1 = fmaf(w1[e], xv[e], p1); }
+                if (WT == WT_INT4) {
+                    p0 *= bf16_to_f32(t.sc[0][j]) * WS<WT_INT4>::SCALE_MUL;
+                    p1 *= bf16_to_f32(t.sc[1][j]) * WS<WT_INT4>::SCALE_MUL;
+                }
+                o0 += p0; o1 += p1;
             }
         }
     };
@@ -384,7 +447,8 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     // the compiler wait for "everything outstanding" at the top of every iteration, which later
     // includes the weights requested for the phase.
     __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0)
-    if (streams) issue_round();
+    start_even(0);
+    issue_even(0);
 
     const int wo_row0 = 2 * kinds[MK_WO].pair0, wo_rows = 2 * kinds[MK_WO].npl;   // same partition for w2
     const int n_att = pos + 1;
@@ -394,21 +458,184 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     const float att_scale = 1.0f / sqrtf((float)HD);
     const unsigned par_c = (ep_head + 1u) & 1u;
 
-    for (int ph = 0; ph <= last_ph; ++ph) {
+    for (int ph = 0; ph <= last_ph; ph += 2) {
+        // ===================================================================== even phase: qkv, w13 or head
+        {
         const int l = min(ph >> 2, L - 1);
         const int kind = ph == 4 * L ? MK_HEAD : (ph & 3);
         const unsigned par = (ep_layer + (unsigned)l + 1u) & 1u;      // stamp of layer l's exchanges
         const float *g1 = (const float *)lptr[l * MEGA_LPTR + 8], *g2 = (const float *)lptr[l * MEGA_LPTR + 9];
         void *kcl = (void *)lptr[l * MEGA_LPTR + 10], *vcl = (void *)lptr[l * MEGA_LPTR + 11];
-        float *xs = xsb + (ph & 1) * D;
+        float *xs = xsb;
         // residual inputs: the qkv stage keeps x for the wo epilogue in buffer 0, the w13 stage keeps
         // x2 for the w2 epilogue in buffer 1
         float *xres_w = xresb + (kind == MK_W13 ? xres_n : 0);
-        const float *xres_r = xresb + (kind == MK_W2 ? xres_n : 0);
-        if (prof && (kind == MK_QKV || kind == MK_HEAD)) prof_n = (ph >> 2) * MEGA_PROF_SLOTS;
+        if (prof && kind != MK_W13) prof_n = (ph >> 2) * MEGA_PROF_SLOTS;
         mark();
 
-        // ================= attention (before the output projection): item (split, head) on workgroup b
+        // ---- stage this phase's input vector in xs
+        float ss = 0.0f;
+        bool ok = true;
+        if (kind == MK_QKV && l == 0) {
+            for (int i = tid; i < D; i += MEGA_THREADS) {
+                float v;
+                if (use_x_in) v = a.x_in[i];
+                else if (WT == WT_F32) v = ((const float *)a.embed)[(size_t)tok * D + i];
+                else v = bf16_to_f32(((const uint16_t *)a.embed)[(size_t)tok * D + i]);
+                xs[xs_pos(i, XSWZ)] = v * g1[i];
+                ss += v * v;
+                if (i >= wo_row0 && i < wo_row0 + wo_rows) xres_w[i - wo_row0] = v;
+            }
+        } else {
+            // qkv / head: X of the previous layer; w13: X2
+            const float *src = kind == MK_W13 ? a.X2 : a.X;
+            const float *gm = kind == MK_QKV ? g1 : kind == MK_W13 ? g2 : a.gfinal;
+            const unsigned pr = kind == MK_QKV ? (par ^ 1u) : kind == MK_HEAD ? ((ep_layer + (unsigned)L) & 1u) : par;
+            const int nres = kind == MK_HEAD ? 0 : wo_rows;
+            ss = mega_poll_vec<XSWZ>(src, D, pr, abortf, xs, gm, xres_w, wo_row0, nres, pt);
+            if (ss < 0.0f) { ok = false; ss = 0.0f; }
+        }
+        ss = wave_sum_dpp(ss);                    // (no LDS round trips; total in lane 63)
+        if (lane == 63) s_red[0][wave] = ss;
+        if (!ok) s_bad = 1;
+        lds_barrier();
+        if (s_bad) return;
+        mark();
+        // This phase's input is here, and so is set A (requested a phase ago; the multiply needs it now
+        // anyway).  The explicit wait tells the compiler so: from here on only the loads requested below
+        // are outstanding, and the multiply of set A runs without waiting for them.
+        __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
+        // the odd phase behind this one gets its first round now
+        if (ph + 1 <= last_ph) { start_odd(ph + 1); issue_odd(ph + 1); }
+        float inv;
+        {
+            float t = 0.0f;
+#pragma unroll
+            for (int w = 0; w < MEGA_WAVES; ++w) t += s_red[0][w];
+            inv = 1.0f / sqrtf(t * (1.0f / (float)D) + 1e-5f);
+        }
+
+        // ---- stream this workgroup's rows in rounds of MEGA_DEPTH tasks
+        float bv = -INFINITY; uint32_t bi = 0x7fffffffu;      // head phase: best logit seen by this wave (lane 63)
+        {
+            const MegaKind k = kinds[kind];
+            const int nm = k.npl > wave ? ((k.npl - wave + MEGA_WAVES - 1) / MEGA_WAVES) * k.segs : 0;
+            const float *fsc = (WT == WT_FP8 && kind != MK_HEAD) ? (const float *)lptr[l * MEGA_LPTR + 4 + kind] : nullptr;
+            int c_pl = wave, c_sg = 0;                        // (local pair, segment) of the next task to fold
+            int f_sg = 0;                                     // segment of the next task to multiply
+            float run0 = 0.0f, run1 = 0.0f;                   // per-lane sums of the pair being walked
+            auto even_round = [&](const int i) {
+                // (all sums are given their zero before the first task: an element left undefined at that point
+                // is filled from whatever register is at hand -- one of the other set's, whose loads are in
+                // flight -- and reading it waits for those loads)
+                float acc[MEGA_DEPTH][2];
+#pragma unroll
+                for (int s = 0; s < MEGA_DEPTH; ++s) { acc[s][0] = 0.0f; acc[s][1] = 0.0f; }
+#pragma unroll
+                for (int s = 0; s < MEGA_DEPTH; ++s) {
+                    if (i + s < nm) {
+                        const int sg = f_sg;
+                        if (++f_sg == k.segs) f_sg = 0;
+                        mul_task(stA[s], xs, sg, k.pieces, acc[s][0], acc[s][1]);
+                    }
+                }
+                if (i == 0) mark();
+                // inside a phase the next round is requested before the sums are finished (its latency
+                // overlaps them); the next phase's rounds belong to the odd phase in between
+                if (i + MEGA_DEPTH < nm) issue_even(ph);
+#pragma unroll
+                for (int s = 0; s < MEGA_DEPTH; ++s) {
+                  if (i + s < nm) {
+                    run0 += acc[s][0]; run1 += acc[s][1];
+                    if (++c_sg == k.segs) {
+                      float s0 = wave_sum_dpp(run0), s1 = wave_sum_dpp(run1);
+                      const int p = c_pl;
+                      run0 = 0.0f; run1 = 0.0f; c_sg = 0; c_pl += MEGA_WAVES;
+                      if (lane == 63) {
+                const int row0 = 2 * (k.pair0 + p);
+                if (fsc) { s0 *= fsc[row0]; s1 *= fsc[row0 + 1]; }
+                if (kind == MK_QKV) {
+                    s0 *= inv; s1 *= inv;
+                    if (row0 < Q + KV) {            // q and k rows: RoPE on the pair
+                        const float c = ropes[2 * p], s = ropes[2 * p + 1];
+                        const float e = s0 * c - s1 * s, o = s1 * c + s0 * s;
+                        s0 = e; s1 = o;
+                    }
+                    if (row0 >= Q) {                // k and v rows enter the cache (and the exchange) in cache precision
+                        const bool isk = row0 < Q + KV;
+                        const int rr = isk ? row0 - Q : row0 - Q - KV;
+                        void *cache = isk ? kcl : vcl;
+                        if (KVBF16) {
+                            const uint16_t eb = f32_to_bf16_rne(s0), ob = f32_to_bf16_rne(s1);
+                            uint16_t *cp = (uint16_t *)cache + (size_t)pos * KV + rr;
+                            cp[0] = eb; cp[1] = ob;
+                            s0 = bf16_to_f32(eb); s1 = bf16_to_f32(ob);
+                        } else {
+                            // the cache keeps what the exchange delivers (stamp bit cleared), so this step and
+                            // every later one attend over the same key / value bits
+                            s0 = __uint_as_float(__float_as_uint(s0) & ~1u); s1 = __uint_as_float(__float_as_uint(s1) & ~1u);
+                            float *cp = (float *)cache + (size_t)pos * KV + rr;
+                            cp[0] = s0; cp[1] = s1;
+                        }
+                    }
+                    st_stamped(a.QKV + row0, s0, par);
+                    st_stamped(a.QKV + row0 + 1, s1, par);
+                } else if (kind == MK_W13) {
+                    const float h1 = s0 * inv, h3 = s1 * inv;
+                    float gte;
+                    if (a.act == 1) { const float lr = h1 > 0.0f ? h1 : 0.5f * h1; gte = lr * lr * h3; }
+                    else { const float sig = 1.0f / (1.0f + expf(-h1)); gte = h1 * sig * h3; }
+                    st_stamped(a.GATE + (k.pair0 + p), gte, par);
+                } else {
+                    s0 *= inv; s1 *= inv;
+                    a.logits[row0] = s0; a.logits[row0 + 1] = s1;
+                    if (better(s0, (uint32_t)row0, bv, bi)) { bv = s0; bi = (uint32_t)row0; }
+                    if (better(s1, (uint32_t)row0 + 1, bv, bi)) { bv = s1; bi = (uint32_t)row0 + 1; }
+                }
+                      }
+                    }
+                  }
+                }
+            };
+            // The first round is taken outside the loop: it runs straight behind the request of the odd
+            // phase's weights, where it is known that set A has arrived and that only the new loads are
+            // outstanding (inside the loop a refilled set A would have to be assumed, and every use of a
+            // weight register would wait for all loads in flight, the other set's included).
+            if (nm > 0) even_round(0);
+            for (int i = MEGA_DEPTH; i < nm; i += MEGA_DEPTH) even_round(i);
+        }
+        mark();
+        if (kind == MK_HEAD) {
+            // the eight per-wave candidates meet in LDS; wave 0 publishes the workgroup's best
+            if (lane == 63) { s_cand_v[wave] = bv; s_cand_i[wave] = bi; }
+            lds_barrier();
+            if (wave == 0) {
+                float cv = lane < MEGA_WAVES ? s_cand_v[lane] : -INFINITY;
+                uint32_t ci = lane < MEGA_WAVES ? s_cand_i[lane] : 0x7fffffffu;
+                wave_argbest(cv, ci);
+                if (lane == 0) {
+                    unsigned long long c = (unsigned long long)__float_as_uint(cv) | ((unsigned long long)(ci | (par_c << 31)) << 32);
+                    __hip_atomic_store(a.CAND + b, c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            mark();
+            break;
+        }
+        mark();
+        }
+
+        // ===================================================================== odd phase: wo or w2
+        {
+        const int oph = ph + 1;
+        const int l = oph >> 2;
+        const int kind = oph & 3;
+        const unsigned par = (ep_layer + (unsigned)l + 1u) & 1u;
+        void *kcl = (void *)lptr[l * MEGA_LPTR + 10], *vcl = (void *)lptr[l * MEGA_LPTR + 11];
+        float *xs = xsb + D;
+        const float *xres_r = xresb + (kind == MK_W2 ? xres_n : 0);
+        mark();
+
+        // ---- attention (before the output projection): item (split, head) on workgroup b
         if (kind == MK_WO && b < a.heads * NS) {
             const int sidx = b / a.heads, h = b - sidx * a.heads, g = h / a.gqa;
             const int t0 = sidx * chunk, t1 = min(n_att, t0 + chunk);
@@ -420,20 +647,16 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             uint4 kr[PRE], vr[PRE];
 #pragma unroll
             for (int i = 0; i < PRE; ++i) { kr[i] = make_uint4(0, 0, 0, 0); vr[i] = make_uint4(0, 0, 0, 0); }
-            // rows older than the new token are already in the cache: the streaming waves fetch
-            // them before q arrives, the polling waves after they have seen it
-            auto kv_first = [&]() {
+            // rows older than the new token are already in the cache: they are fetched before q arrives
 #pragma unroll
-                for (int i = 0; i < PRE; ++i) {
-                    const int t = t0 + slot + i * SLOTS;
-                    if (t < t1 && t != pos) { kr[i] = ldg_u4(kb + (size_t)t * rowb); vr[i] = ldg_u4(vb + (size_t)t * rowb); }
-                }
-            };
-            if (streams) kv_first();
+            for (int i = 0; i < PRE; ++i) {
+                const int t = t0 + slot + i * SLOTS;
+                if (t < t1 && t != pos) { kr[i] = ldg_u4(kb + (size_t)t * rowb); vr[i] = ldg_u4(vb + (size_t)t * rowb); }
+            }
             {
                 // q of head h, k and v of kv-head g: three HD-float pieces of the QKV exchange vector
                 bool ok = true;
-                if (pt >= 0 && pt < 3 * (HD / 4)) {
+                if (pt < 3 * (HD / 4)) {
                     const int which = pt / (HD / 4), i4 = pt - which * (HD / 4);
                     const float *src = a.QKV + (which == 0 ? h * HD : which == 1 ? Q + g * HD : Q + KV + g * HD);
                     float *dst = which == 0 ? qs : which == 1 ? kcur : vcur;
@@ -444,7 +667,6 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                     dst[4 * i4] = __uint_as_float(v.x & ~1u) * mul; dst[4 * i4 + 1] = __uint_as_float(v.y & ~1u) * mul;
                     dst[4 * i4 + 2] = __uint_as_float(v.z & ~1u) * mul; dst[4 * i4 + 3] = __uint_as_float(v.w & ~1u) * mul;
                 }
-                if (!streams) kv_first();
                 if (!ok) s_bad = 1;
                 lds_barrier();
                 if (s_bad) return;
@@ -540,40 +762,27 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             }
         }
 
-        // ================= stage this phase's input vector in xs
-        float ss = 0.0f;
-        bool ok = true;
-        if (kind == MK_QKV && l == 0) {
-            for (int i = tid; i < D; i += MEGA_THREADS) {
-                float v;
-                if (use_x_in) v = a.x_in[i];
-                else if (WT == WT_F32) v = ((const float *)a.embed)[(size_t)tok * D + i];
-                else v = bf16_to_f32(((const uint16_t *)a.embed)[(size_t)tok * D + i]);
-                xs[xs_pos(i, XSWZ)] = v * g1[i];
-                ss += v * v;
-                if (i >= wo_row0 && i < wo_row0 + wo_rows) xres_w[i - wo_row0] = v;
+        // ---- stage this phase's input: the attention partials (wo) or the gate vector (w2)
+        {
+            bool ok = true;
+            float ss;
+            if (kind == MK_WO) {
+                const int n = NS * a.heads * REC;
+                if (BIGPART) ss = mega_poll_vec<0, MEGA_PART_NB, false>(a.PART, n, par, abortf, stage, nullptr, xresb, wo_row0, 0, pt);
+                else ss = mega_poll_vec<0>(a.PART, n, par, abortf, stage, nullptr, xresb, wo_row0, 0, pt);
+            } else {
+                ss = mega_poll_vec<XSWZ>(a.GATE, H, par, abortf, xs, nullptr, xresb, wo_row0, 0, pt);
             }
-        } else {
-            // QKV / head: X of the previous layer; WO: attention partials; W13: X2; W2: gate
-            const float *src = kind == MK_WO ? a.PART : kind == MK_W13 ? a.X2 : kind == MK_W2 ? a.GATE : a.X;
-            const int n = kind == MK_WO ? NS * a.heads * REC : kind == MK_W2 ? H : D;
-            const float *gm = kind == MK_QKV ? g1 : kind == MK_W13 ? g2 : kind == MK_HEAD ? a.gfinal : nullptr;
-            float *dst = kind == MK_WO ? stage : xs;
-            const unsigned pr = kind == MK_QKV ? (par ^ 1u) : kind == MK_HEAD ? ((ep_layer + (unsigned)L) & 1u) : par;
-            const int nres = (kind == MK_QKV || kind == MK_W13) ? wo_rows : 0;
-            if (polls) {
-                if (BIGPART && kind == MK_WO) ss = mega_poll_vec<0, MEGA_PART_NB, false>(src, n, pr, abortf, dst, gm, xres_w, wo_row0, nres, pt);
-                else if (XSWZ == 0 || kind == MK_WO) ss = mega_poll_vec<0>(src, n, pr, abortf, dst, gm, xres_w, wo_row0, nres, pt);
-                else ss = mega_poll_vec<XSWZ>(src, n, pr, abortf, dst, gm, xres_w, wo_row0, nres, pt);
-                if (ss < 0.0f) { ok = false; ss = 0.0f; }
-            }
+            if (ss < 0.0f) ok = false;
+            if (!ok) s_bad = 1;
+            lds_barrier();
+            if (s_bad) return;
         }
-        ss = wave_sum_dpp(ss);                    // (no LDS round trips; total in lane 63)
-        if (lane == 63) s_red[ph & 1][wave] = ss;
-        if (!ok) s_bad = 1;
-        lds_barrier();
-        if (s_bad) return;
         mark();
+        // this phase's input and set B are here (see the even phase): the even phase behind it gets its
+        // first round now
+        __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
+        if (oph + 1 <= last_ph) { start_even(oph + 1); issue_even(oph + 1); }
         if (kind == MK_WO) {
             // fold the split partials of every head into the attention output vector
             const int sstride = a.heads * REC;
@@ -625,145 +834,57 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             lds_barrier();
             mark();
         }
-        float inv = 0.0f;
-        if (kind != MK_WO && kind != MK_W2) {     // (the projections back into the residual stream take no norm)
-            float t = 0.0f;
-#pragma unroll
-            for (int w = 0; w < MEGA_WAVES; ++w) t += s_red[ph & 1][w];
-            inv = 1.0f / sqrtf(t * (1.0f / (float)D) + 1e-5f);
-        }
 
-        // ================= stream this workgroup's rows in rounds of MEGA_DEPTH tasks.  The round's
-        // weights were requested one round (or one phase) earlier; once consumed, the registers are
-        // refilled with the next round, which after the last round is the first round of the NEXT
-        // phase.  A wave owns whole row pairs: it keeps per-lane partial sums across the segments
-        // of a pair, reduces them across lanes once, and its last lane finishes and publishes the
-        // two outputs, so the waves of a workgroup never wait for each other after staging.
-        float bv = -INFINITY; uint32_t bi = 0x7fffffffu;      // head phase: best logit seen by this wave (lane 63)
+        // ---- stream this workgroup's rows: wave w multiplies tasks w, w + 8, ... in rounds of MEGA_DEPTH_B
+        // and leaves each task's two sums in LDS (the staging area of the partials is free by now)
         {
             const MegaKind k = kinds[kind];
-            const int nm = n_mine(kind);
-            const float *fsc = (WT == WT_FP8 && kind != MK_HEAD) ? (const float *)lptr[l * MEGA_LPTR + 4 + kind] : nullptr;
-            int c_pl = wave, c_sg = 0;                        // (local pair, segment) of the next task to fold
-            int f_sg = 0;                                     // segment of the next task to multiply
-            float run0 = 0.0f, run1 = 0.0f;                   // per-lane sums of the pair being walked
-            for (int i = 0; i < nm; i += MEGA_DEPTH) {
-                float acc[MEGA_DEPTH][2];
+            const int nm = k.ntasks > wave ? (k.ntasks - wave + MEGA_WAVES - 1) / MEGA_WAVES : 0;
+            int f_t = wave, f_sg = wave;                     // next task and its segment
+            while (f_sg >= k.segs) f_sg -= k.segs;
+            auto odd_round = [&](const int i) {
+                float acc[MEGA_DEPTH_B][2];
+                int slot_t[MEGA_DEPTH_B];
 #pragma unroll
-                for (int s = 0; s < MEGA_DEPTH; ++s) {
-                    acc[s][0] = 0.0f; acc[s][1] = 0.0f;
+                for (int s = 0; s < MEGA_DEPTH_B; ++s) { acc[s][0] = 0.0f; acc[s][1] = 0.0f; slot_t[s] = 0; }
+#pragma unroll
+                for (int s = 0; s < MEGA_DEPTH_B; ++s) {
+                    slot_t[s] = f_t;
                     if (i + s < nm) {
-                        const int sg = f_sg;
-                        if (++f_sg == k.segs) f_sg = 0;
-#pragma unroll
-                        for (int j = 0; j < 2; ++j) {
-                            const int piece = sg * MEGA_SEG_PIECES + j * 64 + lane;
-                            if (piece < k.pieces) {
-                                float xv[EPL];
-                                constexpr int CPP = EPL / 4;                              // chunks per piece
-                                const int rot = XSWZ ? piece >> (EPL == 32 ? 0 : EPL == 16 ? 1 : 2) : 0;
-#pragma unroll
-                                for (int e = 0; e < EPL; e += 4) {
-                                    float4 tq = *(const float4 *)(xs + piece * EPL + 4 * ((e / 4 + rot) & (CPP - 1)));
-                                    xv[e] = tq.x; xv[e + 1] = tq.y; xv[e + 2] = tq.z; xv[e + 3] = tq.w;
-                                }
-                                float w0[EPL], w1[EPL];
-                                WS<WT>::decode(st[s].w[0][j], w0);
-                                WS<WT>::decode(st[s].w[1][j], w1);
-                                float p0 = 0.0f, p1 = 0.0f;
-#pragma unroll
-                                for (int e = 0; e < EPL; ++e) { p0 = fmaf(w0[e], xv[e], p0); p1 = fmaf(w1[e], xv[e], p1); }
-                                if (WT == WT_INT4) {
-                                    p0 *= bf16_to_f32(st[s].sc[0][j]) * WS<WT_INT4>::SCALE_MUL;
-                                    p1 *= bf16_to_f32(st[s].sc[1][j]) * WS<WT_INT4>::SCALE_MUL;
-                                }
-                                acc[s][0] += p0; acc[s][1] += p1;
-                            }
-                        }
+                        mul_task(stB[s], xs, f_sg, k.pieces, acc[s][0], acc[s][1]);
+                        f_t += MEGA_WAVES; f_sg += MEGA_WAVES;
+                        while (f_sg >= k.segs) f_sg -= k.segs;
                     }
                 }
                 if (i == 0) mark();
-                // inside a phase the next round is requested before the sums are finished (its
-                // latency overlaps them); at the end of a phase the outputs other workgroups wait
-                // for go out first
-                const bool last_round = i + MEGA_DEPTH >= nm;
-                if (!last_round) issue_round();
+                if (i + MEGA_DEPTH_B < nm) issue_odd(oph);
 #pragma unroll
-                for (int s = 0; s < MEGA_DEPTH; ++s) {
-                  if (i + s < nm) {
-                    run0 += acc[s][0]; run1 += acc[s][1];
-                    if (++c_sg == k.segs) {
-                      float s0 = wave_sum_dpp(run0), s1 = wave_sum_dpp(run1);
-                      const int p = c_pl;
-                      run0 = 0.0f; run1 = 0.0f; c_sg = 0; c_pl += MEGA_SW;
-                      if (lane == 63) {
-                const int row0 = 2 * (k.pair0 + p);
-                if (fsc) { s0 *= fsc[row0]; s1 *= fsc[row0 + 1]; }
-                if (kind == MK_QKV) {
-                    s0 *= inv; s1 *= inv;
-                    if (row0 < Q + KV) {            // q and k rows: RoPE on the pair
-                        const float c = ropes[2 * p], s = ropes[2 * p + 1];
-                        const float e = s0 * c - s1 * s, o = s1 * c + s0 * s;
-                        s0 = e; s1 = o;
+                for (int s = 0; s < MEGA_DEPTH_B; ++s) {
+                    if (i + s < nm) {
+                        const float s0 = wave_sum_dpp(acc[s][0]), s1 = wave_sum_dpp(acc[s][1]);
+                        if (lane == 63) { stage[2 * slot_t[s]] = s0; stage[2 * slot_t[s] + 1] = s1; }
                     }
-                    if (row0 >= Q) {                // k and v rows enter the cache (and the exchange) in cache precision
-                        const bool isk = row0 < Q + KV;
-                        const int rr = isk ? row0 - Q : row0 - Q - KV;
-                        void *cache = isk ? kcl : vcl;
-                        if (KVBF16) {
-                            const uint16_t eb = f32_to_bf16_rne(s0), ob = f32_to_bf16_rne(s1);
-                            uint16_t *cp = (uint16_t *)cache + (size_t)pos * KV + rr;
-                            cp[0] = eb; cp[1] = ob;
-                            s0 = bf16_to_f32(eb); s1 = bf16_to_f32(ob);
-                        } else {
-                            // the cache keeps what the exchange delivers (stamp bit cleared), so this step and
-                            // every later one attend over the same key / value bits
-                            s0 = __uint_as_float(__float_as_uint(s0) & ~1u); s1 = __uint_as_float(__float_as_uint(s1) & ~1u);
-                            float *cp = (float *)cache + (size_t)pos * KV + rr;
-                            cp[0] = s0; cp[1] = s1;
-                        }
-                    }
-                    st_stamped(a.QKV + row0, s0, par);
-                    st_stamped(a.QKV + row0 + 1, s1, par);
-                } else if (kind == MK_WO || kind == MK_W2) {
-                    float *dstv = kind == MK_WO ? a.X2 : a.X;
-                    st_stamped(dstv + row0, xres_r[2 * p] + a.alpha * s0, par);
-                    st_stamped(dstv + row0 + 1, xres_r[2 * p + 1] + a.alpha * s1, par);
-                } else if (kind == MK_W13) {
-                    const float h1 = s0 * inv, h3 = s1 * inv;
-                    float gte;
-                    if (a.act == 1) { const float lr = h1 > 0.0f ? h1 : 0.5f * h1; gte = lr * lr * h3; }
-                    else { const float sig = 1.0f / (1.0f + expf(-h1)); gte = h1 * sig * h3; }
-                    st_stamped(a.GATE + (k.pair0 + p), gte, par);
-                } else {
-                    s0 *= inv; s1 *= inv;
-                    a.logits[row0] = s0; a.logits[row0 + 1] = s1;
-                    if (better(s0, (uint32_t)row0, bv, bi)) { bv = s0; bi = (uint32_t)row0; }
-                    if (better(s1, (uint32_t)row0 + 1, bv, bi)) { bv = s1; bi = (uint32_t)row0 + 1; }
                 }
-                      }
-                    }
-                  }
-                }
-                if (last_round) issue_round();
-            }
-        }
-        mark();
-        if (kind == MK_HEAD) {
-            // the eight per-wave candidates meet in LDS; wave 0 publishes the workgroup's best
-            if (lane == 63) { s_cand_v[wave] = bv; s_cand_i[wave] = bi; }
+            };
+            if (nm > 0) odd_round(0);                        // (first round outside the loop, as in the even phase)
+            for (int i = MEGA_DEPTH_B; i < nm; i += MEGA_DEPTH_B) odd_round(i);
             lds_barrier();
-            if (wave == 0) {
-                float cv = lane < MEGA_WAVES ? s_cand_v[lane] : -INFINITY;
-                uint32_t ci = lane < MEGA_WAVES ? s_cand_i[lane] : 0x7fffffffu;
-                wave_argbest(cv, ci);
-                if (lane == 0) {
-                    unsigned long long c = (unsigned long long)__float_as_uint(cv) | ((unsigned long long)(ci | (par_c << 31)) << 32);
-                    __hip_atomic_store(a.CAND + b, c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
+            // thread r finishes local row r: the segments of its pair in order, scale, residual, publish
+            if (tid < 2 * k.npl) {
+                const int p = tid >> 1, which = tid & 1;
+                float sum = 0.0f;
+                for (int sg = 0; sg < k.segs; ++sg) sum += stage[2 * (p * k.segs + sg) + which];
+                const int row = 2 * k.pair0 + tid;
+                if (WT == WT_FP8) sum *= ((const float *)lptr[l * MEGA_LPTR + 4 + kind])[row];
+                float *dstv = kind == MK_WO ? a.X2 : a.X;
+                st_stamped(dstv + row, xres_r[tid] + a.alpha * sum, par);
             }
+            // (the next writer of the staging area is the next attention phase or this loop's next round
+            // of sums, both behind a barrier of the phases in between)
         }
         mark();
+        mark();
+        }
     }
 
     if (!a.do_head) {
