@@ -104,7 +104,6 @@ struct hipdec_model {
     MegaArgs mega{};
     int mega_grid = 0;
     size_t mega_lds = 0;
-    int mega_slots = 0;               // cache rows one attention pass of the persistent kernel covers
     unsigned *d_epochs = nullptr;
     void *xslab = nullptr;                            // uncached slab holding the exchange buffers (uncached_take)
     size_t xslab_cap = 0;
@@ -262,13 +261,7 @@ void launch_attn(hipdec_model *m, const DevLayer &L) {
 template <int WT> void launch_mega_t(hipdec_model *m, const MegaArgs &a) {
     dim3 grid(m->mega_grid), block(MEGA_THREADS);
 #define MEGA2(KVB, HD, BP) hipLaunchKernelGGL((k_mega<WT, KVB, HD, BP>), grid, block, m->mega_lds, m->stream, a)
-    // the kernel's split count at this position (positions of steps enqueued behind this one are
-    // not known here: a run keeps the variant its first step chose; both give the same results)
-    const int n_att = (int)m->len + 1;
-    const int ns = std::max(1, std::min((n_att + m->mega_slots * MEGA_ATT_PRE - 1) / (m->mega_slots * MEGA_ATT_PRE), a.ns_max));
-    const bool bigpart = (size_t)a.heads * ns * (a.hd + MEGA_PREC) / 4 > (size_t)2048;
-#define MEGA(KVB, HD) do { if (bigpart) MEGA2(KVB, HD, MEGA_VAR_BIGPART); else if (a.prof) MEGA2(KVB, HD, MEGA_VAR_STAMPS); \
-                            else MEGA2(KVB, HD, MEGA_VAR_PLAIN); } while (0)
+#define MEGA(KVB, HD) do { if (a.prof) MEGA2(KVB, HD, MEGA_VAR_STAMPS); else MEGA2(KVB, HD, MEGA_VAR_PLAIN); } while (0)
     if (m->kvbf16) { if (m->cfg.hd == 64) MEGA(1, 64); else MEGA(1, 128); }
     else { if (m->cfg.hd == 64) MEGA(0, 64); else MEGA(0, 128); }
 #undef MEGA
@@ -294,9 +287,6 @@ template <int WT> hipError_t mega_set_lds_t(hipdec_model *m) {
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)m->mega_lds);                    \
         if (e == hipSuccess)                                                                                      \
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mega<WT, KVB, HD, MEGA_VAR_STAMPS>),        \
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)m->mega_lds);                \
-        if (e == hipSuccess)                                                                                      \
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mega<WT, KVB, HD, MEGA_VAR_BIGPART>),       \
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)m->mega_lds);                \
     } while (0)
     if (m->kvbf16) { if (m->cfg.hd == 64) MEGA_ATTR(1, 64); else MEGA_ATTR(1, 128); }
@@ -1129,25 +1119,20 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
         max_tasks = std::max(max_tasks, tasks_of(2 * H, D));
         max_tasks = std::max(max_tasks, tasks_of(D, H));
         if (head_inside) max_tasks = std::max(max_tasks, tasks_of(V, D));
-        const size_t kesz = m->kvbf16 ? 2 : 4;
-        const int slots = MEGA_THREADS / (int)(c.hd / (16 / kesz));
         // LDS of the persistent kernel: the staged input vector twice (even phases read D floats, odd
-        // phases max(Q, H)), the attention staging area, the residual inputs twice, the RoPE pairs
-        // and the per-layer pointer table.  The attention split count takes what is left.
+        // phases max(Q, H)), a small staging area (attention: one partial per wave and q / k / v of the new
+        // token; odd phases: two sums per task), the residual inputs twice, the RoPE pairs and the
+        // per-layer pointer table.
         const size_t lds_cap = 160 * 1024 - 2048;
         const size_t xs_floats = D + std::max(Q, H);
         const size_t xres_floats = 2 * ((D / 2 + G - 1) / G) + 2;
         const size_t rope_floats = 2 * (((Q + 2 * KV) / 2 + G - 1) / G) + 2;
         const size_t fixed_lds = (xs_floats + 2 * xres_floats + rope_floats) * 4 + (size_t)MEGA_LPTR * c.nlayers * sizeof(void *);
-        const size_t rec_bytes = (size_t)c.heads * (c.hd + MEGA_PREC) * 4;
-        int ns_max = G / (int)c.heads;
-        const int ns_lds = fixed_lds < lds_cap ? (int)((lds_cap - fixed_lds) / rec_bytes) : 0;
-        if (ns_max > ns_lds) ns_max = ns_lds;
+        int ns_max = G / (int)c.heads;                 // one workgroup per (split, head)
         if (ns_max > 32) ns_max = 32;
-        const size_t stage_floats = std::max((size_t)c.heads * (ns_max > 0 ? ns_max : 1) * (c.hd + MEGA_PREC),
-                                             (size_t)slots * (c.hd + MEGA_PREC) + 3 * c.hd);
+        const size_t odd_tasks = std::max(tasks_of(D, Q), tasks_of(D, H));
+        const size_t stage_floats = std::max((size_t)MEGA_WAVES * (c.hd + MEGA_PREC) + 3 * c.hd, 2 * odd_tasks);
         m->mega_lds = fixed_lds + stage_floats * 4;
-        m->mega_slots = slots;
         const char *env = getenv("HIPDEC_NO_MEGA");
         bool want = !(m->opt.flags & HIPDEC_FLAG_NO_MEGA) && !(env && env[0] == '1');
         bool fits = ns_max >= 1 && m->mega_lds <= lds_cap && (V % 2 == 0) && (int)c.heads <= G &&
@@ -1198,6 +1183,7 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
             a.D = (int)D; a.Q = (int)Q; a.KV = (int)KV; a.H = (int)H; a.V = (int)V; a.L = (int)c.nlayers;
             a.hd = (int)c.hd; a.heads = (int)c.heads; a.gqa = c.gqa_ratio ? (int)c.gqa_ratio : 1;
             a.act = (int)m->opt.ffn_activation; a.ns_max = ns_max; a.seq = (int)S; a.alpha = m->alpha;
+            a.stage_floats = (int)stage_floats;
             m->mega_grid = G;
             hipError_t e;
             switch (wt) {

@@ -23,18 +23,24 @@
 // a workgroup that spins too long raises an abort flag that makes every other workgroup leave too.
 #pragma once
 #include "hipdec_kernels.h"
+#include <type_traits>
 
 #define MEGA_THREADS 512
 #define MEGA_WAVES 8
 #define MEGA_DEPTH 4            // tasks per round of the even phases (16 loads of 16 bytes in flight per lane)
 #ifndef MEGA_DEPTH_B
-#define MEGA_DEPTH_B 2          // tasks per round of the odd phases (wo, w2: few rows per workgroup)
+#define MEGA_DEPTH_B 2          // tasks per round of the odd phases (wo, w2: few rows per workgroup); divides MEGA_DEPTH
 #endif
 #define MEGA_SEG_PIECES 128     // 16-byte pieces of one row per task: 2 per lane
 #define MEGA_SPIN_LIMIT (1u << 22)
 #define MEGA_PREC 4             // attention partial record = HD + 4 floats (acc[HD], max, sum, 0, 0)
 #define MEGA_PROF_SLOTS 32      // timestamps per layer when profiling
 #define MEGA_ATT_PRE 4          // attention: cache-row passes a thread requests ahead
+#ifndef MEGA_ATT_SPLIT_PASSES
+#define MEGA_ATT_SPLIT_PASSES 4 // attention: passes (of 512 / lanes-per-row cache rows) one split covers while splits are to be had
+                                // (600M at 256 positions: 1 pass 0.591, 2 passes 0.573, 4 passes 0.556, 8 passes 0.575 ms per token:
+                                // every further split is two more polls per thread in the fold)
+#endif
 #define MEGA_LPTR 12            // pointers per layer in the LDS copy of the layer table
 
 enum { MK_QKV = 0, MK_WO = 1, MK_W13 = 2, MK_W2 = 3, MK_HEAD = 4, MK_KINDS = 5 };
@@ -57,7 +63,7 @@ struct MegaArgs {
     unsigned *epochs;                                // [0] per-layer exchange counter, [1] head counter, [2] abort
     unsigned long long *prof;                        // nullable: workgroup 0 writes wall-clock stamps here
     int ring_cap;
-    int D, Q, KV, H, V, L, hd, heads, gqa, act, do_head, advance, ns_max, seq;
+    int D, Q, KV, H, V, L, hd, heads, gqa, act, do_head, advance, ns_max, seq, stage_floats;
     float alpha;
 };
 
@@ -137,9 +143,6 @@ __device__ __forceinline__ int xs_pos(int i, int epl) { return (xs_chunk_pos(i >
 // to its use and the loads of one thread stop overlapping.  The price is that a called function
 // starts by waiting for every outstanding load of the wave, the requested weights included; loads
 // return in order, so the polled values could not be seen before those anyway.
-#ifndef MEGA_PART_NB
-#define MEGA_PART_NB 11
-#endif
 #define MEGA_PT MEGA_THREADS                        // polling threads
 // SWZ_EPL: layout of dst (0 plain order, else xs_chunk_pos(., SWZ_EPL)); NB: slots a thread requests
 // before it looks at the first one (every further group of NB costs another round trip).
@@ -231,19 +234,12 @@ template <int WT> struct MegaStage {
     uint32_t sc[2][2];       // int4 group scales (bf16 bits)
 };
 
-// BIGPART: the attention partials (heads x splits records) are more than one request group of the
-// ordinary poll: wait for them with MEGA_PART_NB slots per thread in flight instead (5B: one round
-// trip instead of three, 2.79 -> 2.74 ms per token).  A template parameter, chosen by the host per
-// launch from heads x splits at the current position, because the poll routine's register footprint and a further call site shift the
-// code of the small models (600M: -0.4 % with the wide poll, -3 % with a run-time choice).
-// VAR selects one of three builds of the kernel: MEGA_VAR_PLAIN (ordinary partials poll, no time
-// stamps: the stamp code, although never executed without a profile buffer, costs the 600M step 1.7 %
-// in registers and branches), MEGA_VAR_STAMPS (the same with time stamps, for the step profile) and
-// MEGA_VAR_BIGPART (wide partials poll; keeps the stamp code, which there costs nothing measurable).
-enum { MEGA_VAR_PLAIN = 0, MEGA_VAR_STAMPS = 1, MEGA_VAR_BIGPART = 2 };
+// VAR selects one of two builds of the kernel: MEGA_VAR_PLAIN (no time stamps: the stamp code, although
+// never executed without a profile buffer, costs the 600M step 1.7 % in registers and branches) and
+// MEGA_VAR_STAMPS (the same with time stamps, for the step profile).
+enum { MEGA_VAR_PLAIN = 0, MEGA_VAR_STAMPS = 1 };
 template <int WT, int KVBF16, int HD, int VAR>
 __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
-    constexpr int BIGPART = VAR == MEGA_VAR_BIGPART;
     constexpr int EPL = WS<WT>::EPL;
     constexpr int KESZ = KVBF16 ? 2 : 4;
     constexpr int KEPL = 16 / KESZ;
@@ -268,8 +264,8 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     // vector while another already stages phase p+1's.  Even phases (qkv, w13, head) read D floats,
     // odd phases (wo, w2) max(Q, H).
     float *xsb = smem;                                       // [D] then [max(Q, H)]
-    float *stage = xsb + D + max(Q, H);                      // attention partials / slots
-    const int stage_floats = max(a.heads * a.ns_max * REC, SLOTS * REC + 3 * HD);
+    float *stage = xsb + D + max(Q, H);                      // attention: per-wave partials, q / k / v of the new token; odd phases: per-task sums
+    const int stage_floats = a.stage_floats;                 // host: max(MEGA_WAVES * REC + 3 * HD, 2 * tasks of an odd phase)
     const int xres_n = 2 * ((D / 2 + G - 1) / G) + 2;
     float *xresb = stage + stage_floats;                     // [2][xres_n] residual inputs of this workgroup's wo / w2 rows
     float *ropes = xresb + 2 * xres_n;                       // (cos, sin) of this workgroup's q/k row pairs
@@ -353,32 +349,44 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         e_left = npl > wave ? ((npl - wave + MEGA_WAVES - 1) / MEGA_WAVES) * kinds[kind].segs : 0;
         e_pl = wave; e_sg = 0;
     };
-    auto issue_even = [&](int ph) {
+    struct IssueCtx {                                        // what the loads of one phase's rounds need
+        int pieces, segs, pair0, kg;
+        size_t rb;
+        const char *W;
+        const uint16_t *SC;
+    };
+    auto prep_issue = [&](int ph) {
         const int kind = ph == 4 * L ? MK_HEAD : (ph & 3);
         const MegaKind &k = kinds[kind];
-        const int p_pieces = k.pieces, p_segs = k.segs, p_pair0 = k.pair0, p_kg = k.K / 128;
-        const size_t p_rb = k.row_bytes;
-        const char *p_W = kind == MK_HEAD ? (const char *)a.embed : (const char *)lptr[(ph >> 2) * MEGA_LPTR + kind];
-        const uint16_t *p_SC = kind == MK_HEAD ? nullptr : (const uint16_t *)lptr[(ph >> 2) * MEGA_LPTR + 4 + kind];
+        IssueCtx c;
+        c.pieces = k.pieces; c.segs = k.segs; c.pair0 = k.pair0; c.kg = k.K / 128; c.rb = k.row_bytes;
+        c.W = kind == MK_HEAD ? (const char *)a.embed : (const char *)lptr[(ph >> 2) * MEGA_LPTR + kind];
+        c.SC = kind == MK_HEAD ? nullptr : (const uint16_t *)lptr[(ph >> 2) * MEGA_LPTR + 4 + kind];
+        return c;
+    };
+    // the next task of set A's cursor into t
+    auto issue_even_one = [&](const IssueCtx &c, MegaStage<WT> &t) {
+        if (e_left > 0) {
+            const size_t row = (size_t)2 * (c.pair0 + e_pl);
 #pragma unroll
-        for (int s = 0; s < MEGA_DEPTH; ++s) {
-            if (e_left > 0) {
-                const size_t row = (size_t)2 * (p_pair0 + e_pl);
+            for (int j = 0; j < 2; ++j) {
+                const int piece = e_sg * MEGA_SEG_PIECES + j * 64 + lane;
+                if (piece < c.pieces) {
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int piece = e_sg * MEGA_SEG_PIECES + j * 64 + lane;
-                    if (piece < p_pieces) {
-#pragma unroll
-                        for (int r = 0; r < 2; ++r) {
-                            stA[s].w[r][j] = ld_stream_u4(p_W + (row + r) * p_rb + (size_t)piece * 16);
-                            if (WT == WT_INT4) stA[s].sc[r][j] = ldg_u16(p_SC + (row + r) * p_kg + (piece >> 2));   // 4-bit models keep the head outside
-                        }
+                    for (int r = 0; r < 2; ++r) {
+                        t.w[r][j] = ld_stream_u4(c.W + (row + r) * c.rb + (size_t)piece * 16);
+                        if (WT == WT_INT4) t.sc[r][j] = ldg_u16(c.SC + (row + r) * c.kg + (piece >> 2));   // 4-bit models keep the head outside
                     }
                 }
-                --e_left;
-                if (++e_sg == p_segs) { e_sg = 0; e_pl += MEGA_WAVES; }
             }
+            --e_left;
+            if (++e_sg == c.segs) { e_sg = 0; e_pl += MEGA_WAVES; }
         }
+    };
+    auto issue_even = [&](int ph) {
+        const IssueCtx c = prep_issue(ph);
+#pragma unroll
+        for (int s = 0; s < MEGA_DEPTH; ++s) issue_even_one(c, stA[s]);
     };
     auto start_odd = [&](int ph) {
         const MegaKind &k = kinds[ph & 3];
@@ -386,33 +394,29 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         o_pl = 0; o_sg = wave;
         while (o_sg >= k.segs) { o_sg -= k.segs; ++o_pl; }
     };
-    auto issue_odd = [&](int ph) {
-        const int kind = ph & 3;
-        const MegaKind &k = kinds[kind];
-        const int p_pieces = k.pieces, p_segs = k.segs, p_pair0 = k.pair0, p_kg = k.K / 128;
-        const size_t p_rb = k.row_bytes;
-        const char *p_W = (const char *)lptr[(ph >> 2) * MEGA_LPTR + kind];
-        const uint16_t *p_SC = (const uint16_t *)lptr[(ph >> 2) * MEGA_LPTR + 4 + kind];
+    auto issue_odd_one = [&](const IssueCtx &c, MegaStage<WT> &t) {
+        if (o_left > 0) {
+            const size_t row = (size_t)2 * (c.pair0 + o_pl);
 #pragma unroll
-        for (int s = 0; s < MEGA_DEPTH_B; ++s) {
-            if (o_left > 0) {
-                const size_t row = (size_t)2 * (p_pair0 + o_pl);
+            for (int j = 0; j < 2; ++j) {
+                const int piece = o_sg * MEGA_SEG_PIECES + j * 64 + lane;
+                if (piece < c.pieces) {
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int piece = o_sg * MEGA_SEG_PIECES + j * 64 + lane;
-                    if (piece < p_pieces) {
-#pragma unroll
-                        for (int r = 0; r < 2; ++r) {
-                            stB[s].w[r][j] = ld_stream_u4(p_W + (row + r) * p_rb + (size_t)piece * 16);
-                            if (WT == WT_INT4) stB[s].sc[r][j] = ldg_u16(p_SC + (row + r) * p_kg + (piece >> 2));
-                        }
+                    for (int r = 0; r < 2; ++r) {
+                        t.w[r][j] = ld_stream_u4(c.W + (row + r) * c.rb + (size_t)piece * 16);
+                        if (WT == WT_INT4) t.sc[r][j] = ldg_u16(c.SC + (row + r) * c.kg + (piece >> 2));
                     }
                 }
-                --o_left;
-                o_sg += MEGA_WAVES;
-                while (o_sg >= p_segs) { o_sg -= p_segs; ++o_pl; }
             }
+            --o_left;
+            o_sg += MEGA_WAVES;
+            while (o_sg >= c.segs) { o_sg -= c.segs; ++o_pl; }
         }
+    };
+    auto issue_odd = [&](int ph) {
+        const IssueCtx c = prep_issue(ph);
+#pragma unroll
+        for (int s = 0; s < MEGA_DEPTH_B; ++s) issue_odd_one(c, stB[s]);
     };
     // one task: both rows of a pair times the staged vector over one segment
     auto mul_task = [&](const MegaStage<WT> &t, const float *xs, const int sg, const int pieces, float &o0, float &o1) {
@@ -449,10 +453,12 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0)
     start_even(0);
     issue_even(0);
+    o_left = 0;
+    if (1 <= last_ph) { start_odd(1); issue_odd_one(prep_issue(1), stB[0]); }
 
     const int wo_row0 = 2 * kinds[MK_WO].pair0, wo_rows = 2 * kinds[MK_WO].npl;   // same partition for w2
     const int n_att = pos + 1;
-    int NS = (n_att + SLOTS * PRE - 1) / (SLOTS * PRE);
+    int NS = (n_att + SLOTS * MEGA_ATT_SPLIT_PASSES - 1) / (SLOTS * MEGA_ATT_SPLIT_PASSES);
     NS = max(1, min(NS, a.ns_max));
     const int chunk = (n_att + NS - 1) / NS;
     const float att_scale = 1.0f / sqrtf((float)HD);
@@ -505,8 +511,12 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         // anyway).  The explicit wait tells the compiler so: from here on only the loads requested below
         // are outstanding, and the multiply of set A runs without waiting for them.
         __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
-        // the odd phase behind this one gets its first round now
-        if (ph + 1 <= last_ph) { start_odd(ph + 1); issue_odd(ph + 1); }
+        // Requests are spread over the phases, one task (four loads per lane) at a time, so that each one
+        // finds room in the memory pipeline: requested in one block, a round holds the wave at the
+        // address unit for a good part of the time the block takes to stream.  Here: the second task of
+        // the odd phase behind this one (its first went out at the end of the odd phase before).
+#pragma unroll
+        for (int s = 1; s < MEGA_DEPTH_B; ++s) issue_odd_one(prep_issue(ph + 1 <= last_ph ? ph + 1 : ph), stB[s]);
         float inv;
         {
             float t = 0.0f;
@@ -605,6 +615,9 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             for (int i = MEGA_DEPTH; i < nm; i += MEGA_DEPTH) even_round(i);
         }
         mark();
+        // set A is free: the first task of the next even phase
+        e_left = 0;
+        if (ph + 2 <= last_ph) { start_even(ph + 2); issue_even_one(prep_issue(ph + 2), stA[0]); }
         if (kind == MK_HEAD) {
             // the eight per-wave candidates meet in LDS; wave 0 publishes the workgroup's best
             if (lane == 63) { s_cand_v[wave] = bv; s_cand_i[wave] = bi; }
@@ -639,7 +652,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         if (kind == MK_WO && b < a.heads * NS) {
             const int sidx = b / a.heads, h = b - sidx * a.heads, g = h / a.gqa;
             const int t0 = sidx * chunk, t1 = min(n_att, t0 + chunk);
-            float *qs = stage + SLOTS * REC, *kcur = qs + HD, *vcur = kcur + HD;
+            float *qs = stage + MEGA_WAVES * REC, *kcur = qs + HD, *vcur = kcur + HD;
             const int sub = tid % LPR, slot = tid / LPR;
             const char *kb = (const char *)kcl + ((size_t)g * HD + sub * KEPL) * KESZ;
             const char *vb = (const char *)vcl + ((size_t)g * HD + sub * KEPL) * KESZ;
@@ -732,15 +745,31 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                     }
                 }
             }
+            // the slots of a wave first (lanes o apart hold the same channels of two slots), then the
+            // eight per-wave partials through LDS
 #pragma unroll
-            for (int e = 0; e < KEPL; ++e) stage[slot * REC + sub * KEPL + e] = acc[e];
-            if (sub == 0) { stage[slot * REC + HD] = m; stage[slot * REC + HD + 1] = lsum; }
+            for (int o = LPR; o < 64; o <<= 1) {
+                const float m2 = __shfl_xor(m, o, WAVE), l2 = __shfl_xor(lsum, o, WAVE);
+                const float mn = fmaxf(m, m2);
+                const float e1 = __expf(m - mn), e2 = __expf(m2 - mn);
+                lsum = lsum * e1 + l2 * e2;
+#pragma unroll
+                for (int e = 0; e < KEPL; ++e) acc[e] = acc[e] * e1 + __shfl_xor(acc[e], o, WAVE) * e2;
+                m = mn;
+            }
+            if (lane < LPR) {
+#pragma unroll
+                for (int e = 0; e < KEPL; ++e) stage[wave * REC + lane * KEPL + e] = acc[e];
+                if (lane == 0) { stage[wave * REC + HD] = m; stage[wave * REC + HD + 1] = lsum; }
+            }
             lds_barrier();
             if (tid < HD) {
                 float M = -1e30f;
-                for (int k2 = 0; k2 < SLOTS; ++k2) M = fmaxf(M, stage[k2 * REC + HD]);
+#pragma unroll
+                for (int k2 = 0; k2 < MEGA_WAVES; ++k2) M = fmaxf(M, stage[k2 * REC + HD]);
                 float Ls = 0.0f, A = 0.0f;
-                for (int k2 = 0; k2 < SLOTS; ++k2) {
+#pragma unroll
+                for (int k2 = 0; k2 < MEGA_WAVES; ++k2) {
                     const float w = __expf(stage[k2 * REC + HD] - M);
                     Ls += stage[k2 * REC + HD + 1] * w;
                     A += stage[k2 * REC + tid] * w;
@@ -762,18 +791,53 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             }
         }
 
-        // ---- stage this phase's input: the attention partials (wo) or the gate vector (w2)
+        // ---- stage this phase's input: the folded attention partials (wo) or the gate vector (w2)
+        if (MEGA_DEPTH > 1) issue_even_one(prep_issue(oph + 1 <= last_ph ? oph + 1 : oph), stA[1]);
         {
             bool ok = true;
-            float ss;
             if (kind == MK_WO) {
-                const int n = NS * a.heads * REC;
-                if (BIGPART) ss = mega_poll_vec<0, MEGA_PART_NB, false>(a.PART, n, par, abortf, stage, nullptr, xresb, wo_row0, 0, pt);
-                else ss = mega_poll_vec<0>(a.PART, n, par, abortf, stage, nullptr, xresb, wo_row0, 0, pt);
+                // Thread c folds four neighbouring channels of the attention output: from every split's
+                // record it polls those four sums and the record's (maximum, sum of weights), four splits
+                // in flight at a time, and merges them in split order as the softmax of the whole sequence
+                // would weigh them.  No staging of the records, no pass over them by a few threads, no
+                // barrier before the fold.
+                const unsigned pm = par ? 0xffffffffu : 0u;
+                const __amdgpu_buffer_rsrc_t r = make_rsrc(a.PART, NS * a.heads * REC * 4);
+                for (int c = tid; c < Q / 4 && ok; c += MEGA_THREADS) {
+                    const int h = (4 * c) / HD, j = 4 * c - h * HD;
+                    float M = -1e30f, Ls = 0.0f, o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
+                    for (int s0 = 0; s0 < NS && ok; s0 += 4) {
+                        mega_u4 va[4], vt[4];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const int off = ((min(s0 + q, NS - 1) * a.heads + h) * REC) * 4;
+                            va[q] = ld16_coherent(r, off + j * 4);
+                            vt[q] = ld16_coherent(r, off + HD * 4);
+                        }
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            if (s0 + q < NS && ok) {
+                                const int off = (((s0 + q) * a.heads + h) * REC) * 4;
+                                ok = repoll16(va[q], r, off + j * 4, pm, abortf) && repoll16(vt[q], r, off + HD * 4, pm, abortf);
+                                const float ms = __uint_as_float(vt[q].x & ~1u), ls = __uint_as_float(vt[q].y & ~1u);
+                                const float mn = fmaxf(M, ms);
+                                const float e1 = __expf(M - mn), e2 = __expf(ms - mn);
+                                Ls = Ls * e1 + ls * e2;
+                                o0 = o0 * e1 + __uint_as_float(va[q].x & ~1u) * e2;
+                                o1 = o1 * e1 + __uint_as_float(va[q].y & ~1u) * e2;
+                                o2 = o2 * e1 + __uint_as_float(va[q].z & ~1u) * e2;
+                                o3 = o3 * e1 + __uint_as_float(va[q].w & ~1u) * e2;
+                                M = mn;
+                            }
+                        }
+                    }
+                    const float rl = Ls > 0.0f ? 1.0f / Ls : 0.0f;
+                    *(float4 *)(xs + 4 * xs_chunk_pos(c, XSWZ)) = make_float4(o0 * rl, o1 * rl, o2 * rl, o3 * rl);
+                }
             } else {
-                ss = mega_poll_vec<XSWZ>(a.GATE, H, par, abortf, xs, nullptr, xresb, wo_row0, 0, pt);
+                const float ss = mega_poll_vec<XSWZ>(a.GATE, H, par, abortf, xs, nullptr, xresb, wo_row0, 0, pt);
+                if (ss < 0.0f) ok = false;
             }
-            if (ss < 0.0f) ok = false;
             if (!ok) s_bad = 1;
             lds_barrier();
             if (s_bad) return;
@@ -782,58 +846,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         // this phase's input and set B are here (see the even phase): the even phase behind it gets its
         // first round now
         __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
-        if (oph + 1 <= last_ph) { start_even(oph + 1); issue_even(oph + 1); }
-        if (kind == MK_WO) {
-            // fold the split partials of every head into the attention output vector
-            const int sstride = a.heads * REC;
-            if (tid < a.heads) {          // per head: the weight of each split, exp(m_s - M) / L
-                float *hp2 = stage + tid * REC;
-                float M = -1e30f;
-                for (int s = 0; s < NS; ++s) M = fmaxf(M, hp2[s * sstride + HD]);
-                float Ls = 0.0f;
-                for (int s = 0; s < NS; ++s) Ls += hp2[s * sstride + HD + 1] * __expf(hp2[s * sstride + HD] - M);
-                const float rl = Ls > 0.0f ? 1.0f / Ls : 0.0f;
-                for (int s = 0; s < NS; ++s) hp2[s * sstride + HD + 2] = __expf(hp2[s * sstride + HD] - M) * rl;
-            }
-            lds_barrier();
-            if constexpr (BIGPART) {
-            // many splits and heads: four outputs of a thread side by side (each sums its splits in
-            // order), eight LDS reads in flight per split instead of two (5B +0.6 ... 1.6 %; the 600M
-            // step loses 1 % with it and keeps the plain loop)
-            for (int i0 = tid; i0 < Q; i0 += 4 * MEGA_THREADS) {
-                const float *pv[4], *pw[4];
-                float A[4];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const int i = min(i0 + c * MEGA_THREADS, Q - 1);
-                    const int h = i / HD, j = i - h * HD;
-                    pv[c] = stage + h * REC + j;
-                    pw[c] = stage + h * REC + HD + 2;
-                    A[c] = 0.0f;
-                }
-                for (int s = 0; s < NS; ++s) {
-                    float v[4], w[4];
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) { v[c] = pv[c][s * sstride]; w[c] = pw[c][s * sstride]; }
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) A[c] = fmaf(v[c], w[c], A[c]);
-                }
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    if (i0 + c * MEGA_THREADS < Q) xs[xs_pos(i0 + c * MEGA_THREADS, XSWZ)] = A[c];
-            }
-            } else {
-            for (int i = tid; i < Q; i += MEGA_THREADS) {
-                const int h = i / HD, j = i - h * HD;
-                const float *hp2 = stage + h * REC;
-                float A = 0.0f;
-                for (int s = 0; s < NS; ++s) A = fmaf(hp2[s * sstride + j], hp2[s * sstride + HD + 2], A);
-                xs[xs_pos(i, XSWZ)] = A;
-            }
-            }
-            lds_barrier();
-            mark();
-        }
+        if (MEGA_DEPTH > 2) issue_even_one(prep_issue(oph + 1 <= last_ph ? oph + 1 : oph), stA[2]);
 
         // ---- stream this workgroup's rows: wave w multiplies tasks w, w + 8, ... in rounds of MEGA_DEPTH_B
         // and leaves each task's two sums in LDS (the staging area of the partials is free by now)
@@ -882,6 +895,11 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             // (the next writer of the staging area is the next attention phase or this loop's next round
             // of sums, both behind a barrier of the phases in between)
         }
+        // the rest of the next even phase's first round, and (set B is free) the first task of the next odd phase
+#pragma unroll
+        for (int s = 3; s < MEGA_DEPTH; ++s) issue_even_one(prep_issue(oph + 1 <= last_ph ? oph + 1 : oph), stA[s]);
+        o_left = 0;
+        if (oph + 2 <= last_ph) { start_odd(oph + 2); issue_odd_one(prep_issue(oph + 2), stB[0]); }
         mark();
         mark();
         }
