@@ -343,12 +343,6 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     int o_left = 0, o_pl = 0, o_sg = 0;                      // cursor of set B
     // Lanes past the end of a row and padding tasks issue nothing (a skipped load is not free if it
     // is issued anyway: it still occupies the address unit) and are ignored when the round is consumed.
-    auto start_even = [&](int ph) {
-        const int kind = ph == 4 * L ? MK_HEAD : (ph & 3);
-        const int npl = kinds[kind].npl;
-        e_left = npl > wave ? ((npl - wave + MEGA_WAVES - 1) / MEGA_WAVES) * kinds[kind].segs : 0;
-        e_pl = wave; e_sg = 0;
-    };
     struct IssueCtx {                                        // what the loads of one phase's rounds need
         int pieces, segs, pair0, kg;
         size_t rb;
@@ -363,6 +357,14 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         c.W = kind == MK_HEAD ? (const char *)a.embed : (const char *)lptr[(ph >> 2) * MEGA_LPTR + kind];
         c.SC = kind == MK_HEAD ? nullptr : (const uint16_t *)lptr[(ph >> 2) * MEGA_LPTR + 4 + kind];
         return c;
+    };
+    IssueCtx ctxA = prep_issue(0), ctxB = prep_issue(0);     // of the phase each cursor walks
+    auto start_even = [&](int ph) {
+        const int kind = ph == 4 * L ? MK_HEAD : (ph & 3);
+        const int npl = kinds[kind].npl;
+        e_left = npl > wave ? ((npl - wave + MEGA_WAVES - 1) / MEGA_WAVES) * kinds[kind].segs : 0;
+        e_pl = wave; e_sg = 0;
+        ctxA = prep_issue(ph);
     };
     // the next task of set A's cursor into t
     auto issue_even_one = [&](const IssueCtx &c, MegaStage<WT> &t) {
@@ -383,16 +385,16 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             if (++e_sg == c.segs) { e_sg = 0; e_pl += MEGA_WAVES; }
         }
     };
-    auto issue_even = [&](int ph) {
-        const IssueCtx c = prep_issue(ph);
+    auto issue_even = [&]() {
 #pragma unroll
-        for (int s = 0; s < MEGA_DEPTH; ++s) issue_even_one(c, stA[s]);
+        for (int s = 0; s < MEGA_DEPTH; ++s) issue_even_one(ctxA, stA[s]);
     };
     auto start_odd = [&](int ph) {
         const MegaKind &k = kinds[ph & 3];
         o_left = k.ntasks > wave ? (k.ntasks - wave + MEGA_WAVES - 1) / MEGA_WAVES : 0;
         o_pl = 0; o_sg = wave;
         while (o_sg >= k.segs) { o_sg -= k.segs; ++o_pl; }
+        ctxB = prep_issue(ph);
     };
     auto issue_odd_one = [&](const IssueCtx &c, MegaStage<WT> &t) {
         if (o_left > 0) {
@@ -413,10 +415,9 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             while (o_sg >= c.segs) { o_sg -= c.segs; ++o_pl; }
         }
     };
-    auto issue_odd = [&](int ph) {
-        const IssueCtx c = prep_issue(ph);
+    auto issue_odd = [&]() {
 #pragma unroll
-        for (int s = 0; s < MEGA_DEPTH_B; ++s) issue_odd_one(c, stB[s]);
+        for (int s = 0; s < MEGA_DEPTH_B; ++s) issue_odd_one(ctxB, stB[s]);
     };
     // one task: both rows of a pair times the staged vector over one segment
     auto mul_task = [&](const MegaStage<WT> &t, const float *xs, const int sg, const int pieces, float &o0, float &o1) {
@@ -452,9 +453,9 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     // includes the weights requested for the phase.
     __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0)
     start_even(0);
-    issue_even(0);
+    issue_even();
     o_left = 0;
-    if (1 <= last_ph) { start_odd(1); issue_odd_one(prep_issue(1), stB[0]); }
+    if (1 <= last_ph) { start_odd(1); issue_odd_one(ctxB, stB[0]); }
 
     const int wo_row0 = 2 * kinds[MK_WO].pair0, wo_rows = 2 * kinds[MK_WO].npl;   // same partition for w2
     const int n_att = pos + 1;
@@ -516,7 +517,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         // address unit for a good part of the time the block takes to stream.  Here: the second task of
         // the odd phase behind this one (its first went out at the end of the odd phase before).
 #pragma unroll
-        for (int s = 1; s < MEGA_DEPTH_B; ++s) issue_odd_one(prep_issue(ph + 1 <= last_ph ? ph + 1 : ph), stB[s]);
+        for (int s = 1; s < MEGA_DEPTH_B; ++s) issue_odd_one(ctxB, stB[s]);
         float inv;
         {
             float t = 0.0f;
@@ -526,7 +527,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         }
 
         // ---- stream this workgroup's rows in rounds of MEGA_DEPTH tasks
-        float bv = -INFINITY; uint32_t bi = 0x7fffffffu;      // head phase: best logit seen by this wave (lane 63)
+        float bv = -INFINITY; uint32_t bi = 0x7fffffffu;      // head phase: best logit this lane has finished
         {
             const MegaKind k = kinds[kind];
             const int nm = k.npl > wave ? ((k.npl - wave + MEGA_WAVES - 1) / MEGA_WAVES) * k.segs : 0;
@@ -552,16 +553,29 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                 if (i == 0) mark();
                 // inside a phase the next round is requested before the sums are finished (its latency
                 // overlaps them); the next phase's rounds belong to the odd phase in between
-                if (i + MEGA_DEPTH < nm) issue_even(ph);
+                if (i + MEGA_DEPTH < nm) issue_even();
+                float fin0 = 0.0f, fin1 = 0.0f;
+                int fin_p = 0, n_fin = 0;
 #pragma unroll
                 for (int s = 0; s < MEGA_DEPTH; ++s) {
                   if (i + s < nm) {
                     run0 += acc[s][0]; run1 += acc[s][1];
                     if (++c_sg == k.segs) {
-                      float s0 = wave_sum_dpp(run0), s1 = wave_sum_dpp(run1);
-                      const int p = c_pl;
+                      // a finished pair: its two sums go to lane n_fin; the pairs of a round are finished
+                      // side by side in different lanes, after the round's last task
+                      const float t0 = wave_sum_dpp(run0), t1 = wave_sum_dpp(run1);
+                      const float b0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(t0), 63));
+                      const float b1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(t1), 63));
+                      if (lane == n_fin) { fin0 = b0; fin1 = b1; fin_p = c_pl; }
+                      ++n_fin;
                       run0 = 0.0f; run1 = 0.0f; c_sg = 0; c_pl += MEGA_WAVES;
-                      if (lane == 63) {
+                    }
+                  }
+                }
+                if (lane < n_fin) {
+                      float s0 = fin0, s1 = fin1;
+                      const int p = fin_p;
+                      {
                 const int row0 = 2 * (k.pair0 + p);
                 if (fsc) { s0 *= fsc[row0]; s1 *= fsc[row0 + 1]; }
                 if (kind == MK_QKV) {
@@ -603,8 +617,6 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                     if (better(s1, (uint32_t)row0 + 1, bv, bi)) { bv = s1; bi = (uint32_t)row0 + 1; }
                 }
                       }
-                    }
-                  }
                 }
             };
             // The first round is taken outside the loop: it runs straight behind the request of the odd
@@ -615,12 +627,10 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             for (int i = MEGA_DEPTH; i < nm; i += MEGA_DEPTH) even_round(i);
         }
         mark();
-        // set A is free: the first task of the next even phase
-        e_left = 0;
-        if (ph + 2 <= last_ph) { start_even(ph + 2); issue_even_one(prep_issue(ph + 2), stA[0]); }
         if (kind == MK_HEAD) {
             // the eight per-wave candidates meet in LDS; wave 0 publishes the workgroup's best
-            if (lane == 63) { s_cand_v[wave] = bv; s_cand_i[wave] = bi; }
+            wave_argbest(bv, bi);                             // (each finishing lane kept its own best)
+            if (lane == 0) { s_cand_v[wave] = bv; s_cand_i[wave] = bi; }
             lds_barrier();
             if (wave == 0) {
                 float cv = lane < MEGA_WAVES ? s_cand_v[lane] : -INFINITY;
@@ -792,7 +802,13 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         }
 
         // ---- stage this phase's input: the folded attention partials (wo) or the gate vector (w2)
-        if (MEGA_DEPTH > 1) issue_even_one(prep_issue(oph + 1 <= last_ph ? oph + 1 : oph), stA[1]);
+        // Set A is free since the even phase's last round: the first two tasks of the next even phase go
+        // out here, behind the attention (the workgroups that attend are the ones every other workgroup
+        // waits for; nothing that can wait is put in front of their work).
+        e_left = 0;
+        if (oph + 1 <= last_ph) start_even(oph + 1);
+        issue_even_one(ctxA, stA[0]);
+        if (MEGA_DEPTH > 1) issue_even_one(ctxA, stA[1]);
         {
             bool ok = true;
             if (kind == MK_WO) {
@@ -846,7 +862,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         // this phase's input and set B are here (see the even phase): the even phase behind it gets its
         // first round now
         __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
-        if (MEGA_DEPTH > 2) issue_even_one(prep_issue(oph + 1 <= last_ph ? oph + 1 : oph), stA[2]);
+        if (MEGA_DEPTH > 2) issue_even_one(ctxA, stA[2]);
 
         // ---- stream this workgroup's rows: wave w multiplies tasks w, w + 8, ... in rounds of MEGA_DEPTH_B
         // and leaves each task's two sums in LDS (the staging area of the partials is free by now)
@@ -870,7 +886,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                     }
                 }
                 if (i == 0) mark();
-                if (i + MEGA_DEPTH_B < nm) issue_odd(oph);
+                if (i + MEGA_DEPTH_B < nm) issue_odd();
 #pragma unroll
                 for (int s = 0; s < MEGA_DEPTH_B; ++s) {
                     if (i + s < nm) {
@@ -897,9 +913,9 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         }
         // the rest of the next even phase's first round, and (set B is free) the first task of the next odd phase
 #pragma unroll
-        for (int s = 3; s < MEGA_DEPTH; ++s) issue_even_one(prep_issue(oph + 1 <= last_ph ? oph + 1 : oph), stA[s]);
+        for (int s = 3; s < MEGA_DEPTH; ++s) issue_even_one(ctxA, stA[s]);
         o_left = 0;
-        if (oph + 2 <= last_ph) { start_odd(oph + 2); issue_odd_one(prep_issue(oph + 2), stB[0]); }
+        if (oph + 2 <= last_ph) { start_odd(oph + 2); issue_odd_one(ctxB, stB[0]); }
         mark();
         mark();
         }
