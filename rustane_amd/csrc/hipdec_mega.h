@@ -35,7 +35,9 @@
 #define MEGA_SPIN_LIMIT (1u << 22)
 #define MEGA_PREC 4             // attention partial record = HD + 4 floats (acc[HD], max, sum, 0, 0)
 #define MEGA_PROF_SLOTS 32      // timestamps per layer when profiling
+#ifndef MEGA_ATT_PRE
 #define MEGA_ATT_PRE 4          // attention: cache-row passes a thread requests ahead
+#endif
 #ifndef MEGA_ATT_SPLIT_PASSES
 #define MEGA_ATT_SPLIT_PASSES 4 // attention: passes (of 512 / lanes-per-row cache rows) one split covers while splits are to be had
                                 // (600M at 256 positions: 1 pass 0.591, 2 passes 0.573, 4 passes 0.556, 8 passes 0.575 ms per token:
@@ -255,7 +257,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     __shared__ uint32_t s_cand_i[MEGA_WAVES];
     __shared__ int s_bad;                       // set once by any thread whose wait was aborted
 
-    const int tid = threadIdx.x, lane = tid & 63;
+    int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: per-wave bookkeeping stays on the scalar unit
     if (tid == 0) s_bad = 0;
     const int G = gridDim.x, b = blockIdx.x;
@@ -466,6 +468,9 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     const unsigned par_c = (ep_head + 1u) & 1u;
 
     for (int ph = 0; ph <= last_ph; ph += 2) {
+        // The thread's index is made opaque here, so that nothing derived from it (addresses, lane
+        // masks) is kept in registers across the phases; recomputing is a few instructions per use.
+        asm volatile("" : "+v"(tid), "+v"(lane));
         // ===================================================================== even phase: qkv, w13 or head
         {
         const int l = min(ph >> 2, L - 1);
@@ -548,6 +553,9 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                         const int sg = f_sg;
                         if (++f_sg == k.segs) f_sg = 0;
                         mul_task(stA[s], xs, sg, k.pieces, acc[s][0], acc[s][1]);
+                        // Tasks are not interleaved: the operands of four tasks side by side take more
+                        // registers than the two weight sets leave, and the scheduler would take them.
+                        __builtin_amdgcn_sched_barrier(0);
                     }
                 }
                 if (i == 0) mark();
@@ -881,6 +889,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
                     slot_t[s] = f_t;
                     if (i + s < nm) {
                         mul_task(stB[s], xs, f_sg, k.pieces, acc[s][0], acc[s][1]);
+                        __builtin_amdgcn_sched_barrier(0);
                         f_t += MEGA_WAVES; f_sg += MEGA_WAVES;
                         while (f_sg >= k.segs) f_sg -= k.segs;
                     }
