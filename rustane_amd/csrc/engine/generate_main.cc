@@ -69,6 +69,22 @@ bool model_from_name(const std::string &name, ModelConfig *cfg) {
     return true;
 }
 
+// a float as the reference's "{}" prints it: the shortest decimal that reads back as the same f32, never an exponent
+std::string format_f32(float v) {
+    char buf[64];
+    for (int p = 1; p <= 9; ++p) {
+        snprintf(buf, sizeof buf, "%.*g", p, (double)v);
+        if (strtof(buf, nullptr) == v) break;
+    }
+    if (strchr(buf, 'e') || strchr(buf, 'E')) {
+        snprintf(buf, sizeof buf, "%.12f", (double)v);
+        size_t n = strlen(buf);
+        while (n > 1 && buf[n - 1] == '0') buf[--n] = 0;
+        if (n > 1 && buf[n - 1] == '.') buf[--n] = 0;
+    }
+    return buf;
+}
+
 std::string format_ids(const std::vector<uint32_t> &ids) {
     std::string s;
     for (size_t i = 0; i < ids.size(); ++i) { if (i) s += ","; s += std::to_string(ids[i]); }
@@ -142,16 +158,34 @@ int main(int argc, char **argv) {
     }
     if (prompt.empty()) fail("pass --prompt-ids or --random-prompt");
 
-    if (!jsonl_session)
+    if (!jsonl_session && checkpoint.empty())        // (a synthetic model has no "loaded checkpoint" line: its shape instead)
         printf("model=%s dim=%zu hidden=%zu heads=%zu hd=%zu nlayers=%zu seq=%zu vocab=%zu params=%zu\n", model.c_str(),
                cfg.dim, cfg.hidden, cfg.heads, cfg.hd, cfg.nlayers, cfg.seq, cfg.vocab, cfg.param_count());
-    DecodeSelection planned = select_decode_mode(cfg, req.decode_backend, prompt.size() < cfg.seq ? prompt.size() : cfg.seq,
-                                                 req.steps);
-    if (!jsonl_session) {
-        printf("decode_backend_request=%s decode_mode=%s", decode_backend_str(req.decode_backend), decode_mode_str(planned.mode));
-        if (planned.fallback_reason) printf(" fallback_reason=%s", planned.fallback_reason);
-        if (planned.auto_reason) printf(" auto_reason=%s", planned.auto_reason);
-        printf("\n");
+    const size_t effective_context_len = prompt.size() < cfg.seq ? prompt.size() : cfg.seq;         // generate.rs:519
+    DecodeSelection planned = select_decode_mode(cfg, req.decode_backend, effective_context_len, req.steps);
+    const bool greedy_sampling = req.temperature <= 0.0f || req.top_k == 1;                          // generate.rs:522
+    if (!jsonl_session) {                                                                            // generate.rs:524-566
+        printf("prompt_len=%zu effective_context_len=%zu steps=%zu temperature=%s top_k=%zu decode_backend_request=%s "
+               "decode_mode=%s greedy_sampling=%s\n",
+               prompt.size(), effective_context_len, req.steps, format_f32(req.temperature).c_str(), req.top_k,
+               decode_backend_str(req.decode_backend), decode_mode_str(planned.mode), greedy_sampling ? "true" : "false");
+        if (prompt.size() > cfg.seq) printf("prompt_truncated=true kept_last_tokens=%zu\n", effective_context_len);
+        if (planned.auto_reason)         // (the threshold keeps the reference's key: log readers look for it)
+            printf("decode_backend_auto_reason=%s model_params=%zu auto_metal_threshold=%zu\n", planned.auto_reason,
+                   cfg.param_count(), AUTO_KV_PARAM_THRESHOLD);
+        if (planned.fallback_reason) printf("decode_backend_fallback=true reason=%s\n", planned.fallback_reason);
+        printf("samples=%zu prefix_reuse=%s\n", req.samples, req.samples > 1 ? "enabled" : "disabled");
+        if (planned.mode == DecodeMode::KvCacheHip && !greedy_sampling) {                            // generate.rs:312-333
+            if (req.top_k > 0) {
+                if (req.top_k <= MAX_GPU_TOPK)
+                    printf("cached_sampling_path=gpu_topk_candidates top_k=%zu gpu_topk_capacity=%zu\n", req.top_k, MAX_GPU_TOPK);
+                else
+                    printf("cached_sampling_path=full_logits_cpu_sample reason=top_k_exceeds_gpu_capacity requested_top_k=%zu "
+                           "gpu_topk_capacity=%zu\n", req.top_k, MAX_GPU_TOPK);
+            } else {
+                printf("cached_sampling_path=gpu_block_stats_exact\n");
+            }
+        }
     }
 
     ModelWeights weights = checkpoint.empty()
@@ -169,19 +203,34 @@ int main(int argc, char **argv) {
     GenerationBatch batch;
     if (!session.generate(req, &batch, &err)) fail(err);
 
+    // generate.rs:609-728
     const double prefill_tps = batch.prefill_elapsed > 0 ? (double)session.prompt_len() / batch.prefill_elapsed : 0.0;
-    const size_t decode_steps = req.steps ? req.steps - 1 : 0;                                       // generate.rs:612
+    const size_t decode_steps = req.steps ? req.steps - 1 : 0;
+    const double avg_decode_tps = decode_steps > 0 && batch.avg_decode_elapsed > 0 ? (double)decode_steps / batch.avg_decode_elapsed : 0.0;
     const double total_tps = batch.total_elapsed > 0 ? (double)(req.steps * req.samples) / batch.total_elapsed : 0.0;
+    auto sample_tps = [&](const SampleResult &r) {
+        return decode_steps > 0 && r.decode_elapsed > 0 ? (double)decode_steps / r.decode_elapsed : 0.0;
+    };
     printf("prompt_ids=%s\n", format_ids(prompt).c_str());
-    for (size_t i = 0; i < batch.results.size(); ++i) {
-        const SampleResult &r = batch.results[i];
-        if (req.samples > 1) printf("sample=%zu seed=%llu\n", i, (unsigned long long)r.seed);
+    if (req.samples == 1) {
+        const SampleResult &r = batch.results[0];
         printf("generated_ids=%s\n", format_ids(r.sampled).c_str());
         printf("full_sequence=%s\n", format_ids(r.generated).c_str());
-        printf("decode_steps=%zu decode_time=%.2fms decode_tok/s=%.2f\n", decode_steps, r.decode_elapsed * 1e3,
-               decode_steps && r.decode_elapsed > 0 ? (double)decode_steps / r.decode_elapsed : 0.0);
+        printf("prefill_time=%.2fms prefill_tok/s=%.2f\n", batch.prefill_elapsed * 1e3, prefill_tps);
+        printf("decode_steps=%zu decode_time=%.2fms decode_tok/s=%.2f\n", decode_steps, r.decode_elapsed * 1e3, sample_tps(r));
+    } else {
+        for (size_t i = 0; i < batch.results.size(); ++i) {
+            const SampleResult &r = batch.results[i];
+            printf("sample%zu_seed=%llu\n", i, (unsigned long long)r.seed);
+            printf("sample%zu_generated_ids=%s\n", i, format_ids(r.sampled).c_str());
+            printf("sample%zu_full_sequence=%s\n", i, format_ids(r.generated).c_str());
+            printf("sample%zu_decode_steps=%zu sample%zu_decode_time=%.2fms sample%zu_decode_tok/s=%.2f\n", i, decode_steps, i,
+                   r.decode_elapsed * 1e3, i, sample_tps(r));
+        }
+        printf("prefill_time=%.2fms prefill_tok/s=%.2f\n", batch.prefill_elapsed * 1e3, prefill_tps);
+        printf("samples_decode_time_total=%.2fms samples_decode_time_avg=%.2fms avg_decode_tok/s=%.2f\n",
+               batch.total_decode_elapsed * 1e3, batch.avg_decode_elapsed * 1e3, avg_decode_tps);
     }
-    printf("prefill_time=%.2fms prefill_tok/s=%.2f\n", batch.prefill_elapsed * 1e3, prefill_tps);
     printf("total_generation_time=%.2fms overall_tok/s=%.2f\n", batch.total_elapsed * 1e3, total_tps);
     return 0;
 }

@@ -96,3 +96,93 @@ def test_binary_session_answers_equal_direct_session_calls(tmp_path):
     assert list(out[0]["results"][0]) == ["seed", "generated_ids", "full_sequence", "generated_text", "full_text",
                                           "decode_time_ms", "decode_tok_per_s"]
     assert out[1]["request_prefill_ms"] > 0 and out[0]["request_prefill_ms"] == 0
+
+
+def _report(stdout):
+    """The one-shot report as a list of lines and a dict of its space-separated key=value fields."""
+    lines = stdout.splitlines()
+    fields = {}
+    for ln in lines:
+        for part in ln.split(" "):
+            if "=" in part:
+                k, v = part.split("=", 1)
+                fields[k] = v
+    return lines, fields
+
+
+@pytest.mark.gpu
+def test_one_shot_report_lines_follow_the_reference(tmp_path):
+    """`generate` without --jsonl-session prints the reference's report (generate.rs:524-566 before the run,
+    :609-728 after it): same keys, same order, ids equal to a direct session's."""
+    cfg = Config.make(dim=256, hidden=640, heads=2, hd=128, seq=96, nlayers=2, vocab=320)
+    w = synth.make_weights(cfg, seed=8, std=0.08, round_bf16=True)
+    path = tmp_path / "ckpt_000007.bin"
+    engine.write_checkpoint(path, cfg, w, step=7)
+    base = [1, 2, 3, 4, 5, 6, 7, 8, 9]
+    ids = ",".join(map(str, base))
+    common = [GENERATE, "--checkpoint", str(path), "--prompt-ids", ids, "--weight-dtype", "bf16", "--kv-dtype", "f32"]
+    sess = engine.InferenceSession(cfg, w, base, weight_dtype=1, kv_dtype=0)
+    hip = engine.DecodeBackendRequest.HIP
+
+    # one greedy sample
+    proc = subprocess.run(common + ["--steps", "6", "--decode-backend", "hip"], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stderr
+    lines, f = _report(proc.stdout)
+    want = sess.generate(engine.GenerationRequest(hip, steps=6)).results[0]
+    assert lines[0] == "loaded checkpoint: step=7 model=2L 256D 640H 320V seq=96"
+    assert lines[1] == ("prompt_len=9 effective_context_len=9 steps=6 temperature=0 top_k=0 decode_backend_request=hip "
+                        "decode_mode=kv_cache_hip greedy_sampling=true")
+    assert lines[2] == "samples=1 prefix_reuse=disabled"
+    assert lines[3] == "prompt_ids=" + ids
+    assert lines[4] == "generated_ids=" + ",".join(str(int(t)) for t in want.sampled)
+    assert lines[5] == "full_sequence=" + ",".join(str(int(t)) for t in want.generated)
+    assert [ln.split("=")[0] for ln in lines[6:]] == ["prefill_time", "decode_steps", "total_generation_time"]
+    assert f["decode_steps"] == "5" and f["prefill_time"].endswith("ms") and f["decode_time"].endswith("ms")
+    assert float(f["prefill_tok/s"]) > 0 and float(f["decode_tok/s"]) > 0 and float(f["overall_tok/s"]) > 0
+    assert len(lines) == 9
+
+    # two sampled continuations, candidates from the device: per-sample lines and the averages
+    proc = subprocess.run(common + ["--steps", "5", "--temperature", "0.8", "--top-k", "4", "--samples", "2", "--seed", "5",
+                                    "--decode-backend", "hip"], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stderr
+    lines, f = _report(proc.stdout)
+    want = sess.generate(engine.GenerationRequest(hip, steps=5, temperature=0.8, top_k=4, samples=2, seed=5)).results
+    assert lines[1] == ("prompt_len=9 effective_context_len=9 steps=5 temperature=0.8 top_k=4 decode_backend_request=hip "
+                        "decode_mode=kv_cache_hip greedy_sampling=false")
+    assert lines[2] == "samples=2 prefix_reuse=enabled"
+    assert lines[3] == "cached_sampling_path=gpu_topk_candidates top_k=4 gpu_topk_capacity=32"
+    assert lines[4] == "prompt_ids=" + ids
+    at = 5
+    for i, r in enumerate(want):
+        assert lines[at] == "sample%d_seed=%d" % (i, r.seed)
+        assert lines[at + 1] == "sample%d_generated_ids=%s" % (i, ",".join(str(int(t)) for t in r.sampled))
+        assert lines[at + 2] == "sample%d_full_sequence=%s" % (i, ",".join(str(int(t)) for t in r.generated))
+        assert lines[at + 3].startswith("sample%d_decode_steps=4 sample%d_decode_time=" % (i, i))
+        assert " sample%d_decode_tok/s=" % i in lines[at + 3]
+        at += 4
+    assert [ln.split("=")[0] for ln in lines[at:]] == ["prefill_time", "samples_decode_time_total", "total_generation_time"]
+    assert "samples_decode_time_avg" in f and "avg_decode_tok/s" in f
+    assert len(lines) == at + 3
+
+    # the planner's notes: auto on a small model, a window that overflows, block statistics, a wide top-k
+    proc = subprocess.run(common + ["--steps", "2"], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stderr
+    lines, f = _report(proc.stdout)
+    assert f["decode_backend_request"] == "auto" and f["decode_mode"] == "naive_full_context"
+    assert lines[2] == "decode_backend_auto_reason=model_param_count_lt_threshold model_params=%d auto_metal_threshold=20000000" % (
+        cfg.param_count())
+    proc = subprocess.run(common[:4] + [",".join(str(1 + i % 300) for i in range(100)), "--weight-dtype", "bf16", "--steps", "3",
+                                        "--decode-backend", "hip"], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stderr
+    lines, f = _report(proc.stdout)
+    assert f["prompt_len"] == "100" and f["effective_context_len"] == "96"
+    assert lines[2] == "prompt_truncated=true kept_last_tokens=96"
+    assert lines[3] == "decode_backend_fallback=true reason=requested_length_exceeds_cfg_seq"
+    for extra, note in ((["--temperature", "1.5"], "cached_sampling_path=gpu_block_stats_exact"),
+                        (["--temperature", "0.7", "--top-k", "40"],
+                         "cached_sampling_path=full_logits_cpu_sample reason=top_k_exceeds_gpu_capacity requested_top_k=40 "
+                         "gpu_topk_capacity=32")):
+        proc = subprocess.run(common + ["--steps", "3", "--decode-backend", "hip"] + extra, capture_output=True, text=True,
+                              timeout=120)
+        assert proc.returncode == 0, proc.stderr
+        assert note in proc.stdout.splitlines()
