@@ -64,7 +64,18 @@ bool infer_hidden(size_t dim, size_t nlayers, size_t vocab, size_t payload_float
 
 }  // namespace
 
-bool parse_checkpoint(const uint8_t *bytes, size_t len, Checkpoint *out, std::string *err) {
+bool parse_checkpoint_shape(const std::string &text, CheckpointShape *out, std::string *err) {
+    unsigned long long h = 0, k = 0, e = 0, f = 0;
+    char tail = 0;
+    const int n = sscanf(text.c_str(), " heads=%llu kv_heads=%llu hd=%llu hidden=%llu %c", &h, &k, &e, &f, &tail);
+    if (n != 4) return bad(err, "checkpoint shape file must read: heads=H kv_heads=K hd=E hidden=F");
+    if (!h || !k || !e || !f || h % k != 0 || e % 2 != 0)
+        return bad(err, "checkpoint shape file describes no valid model (heads a multiple of kv_heads, even hd, no zeros)");
+    out->heads = h; out->kv_heads = k; out->hd = e; out->hidden = f;
+    return true;
+}
+
+bool parse_checkpoint(const uint8_t *bytes, size_t len, Checkpoint *out, std::string *err, const CheckpointShape *shape) {
     if (len < kHeaderV1) return bad(err, "checkpoint too small for header");
     if (memcmp(bytes, "RSTK", 4) != 0) return bad(err, "invalid checkpoint magic");
     size_t cur = 4;
@@ -83,13 +94,21 @@ bool parse_checkpoint(const uint8_t *bytes, size_t len, Checkpoint *out, std::st
         act = (FfnActivation)code;
     }
     if (dim == 0 || nlayers == 0 || vocab == 0 || seq == 0) return bad(err, "checkpoint config contains zero dimension");
-    if (dim % 128 != 0) return bad(err, "checkpoint dim " + std::to_string(dim) + " is not divisible by 128");
+    if (!shape && dim % 128 != 0) return bad(err, "checkpoint dim " + std::to_string(dim) + " is not divisible by 128");
     if ((len - cur) % 4 != 0) return bad(err, "checkpoint payload is not aligned to f32 values");
     const size_t payload_floats = (len - cur) / 4;
-    const size_t heads = dim / 128;
-    size_t hidden = 0;
-    if (!infer_hidden(dim, nlayers, vocab, payload_floats, &hidden, err)) return false;
-    out->cfg = ModelConfig::make(dim, hidden, heads, heads, 128, seq, nlayers, vocab, act);
+    if (shape) {
+        out->cfg = ModelConfig::make(dim, shape->hidden, shape->heads, shape->kv_heads, shape->hd, seq, nlayers, vocab, act);
+        const ModelConfig &sc = out->cfg;
+        const size_t per_layer = sc.dim * sc.q_dim + 2 * sc.dim * sc.kv_dim + sc.q_dim * sc.dim + 3 * sc.dim * sc.hidden + 2 * sc.dim;
+        if (payload_floats != sc.vocab * sc.dim + sc.dim + sc.nlayers * per_layer)
+            return bad(err, "checkpoint payload does not match the shape file beside it");
+    } else {
+        const size_t heads = dim / 128;
+        size_t hidden = 0;
+        if (!infer_hidden(dim, nlayers, vocab, payload_floats, &hidden, err)) return false;
+        out->cfg = ModelConfig::make(dim, hidden, heads, heads, 128, seq, nlayers, vocab, act);
+    }
     out->step = step;
     const ModelConfig &c = out->cfg;
     ModelWeights &w = out->weights;
@@ -113,6 +132,15 @@ bool parse_checkpoint(const uint8_t *bytes, size_t len, Checkpoint *out, std::st
 }
 
 bool load_checkpoint(const std::string &path, Checkpoint *out, std::string *err) {
+    CheckpointShape shape;
+    bool have_shape = false;
+    if (FILE *sf = fopen((path + ".shape").c_str(), "r")) {
+        char line[256] = {0};
+        const size_t got = fread(line, 1, sizeof line - 1, sf);
+        fclose(sf);
+        if (!parse_checkpoint_shape(std::string(line, got), &shape, err)) return false;
+        have_shape = true;
+    }
     const int fd = open(path.c_str(), O_RDONLY);
     if (fd < 0) return bad(err, "cannot open " + path + ": " + strerror(errno));
     struct stat st;
@@ -122,16 +150,24 @@ bool load_checkpoint(const std::string &path, Checkpoint *out, std::string *err)
     void *p = mmap(nullptr, len, PROT_READ, MAP_PRIVATE, fd, 0);
     close(fd);
     if (p == MAP_FAILED) return bad(err, "cannot map " + path + ": " + strerror(errno));
-    const bool ok = parse_checkpoint((const uint8_t *)p, len, out, err);
+    const bool ok = parse_checkpoint((const uint8_t *)p, len, out, err, have_shape ? &shape : nullptr);
     munmap(p, len);
     return ok;
 }
 
 bool write_checkpoint(const std::string &path, const ModelConfig &c, const ModelWeights &w, uint32_t step,
                       std::string *err) {
-    if (c.hd != 128 || c.kv_heads != c.heads || c.dim != c.heads * 128)
-        return bad(err, "the checkpoint header cannot describe this model (needs hd 128, kv_heads = heads, dim = heads * 128)");
+    const bool needs_shape = c.hd != 128 || c.kv_heads != c.heads || c.dim != c.heads * 128;
     if (w.layers.size() != c.nlayers) return bad(err, "layer count does not match the configuration");
+    const std::string shape_path = path + ".shape";
+    if (needs_shape) {
+        FILE *sf = fopen(shape_path.c_str(), "w");
+        if (!sf) return bad(err, "cannot create " + shape_path + ": " + strerror(errno));
+        const bool sok = fprintf(sf, "heads=%zu kv_heads=%zu hd=%zu hidden=%zu\n", c.heads, c.kv_heads, c.hd, c.hidden) > 0;
+        if (fclose(sf) != 0 || !sok) return bad(err, "short write writing " + shape_path);
+    } else {
+        (void)remove(shape_path.c_str());                   // a stale side file would override the header's shape
+    }
     FILE *f = fopen(path.c_str(), "wb");
     if (!f) return bad(err, "cannot create " + path + ": " + strerror(errno));
     const uint32_t head[7] = {kVersion, step, (uint32_t)c.dim, (uint32_t)c.nlayers, (uint32_t)c.vocab, (uint32_t)c.seq,

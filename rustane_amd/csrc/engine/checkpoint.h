@@ -5,6 +5,12 @@
 //   wq wk wv wo w1 w3 w2 gamma1 gamma2.
 // The header carries neither heads nor hidden: heads = dim / 128 (hd = 128, MHA) and hidden follows
 // from the payload size (checkpoint.rs:101-117, :168-214).
+//
+// Models the header cannot describe (another head size, grouped KV heads) keep the same file and
+// get a side file PATH.shape beside it, one line of text:
+//   heads=H kv_heads=K hd=E hidden=F
+// The reader takes the shape from the side file when there is one and checks the payload size
+// against it; the reference has no such file and reads (or rejects) the main file as before.
 #pragma once
 #include <string>
 
@@ -18,12 +24,20 @@ struct Checkpoint {
     uint32_t step = 0;
 };
 
+struct CheckpointShape {
+    size_t heads = 0, kv_heads = 0, hd = 0, hidden = 0;
+};
+// the side file's line; false and a message on anything else
+bool parse_checkpoint_shape(const std::string &text, CheckpointShape *out, std::string *err);
+
 // checkpoint.rs:30-166.  Returns false and the reference's message in *err on malformed input.
-bool parse_checkpoint(const uint8_t *bytes, size_t len, Checkpoint *out, std::string *err);
+// shape: the side file's content, or null for a file the header describes.
+bool parse_checkpoint(const uint8_t *bytes, size_t len, Checkpoint *out, std::string *err,
+                      const CheckpointShape *shape = nullptr);
 // checkpoint.rs:25-28 (the file is mapped, not read into a second buffer)
 bool load_checkpoint(const std::string &path, Checkpoint *out, std::string *err);
-// train.rs:609-647: version-2 header and tensor order; the model must be one the header can
-// describe (hd = 128, kv_heads = heads, dim = heads * 128)
+// train.rs:609-647: version-2 header and tensor order; a model the header cannot describe
+// (hd != 128, kv_heads != heads or dim != heads * 128) also gets the side file
 bool write_checkpoint(const std::string &path, const ModelConfig &cfg, const ModelWeights &w, uint32_t step,
                       std::string *err);
 

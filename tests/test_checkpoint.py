@@ -93,10 +93,39 @@ def test_writer_emits_the_documented_layout_and_round_trips(tmp_path):
     assert_same_weights(got_w, w)
     with pytest.raises(engine.CheckpointError):
         engine.load_checkpoint(tmp_path / "missing.bin")
-    # the header has no place for hd or kv_heads: such models are refused, not written wrongly
-    gqa = Config.make(dim=256, hidden=384, heads=4, hd=64, seq=64, nlayers=1, vocab=32, kv_heads=2)
-    with pytest.raises(engine.CheckpointError):
-        engine.write_checkpoint(tmp_path / "x.bin", gqa, synth.make_weights(gqa, seed=1, std=0.05))
+
+
+def test_models_the_header_cannot_describe_round_trip_through_the_shape_file(tmp_path):
+    """The header has no place for hd, kv_heads or hidden (checkpoint.rs:83-112 assumes hd 128, MHA and
+    infers hidden): such a model keeps the reference's file layout and gets PATH.shape beside it."""
+    gqa = Config.make(dim=192, hidden=320, heads=3, hd=64, seq=64, nlayers=2, vocab=48, kv_heads=1)   # the tiny workload's kind
+    w = synth.make_weights(gqa, seed=1, std=0.05)
+    path = tmp_path / "tiny.bin"
+    engine.write_checkpoint(path, gqa, w, step=9, ffn_activation=1)
+    assert (tmp_path / "tiny.bin.shape").read_text() == "heads=3 kv_heads=1 hd=64 hidden=320\n"
+    assert path.read_bytes() == file_bytes(gqa, w, step=9, act=1)            # the main file is the documented layout
+    cfg2, w2, step, act = engine.load_checkpoint(path)
+    assert (step, act) == (9, 1)
+    assert (cfg2.dim, cfg2.hidden, cfg2.heads, cfg2.kv_heads, cfg2.hd, cfg2.q_dim, cfg2.kv_dim) == (192, 320, 3, 1, 64, 192, 64)
+    assert_same_weights(w2, w)
+    # without the side file the main file is read as the reference reads it: rejected here (dim % 128)
+    with pytest.raises(engine.CheckpointError, match="checkpoint dim 192 is not divisible by 128"):
+        engine.parse_checkpoint(path.read_bytes())
+    # a side file that does not fit the payload, or does not parse
+    (tmp_path / "tiny.bin.shape").write_text("heads=3 kv_heads=1 hd=64 hidden=352\n")
+    with pytest.raises(engine.CheckpointError, match="does not match the shape file"):
+        engine.load_checkpoint(path)
+    (tmp_path / "tiny.bin.shape").write_text("heads=3 kv_heads=2 hd=64 hidden=320\n")
+    with pytest.raises(engine.CheckpointError, match="no valid model"):
+        engine.load_checkpoint(path)
+    (tmp_path / "tiny.bin.shape").write_text("heads=3 hd=64\n")
+    with pytest.raises(engine.CheckpointError, match="must read: heads=H kv_heads=K hd=E hidden=F"):
+        engine.load_checkpoint(path)
+    # a model the header describes leaves no side file behind, and removes a stale one
+    cfg = cfg_small()
+    engine.write_checkpoint(path, cfg, synth.make_weights(cfg, seed=6, std=0.05), step=1)
+    assert not (tmp_path / "tiny.bin.shape").exists()
+    assert engine.load_checkpoint(path)[0].hd == 128
 
 
 @pytest.mark.gpu
