@@ -454,14 +454,23 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     // the compiler wait for "everything outstanding" at the top of every iteration, which later
     // includes the weights requested for the phase.
     __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0)
+    // A model whose phases are a single round for every wave (the widest share of a kind: ceil(pairs / G)
+    // pairs) is bound by the exchanges, not by the stream: there, a request is only put in front of a
+    // poll when the multiply behind that poll needs it (loads return in order, so the polled vector
+    // is seen after everything requested before it).  A model with several rounds per phase keeps the
+    // earliest possible requests.
+    auto own_rounds = [&](int rows, int kind) { return (((rows / 2 + G - 1) / G + MEGA_WAVES - 1) / MEGA_WAVES) * kinds[kind].segs; };
+    auto dealt_rounds = [&](int rows, int kind) { return (((rows / 2 + G - 1) / G) * kinds[kind].segs + MEGA_WAVES - 1) / MEGA_WAVES; };
+    const bool qkv_one_round = own_rounds(Q + 2 * KV, MK_QKV) <= MEGA_DEPTH;
+    const bool b0_late = qkv_one_round && own_rounds(2 * H, MK_W13) <= MEGA_DEPTH && dealt_rounds(D, MK_WO) <= MEGA_DEPTH_B &&
+                         dealt_rounds(D, MK_W2) <= MEGA_DEPTH_B;
     start_even(0);
     issue_even();
     o_left = 0;
-    if (1 <= last_ph) { start_odd(1); issue_odd_one(ctxB, stB[0]); }
+    if (1 <= last_ph) { start_odd(1); if (!b0_late) issue_odd_one(ctxB, stB[0]); }
 
     const int wo_row0 = 2 * kinds[MK_WO].pair0, wo_rows = 2 * kinds[MK_WO].npl;   // same partition for w2
-    // the qkv phase is one round for every wave of every workgroup (the widest share: ceil(pairs / G) pairs)
-    const bool qkv_one_round = (((Q + 2 * KV) / 2 + G - 1) / G + MEGA_WAVES - 1) / MEGA_WAVES * kinds[MK_QKV].segs <= MEGA_DEPTH;
+
     const int n_att = pos + 1;
     int NS = (n_att + SLOTS * MEGA_ATT_SPLIT_PASSES - 1) / (SLOTS * MEGA_ATT_SPLIT_PASSES);
     NS = max(1, min(NS, a.ns_max));
@@ -522,7 +531,9 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         // Requests are spread over the phases, one task (four loads per lane) at a time, so that each one
         // finds room in the memory pipeline: requested in one block, a round holds the wave at the
         // address unit for a good part of the time the block takes to stream.  Here: the second task of
-        // the odd phase behind this one (its first went out at the end of the odd phase before).
+        // the odd phase behind this one (its first went out at the end of the odd phase before, or goes
+        // out here: b0_late).
+        if (b0_late) issue_odd_one(ctxB, stB[0]);
 #pragma unroll
         for (int s = 1; s < MEGA_DEPTH_B; ++s) issue_odd_one(ctxB, stB[s]);
         float inv;
@@ -937,7 +948,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
 #pragma unroll
         for (int s = 3; s < MEGA_DEPTH; ++s) issue_even_one(ctxA, stA[s]);
         o_left = 0;
-        if (oph + 2 <= last_ph) { start_odd(oph + 2); issue_odd_one(ctxB, stB[0]); }
+        if (oph + 2 <= last_ph) { start_odd(oph + 2); if (!b0_late) issue_odd_one(ctxB, stB[0]); }
         mark();
         mark();
         }
