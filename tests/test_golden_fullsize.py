@@ -47,7 +47,9 @@ def test_oracle_reproduces_the_fullsize_vector():
     orc = O.Oracle(cfg, w, kv_round_bf16=(g["kv_cache"] == "bf16"))
     lg, _, _ = orc.forward_window(ids)
     check_logits(g, lg[0], 1e-5)
-    assert len(g["greedy_stream"]) == 256 and g["greedy_min_top2_gap"] > 50 * 1e-4 * g["logit_abs_max"]
+    # the closest call of the 256 greedy steps is decided by more than twice the logits tolerance of the
+    # GPU tests (1e-4 of the largest logit): a device within tolerance reproduces the whole stream
+    assert len(g["greedy_stream"]) == 256 and g["greedy_min_top2_gap"] > 2 * 1e-4 * g["logit_abs_max"]
     sampled, _ = orc.run_cached_sample(ids, lg[0], 40)          # a prefix here; the GPU suite checks all 256 steps
     assert [int(t) for t in sampled] == g["greedy_stream"][:40]
     for st in g["sampled_streams"]:

@@ -177,8 +177,8 @@ def test_5b_quantised_prefill_paths_and_chained_run_agree(w5b, wdt):
 def test_5b_bf16_workload_prefill_paths_and_fullvocab_sampled_run(w5b):
     """The 5B bf16 workload at its own shape: 1024-token prompt, bf16 cache, then full-vocabulary
     sampling at temperature 1.0 through the block-statistics path.  (i) The chunked matrix-core
-    prefill against one token step per prompt row (the persistent kernel, which moves to its
-    many-partials build on the way: 32 heads x 3 splits from position 256).  (ii) 24 steps of
+    prefill against one token step per prompt row (the persistent kernel, whose fold covers
+    32 heads x up to 8 splits on the way).  (ii) 24 steps of
     hipdec_decode_fullvocab_sampled_run against the reference's loop built from the per-step calls
     and the oracle's two draws (inference.rs:600-625), tokens and RNG state."""
     cfg, w = w5b

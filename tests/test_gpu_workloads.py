@@ -1,5 +1,5 @@
-"""GPU checks of the decode path at the shapes and kernel builds the benchmark workloads run, through the
-C ABI: the persistent step kernel's build for many attention partials against the oracle, odd layer
+"""GPU checks of the decode path at the shapes the benchmark workloads run, through the C ABI: the
+persistent step kernel with many attention partials per fold (several splits of many heads) against the oracle, odd layer
 counts (the exchange stamps alternate with the layer index, so their parity at a launch depends on the
 layer count and on how many launches came before), bit-for-bit repeatability whatever that parity,
 and the multi-sample workload at its own shape (512-token prompt, bf16 cache, 8 samples of 256 steps)
@@ -35,18 +35,18 @@ def splits_at(cfg, kv_bf16, pos):
                                                    (WeightDtype.BF16, KvDtype.BF16, 400, 5e-3),
                                                    (WeightDtype.FP8_E4M3, KvDtype.BF16, 400, 8e-3),
                                                    (WeightDtype.INT4_G128, KvDtype.BF16, 400, 8e-3)])
-def test_wide_partials_build_against_the_oracle(wdt, kvdt, n_prompt, tol):
-    """With heads x splits x (hd + 4) / 4 above 2048 the host launches the kernel build that polls the
-    attention partials with more slots in flight and folds them four outputs at a time.  16 heads of
-    128 reach that at 4 splits: 193 positions with an fp32 cache, 385 with a bf16 cache (bf16, e4m3 and
-    4-bit weight streams, the quantised ones against the oracle on the de-quantised weights).  Logits and
-    greedy ids of the steps after the prompt against the oracle, for the chunked prefill and for the
-    token-step prefill (which crosses the switch between the two builds on its way), and against the
+def test_many_attention_partials_against_the_oracle(wdt, kvdt, n_prompt, tol):
+    """Every workgroup of the persistent kernel folds all heads x splits attention partials while it polls
+    them.  16 heads of 128 at 4 splits (193 positions with an fp32 cache, 385 with a bf16 cache) are 64
+    records of 132 floats per fold: more than 2048 16-byte slots, four dependent groups per thread (bf16,
+    e4m3 and 4-bit weight streams, the quantised ones against the oracle on the de-quantised weights).
+    Logits and greedy ids of the steps after the prompt against the oracle, for the chunked prefill and
+    for the token-step prefill (whose split count grows on the way), and against the
     one-kernel-per-product path."""
     cfg = Config.make(dim=2048, hidden=2048, heads=16, hd=128, seq=512, nlayers=2, vocab=2048)
     kv_bf16 = kvdt == KvDtype.BF16
-    assert cfg.heads * splits_at(cfg, kv_bf16, n_prompt) * (cfg.hd + 4) // 4 > 2048       # the wide build runs
-    assert cfg.heads * splits_at(cfg, kv_bf16, 100) * (cfg.hd + 4) // 4 <= 2048           # and the plain one before it
+    assert cfg.heads * splits_at(cfg, kv_bf16, n_prompt) * (cfg.hd + 4) // 4 > 2048       # four splits of 16 heads
+    assert splits_at(cfg, kv_bf16, 100) < splits_at(cfg, kv_bf16, n_prompt)               # fewer on the way there
     w = synth.make_weights(cfg, seed=5, std=0.05, round_bf16=True)
     ids = synth.make_prompt(11, cfg.vocab, n_prompt)
     # 8-bit / 4-bit weights: the oracle multiplies with the de-quantised matrices
@@ -69,7 +69,7 @@ def test_wide_partials_build_against_the_oracle(wdt, kvdt, n_prompt, tol):
             assert rel_err(got, want) < tol, (name, step)
             assert int(np.argmax(got)) == int(O.argmax_lower(want)), (name, step)
         tok = int(O.argmax_lower(want))
-    # a device-chained greedy run of the wide build against single calls of the per-product path
+    # a device-chained greedy run at that split count against single calls of the per-product path
     a, c = devs["chunked"], devs["per product"]
     a.set_len(n_prompt)
     c.set_len(n_prompt)
