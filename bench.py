@@ -220,6 +220,19 @@ def measure(args, workload, with_cpu_baseline):
     prefill_wall_ms = (time.perf_counter() - t0) * 1e3
     prefill_dev_ms = dev.last_device_ms()
     first = int(np.argmax(logits))
+    # the same prompt with the prefill GEMMs on single-bf16 activations (an option, not the default: the
+    # headline prefill figure keeps the fp32-grade activation pair); the cache is rebuilt with the pair afterwards
+    prefill_bf16_act = None
+    if wdt != WeightDtype.F32 and n_prompt >= 8:
+        dev.set_prefill_bf16_act(True)
+        dev.set_len(0)
+        lg1 = dev.prefill(prompt)
+        prefill_bf16_act = {"prefill_ms": dev.last_device_ms(),
+                            "max_logit_diff_rel": float(np.abs(lg1 - logits).max() / np.abs(logits).max()),
+                            "same_first_token": bool(int(np.argmax(lg1)) == first)}
+        dev.set_prefill_bf16_act(False)
+        dev.set_len(0)
+        dev.prefill(prompt)
     # algorithmic prefill flops: 2*T*(linear params) + causal attention + the LM head on the last row
     lin = cfg.nlayers * (cfg.dim * (cfg.q_dim + 2 * cfg.kv_dim) + cfg.q_dim * cfg.dim + 3 * cfg.dim * cfg.hidden)
     T = n_prompt
@@ -229,8 +242,10 @@ def measure(args, workload, with_cpu_baseline):
     room = cfg.seq - n_prompt
     K, W = args.steps, args.warmup
     if workload == "c4_5b_bf16_bs1":
-        return run_c4_sampled(args, workload, cfg, dev, kvdt, logits, n_prompt, gen_steps, prefill_dev_ms, prefill_wall_ms,
-                              prefill_flops, mfma_peak)
+        out = run_c4_sampled(args, workload, cfg, dev, kvdt, logits, n_prompt, gen_steps, prefill_dev_ms, prefill_wall_ms,
+                             prefill_flops, mfma_peak)
+        out["prefill_bf16_act"] = prefill_bf16_act
+        return out
     if W > 0:
         dev.decode_greedy_run(first, min(W, room))
     # timed region: exactly K greedy steps, in runs that restart at the end of the prompt so every
@@ -280,6 +295,8 @@ def measure(args, workload, with_cpu_baseline):
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(workload),
                      "traffic_source": TRAFFIC_SOURCE, "bytes_per_step": bytes_per_step},
     }
+    if prefill_bf16_act:
+        out["prefill_bf16_act"] = prefill_bf16_act
     if with_cpu_baseline:
         replay = workload in ("c1_tiny_fp32", "c2_600m_bf16_bs1")      # the oracle can afford the prompt here
         out["cpu_baseline"] = cpu_baseline(cfg, weights, kvdt == KvDtype.BF16, prompt if replay else None,
@@ -296,6 +313,8 @@ def summary(r):
          "bytes_per_step": r["roofline"]["bytes_per_step"]}
     if "prefill_roofline" in r:
         e["prefill_mfma_frac"] = r["prefill_roofline"]["frac"]
+    if r.get("prefill_bf16_act"):
+        e["prefill_bf16_act"] = r["prefill_bf16_act"]
     if "mfma_roofline" in r:
         e["step_mfma_frac"] = r["mfma_roofline"]["frac"]
     return e

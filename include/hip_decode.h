@@ -76,6 +76,10 @@ typedef struct {
 #define HIPDEC_FLAG_NO_MEGA 2u    /* one kernel per matrix product instead of the persistent per-token kernel */
 #define HIPDEC_FLAG_PREFILL_STEPS 4u /* hipdec_prefill runs one token step per prompt row instead of the
                                         chunked matrix-core path (which bf16 and e4m3 weights use by default) */
+#define HIPDEC_FLAG_PREFILL_BF16_ACT 8u /* the chunked prefill's GEMMs multiply the weights by the activations rounded
+                                        to one bf16 number instead of the (hi, lo) pair that keeps 16 mantissa bits:
+                                        half the matrix-core work, prompt logits within ~1e-2 of the token path
+                                        (meant for 8-bit / 4-bit weights, whose own rounding is coarser) */
 
 typedef struct hipdec_model hipdec_model;
 
@@ -91,6 +95,11 @@ const char *hipdec_last_error(const hipdec_model *m);
 /* Model::len / Model::set_len, lib.rs:209-215 (set_len clamps to cfg.seq). */
 size_t hipdec_len(const hipdec_model *m);
 int hipdec_set_len(hipdec_model *m, size_t len);
+
+/* Switches how hipdec_prefill multiplies from now on: on != 0 sets HIPDEC_FLAG_PREFILL_BF16_ACT, 0 clears
+ * it.  (No counterpart in the reference, whose prefill precision is fixed by the ANE's fp16; the other
+ * flags are fixed at hipdec_create.) */
+int hipdec_set_prefill_bf16_act(hipdec_model *m, int on);
 
 /* Model::seed_layer_cache_from_channel_first, lib.rs:217-237:
  * cache[pos*kv_dim + d] = k_rope_cf[d*seq + pos] for pos < live_len, the rest zero. */

@@ -571,9 +571,13 @@ int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, c
     }
     const int bn = PF_BN_OF(wt);
     dim3 grid((N + bn - 1) / bn, (T + PF_BM - 1) / PF_BM, sp.splits), block(256);
-    if (wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm<WT_BF16>, grid, block, 0, m->stream, g);
-    else if (wt == WT_FP8) hipLaunchKernelGGL(k_pf_gemm<WT_FP8>, grid, block, 0, m->stream, g);
-    else hipLaunchKernelGGL(k_pf_gemm<WT_INT4>, grid, block, 0, m->stream, g);
+    const bool lo = !(m->opt.flags & HIPDEC_FLAG_PREFILL_BF16_ACT);
+#define PFG(WTX) do { if (lo) hipLaunchKernelGGL((k_pf_gemm<WTX, true>), grid, block, 0, m->stream, g); \
+                      else hipLaunchKernelGGL((k_pf_gemm<WTX, false>), grid, block, 0, m->stream, g); } while (0)
+    if (wt == WT_BF16) PFG(WT_BF16);
+    else if (wt == WT_FP8) PFG(WT_FP8);
+    else PFG(WT_INT4);
+#undef PFG
     return sp.splits;
 }
 
@@ -1255,6 +1259,7 @@ int hipdec_create(const hipdec_config *cfg, const hipdec_layer_f32 *layers, size
     // graph replays still see every kernel)
     if (const char *e = getenv("HIPDEC_NO_GRAPH")) if (e[0] == '1') o.flags |= HIPDEC_FLAG_NO_GRAPH;
     if (const char *e = getenv("HIPDEC_PREFILL_STEPS")) if (e[0] == '1') o.flags |= HIPDEC_FLAG_PREFILL_STEPS;
+    if (const char *e = getenv("HIPDEC_PREFILL_BF16_ACT")) if (e[0] == '1') o.flags |= HIPDEC_FLAG_PREFILL_BF16_ACT;
     m->opt = o;
     m->wt = (int)o.weight_dtype;
     m->embed_wt = o.weight_dtype == HIPDEC_W_F32 ? WT_F32 : WT_BF16;
@@ -1275,6 +1280,13 @@ size_t hipdec_len(const hipdec_model *m) { return m ? m->len : 0; }
 int hipdec_set_len(hipdec_model *m, size_t len) {
     if (!m) return HIPDEC_ERR_ARG;
     m->len = len < m->cfg.seq ? len : m->cfg.seq;
+    return HIPDEC_OK;
+}
+
+int hipdec_set_prefill_bf16_act(hipdec_model *m, int on) {
+    if (!m) return HIPDEC_ERR_ARG;
+    if (on) m->opt.flags |= HIPDEC_FLAG_PREFILL_BF16_ACT;
+    else m->opt.flags &= ~HIPDEC_FLAG_PREFILL_BF16_ACT;
     return HIPDEC_OK;
 }
 

@@ -211,7 +211,8 @@ __device__ __forceinline__ pf_bf16x8 pf_frag(const uint16_t *p) {
 // 2 x (PF_BN / 64) MFMA tiles.  Operand layout of v_mfma_f32_32x32x16_bf16: lane l supplies row
 // (l % 32), reduction elements 8 * (l / 32) .. + 7 of both operands; result register i of lane l is
 // C[8 * (i / 4) + 4 * (l / 32) + i % 4][l % 32].
-template <int WT>
+// LO: multiply by the lo parts of the activations too (false: the hi parts only, half the matrix work)
+template <int WT, bool LO = true>
 __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g) {
     constexpr int PF_BN = PF_BN_OF(WT);
     __shared__ __align__(16) uint16_t sAh[PF_BM * PF_LDS_STRIDE];
@@ -260,7 +261,7 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
             s.ah[j] = zero4; s.al[j] = zero4;
             if (k < g.K) {
                 s.ah[j] = *(const uint4 *)(g.Ahi + ta * g.K + k);
-                s.al[j] = *(const uint4 *)(g.Alo + ta * g.K + k);
+                if (LO) s.al[j] = *(const uint4 *)(g.Alo + ta * g.K + k);
             }
         }
 #pragma unroll
@@ -295,7 +296,7 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
         for (int j = 0; j < 4; ++j) {
             const int c = tid + 256 * j, row = c >> 3, kc = c & 7;
             *(uint4 *)(sAh + row * PF_LDS_STRIDE + kc * 8) = s.ah[j];
-            *(uint4 *)(sAl + row * PF_LDS_STRIDE + kc * 8) = s.al[j];
+            if (LO) *(uint4 *)(sAl + row * PF_LDS_STRIDE + kc * 8) = s.al[j];
         }
         if (WT == WT_BF16) {
 #pragma unroll
@@ -353,7 +354,7 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt) {
                 ah[mt] = pf_frag(sAh + (64 * wm + 32 * mt + r) * PF_LDS_STRIDE + 16 * j + kq);
-                al[mt] = pf_frag(sAl + (64 * wm + 32 * mt + r) * PF_LDS_STRIDE + 16 * j + kq);
+                if (LO) al[mt] = pf_frag(sAl + (64 * wm + 32 * mt + r) * PF_LDS_STRIDE + 16 * j + kq);
             }
             // two workgroups per CU: one weight fragment at a time keeps the kernel within 128 registers
             // (the other workgroup covers the LDS latency); alone on the CU, all fragments are requested first
@@ -373,10 +374,10 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
                     if (WT == WT_INT4) {
                         pf_f32x16 &t = accg[mt % (WT == WT_INT4 ? 2 : 1)][nt % (WT == WT_INT4 ? NT : 1)];
                         t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mt], bf, t, 0, 0, 0);
-                        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], bf, t, 0, 0, 0);
+                        if (LO) t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], bf, t, 0, 0, 0);
                     } else {
                         acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mt], bf, acc[mt][nt], 0, 0, 0);
-                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], bf, acc[mt][nt], 0, 0, 0);
+                        if (LO) acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], bf, acc[mt][nt], 0, 0, 0);
                     }
                 }
             }
