@@ -220,17 +220,23 @@ def measure(args, workload, with_cpu_baseline):
     prefill_wall_ms = (time.perf_counter() - t0) * 1e3
     prefill_dev_ms = dev.last_device_ms()
     first = int(np.argmax(logits))
-    # the same prompt with the prefill GEMMs on single-bf16 activations (an option, not the default: the
-    # headline prefill figure keeps the fp32-grade activation pair); the cache is rebuilt with the pair afterwards
-    prefill_bf16_act = None
-    if wdt != WeightDtype.F32 and n_prompt >= 8:
-        dev.set_prefill_bf16_act(True)
-        dev.set_len(0)
-        lg1 = dev.prefill(prompt)
-        prefill_bf16_act = {"prefill_ms": dev.last_device_ms(),
-                            "max_logit_diff_rel": float(np.abs(lg1 - logits).max() / np.abs(logits).max()),
-                            "same_first_token": bool(int(np.argmax(lg1)) == first)}
-        dev.set_prefill_bf16_act(False)
+    # The same prompt under the other activation formats of the prefill GEMMs (the headline figure is the
+    # model's default: one fp16 number per activation for 8-bit / 4-bit weights with a bf16 cache, the (hi, lo)
+    # bf16 pair otherwise); differences are against the default's prompt logits.  The cache is rebuilt with the default afterwards.
+    prefill_options = None
+    if wdt != WeightDtype.F32 and n_prompt > 32:
+        default_mode = 2 if (kvdt == KvDtype.BF16 and wdt in (WeightDtype.FP8_E4M3, WeightDtype.INT4_G128)) else 0
+        prefill_options = {"default": ("bf16_pair", "bf16", "f16")[default_mode] + "_activations"}
+        for name, mode in (("bf16_pair_activations", 0), ("bf16_activations", 1), ("f16_activations", 2)):
+            if mode == default_mode:
+                continue
+            dev.set_prefill_activations(mode)
+            dev.set_len(0)
+            lg1 = dev.prefill(prompt)
+            prefill_options[name] = {"prefill_ms": dev.last_device_ms(),
+                                     "max_logit_diff_rel": float(np.abs(lg1 - logits).max() / np.abs(logits).max()),
+                                     "same_first_token": bool(int(np.argmax(lg1)) == first)}
+        dev.set_prefill_activations(default_mode)
         dev.set_len(0)
         dev.prefill(prompt)
     # algorithmic prefill flops: 2*T*(linear params) + causal attention + the LM head on the last row
@@ -244,7 +250,7 @@ def measure(args, workload, with_cpu_baseline):
     if workload == "c4_5b_bf16_bs1":
         out = run_c4_sampled(args, workload, cfg, dev, kvdt, logits, n_prompt, gen_steps, prefill_dev_ms, prefill_wall_ms,
                              prefill_flops, mfma_peak)
-        out["prefill_bf16_act"] = prefill_bf16_act
+        out["prefill_options"] = prefill_options
         return out
     if W > 0:
         dev.decode_greedy_run(first, min(W, room))
@@ -295,8 +301,8 @@ def measure(args, workload, with_cpu_baseline):
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(workload),
                      "traffic_source": TRAFFIC_SOURCE, "bytes_per_step": bytes_per_step},
     }
-    if prefill_bf16_act:
-        out["prefill_bf16_act"] = prefill_bf16_act
+    if prefill_options:
+        out["prefill_options"] = prefill_options
     if with_cpu_baseline:
         replay = workload in ("c1_tiny_fp32", "c2_600m_bf16_bs1")      # the oracle can afford the prompt here
         out["cpu_baseline"] = cpu_baseline(cfg, weights, kvdt == KvDtype.BF16, prompt if replay else None,
@@ -313,8 +319,8 @@ def summary(r):
          "bytes_per_step": r["roofline"]["bytes_per_step"]}
     if "prefill_roofline" in r:
         e["prefill_mfma_frac"] = r["prefill_roofline"]["frac"]
-    if r.get("prefill_bf16_act"):
-        e["prefill_bf16_act"] = r["prefill_bf16_act"]
+    if r.get("prefill_options"):
+        e["prefill_options"] = r["prefill_options"]
     if "mfma_roofline" in r:
         e["step_mfma_frac"] = r["mfma_roofline"]["frac"]
     return e

@@ -80,6 +80,12 @@ typedef struct {
                                         to one bf16 number instead of the (hi, lo) pair that keeps 16 mantissa bits:
                                         half the matrix-core work, prompt logits within ~1e-2 of the token path
                                         (meant for 8-bit / 4-bit weights, whose own rounding is coarser) */
+#define HIPDEC_FLAG_PREFILL_F16_ACT 16u /* the same with the activations rounded to one fp16 number (11 mantissa bits,
+                                        saturating at +-65504; the weights are widened to fp16 exactly): half the
+                                        matrix-core work, the precision of the reference's own fp16 prefill;
+                                        the default of 8-bit / 4-bit models with a bf16 cache */
+#define HIPDEC_FLAG_PREFILL_PAIR_ACT 32u /* the (hi, lo) bf16 pair, 16 mantissa bits (the default of every other
+                                        model), also for those */
 
 typedef struct hipdec_model hipdec_model;
 
@@ -96,10 +102,11 @@ const char *hipdec_last_error(const hipdec_model *m);
 size_t hipdec_len(const hipdec_model *m);
 int hipdec_set_len(hipdec_model *m, size_t len);
 
-/* Switches how hipdec_prefill multiplies from now on: on != 0 sets HIPDEC_FLAG_PREFILL_BF16_ACT, 0 clears
- * it.  (No counterpart in the reference, whose prefill precision is fixed by the ANE's fp16; the other
- * flags are fixed at hipdec_create.) */
-int hipdec_set_prefill_bf16_act(hipdec_model *m, int on);
+/* How hipdec_prefill carries activations into its GEMMs from now on: 0 the (hi, lo) bf16 pair
+ * (HIPDEC_FLAG_PREFILL_PAIR_ACT), 1 one bf16 number (_BF16_ACT), 2 one fp16 number (_F16_ACT).
+ * (No counterpart in the reference, whose prefill precision is fixed by the ANE's fp16; the other flags
+ * are fixed at hipdec_create.) */
+int hipdec_set_prefill_activations(hipdec_model *m, int mode);
 
 /* Model::seed_layer_cache_from_channel_first, lib.rs:217-237:
  * cache[pos*kv_dim + d] = k_rope_cf[d*seq + pos] for pos < live_len, the rest zero. */

@@ -77,6 +77,7 @@ struct hipdec_model {
     hipdec_config cfg{};
     hipdec_options opt{};
     int wt = WT_F32, embed_wt = WT_F32, kvbf16 = 0;
+    int pf_act = PF_ACT_PAIR;            // how the chunked prefill carries activations into its GEMMs (PF_ACT_*)
     int num_cu = 256;
     hipStream_t stream = nullptr;
     std::vector<DevLayer> layers;
@@ -558,8 +559,9 @@ int pf_ensure(hipdec_model *m, int T, bool with_head = false) {
 }
 
 // P[z][t][n] = sum over the z-th K slice of A[t][k] * W[n][k]; returns the number of planes
+// act: PF_ACT_* of the activation arrays (the few-row kernel only takes pairs)
 int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, const void *W, const void *scales,
-            int T, int N, int K) {
+            int T, int N, int K, int act = PF_ACT_PAIR) {
     const PfSplit sp = pf_split_k(m, wt, T, N, K);
     PfGemm g{Ahi, Alo, W, wt == WT_INT4 ? (const uint16_t *)scales : nullptr, m->pf.P, T, N, K, sp.steps_per_split};
     if (T <= kSkinnyRows && wt != WT_INT4) {
@@ -571,9 +573,9 @@ int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, c
     }
     const int bn = PF_BN_OF(wt);
     dim3 grid((N + bn - 1) / bn, (T + PF_BM - 1) / PF_BM, sp.splits), block(256);
-    const bool lo = !(m->opt.flags & HIPDEC_FLAG_PREFILL_BF16_ACT);
-#define PFG(WTX) do { if (lo) hipLaunchKernelGGL((k_pf_gemm<WTX, true>), grid, block, 0, m->stream, g); \
-                      else hipLaunchKernelGGL((k_pf_gemm<WTX, false>), grid, block, 0, m->stream, g); } while (0)
+#define PFG(WTX) do { if (act == PF_ACT_F16) hipLaunchKernelGGL((k_pf_gemm<WTX, PF_ACT_F16>), grid, block, 0, m->stream, g); \
+                      else if (act == PF_ACT_BF16) hipLaunchKernelGGL((k_pf_gemm<WTX, PF_ACT_BF16>), grid, block, 0, m->stream, g); \
+                      else hipLaunchKernelGGL((k_pf_gemm<WTX, PF_ACT_PAIR>), grid, block, 0, m->stream, g); } while (0)
     if (wt == WT_BF16) PFG(WT_BF16);
     else if (wt == WT_FP8) PFG(WT_FP8);
     else PFG(WT_INT4);
@@ -582,33 +584,33 @@ int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, c
 }
 
 // launches shared by the prompt prefill and the multi-sample step
-void pf_launch_embed(hipdec_model *m, int T) {
+void pf_launch_embed(hipdec_model *m, int T, int f16 = 0) {
     PrefillWork &w = m->pf;
     const int D = (int)m->cfg.dim;
     dim3 grid((D + PF_CHUNK - 1) / PF_CHUNK, T), block(PF_CHUNK);
     if (m->embed_wt == WT_F32)
         hipLaunchKernelGGL(k_pf_embed<WT_F32>, grid, block, 0, m->stream, m->embed, w.ids, w.x, m->layers[0].g1, w.xn_hi,
-                           w.xn_lo, w.ssq, D);
+                           w.xn_lo, w.ssq, D, f16);
     else
         hipLaunchKernelGGL(k_pf_embed<WT_BF16>, grid, block, 0, m->stream, m->embed, w.ids, w.x, m->layers[0].g1, w.xn_hi,
-                           w.xn_lo, w.ssq, D);
+                           w.xn_lo, w.ssq, D, f16);
 }
 void pf_launch_resid(hipdec_model *m, int T, int splits, const void *wscale, const float *resid, float *out,
-                     const float *gamma) {
+                     const float *gamma, int f16 = 0) {
     PrefillWork &w = m->pf;
     const int D = (int)m->cfg.dim;
     dim3 grid((D + PF_CHUNK - 1) / PF_CHUNK, T), block(PF_CHUNK);
     hipLaunchKernelGGL(k_pf_resid, grid, block, 0, m->stream, w.P, splits, (size_t)T * D,
                        m->wt == WT_FP8 ? (const float *)wscale : nullptr, resid, m->alpha, out, gamma, w.xn_hi, w.xn_lo,
-                       w.ssq, D);
+                       w.ssq, D, f16);
 }
-void pf_launch_gate(hipdec_model *m, int T, int splits, const void *wscale) {
+void pf_launch_gate(hipdec_model *m, int T, int splits, const void *wscale, int f16 = 0) {
     PrefillWork &w = m->pf;
     const int D = (int)m->cfg.dim, H = (int)m->cfg.hidden;
     const size_t items = (size_t)T * (H / 4);
     hipLaunchKernelGGL(k_pf_gate_epi, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, m->stream, w.P, splits,
                        (size_t)T * 2 * H, m->wt == WT_FP8 ? (const float *)wscale : nullptr, w.gate_hi, w.gate_lo, w.ssq,
-                       (D + PF_CHUNK - 1) / PF_CHUNK, D, T, H, (int)m->opt.ffn_activation);
+                       (D + PF_CHUNK - 1) / PF_CHUNK, D, T, H, (int)m->opt.ffn_activation, f16);
 }
 
 // Runs prompt rows ids[0..n) at positions len .. len+n-1 through every layer, chunk by chunk; on
@@ -629,14 +631,18 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
         HCHK(hipStreamSynchronize(m->stream));                  // the pinned id buffer is free again
         memcpy(w.h_ids, ids + done, (size_t)T * 4);
         HCHK(hipMemcpyAsync(w.ids, w.h_ids, (size_t)T * 4, hipMemcpyHostToDevice, m->stream));
-        pf_launch_embed(m, T);
+        // how this chunk's activations travel between its kernels (the few-row GEMM only takes pairs)
+        const bool tiled = !(T <= kSkinnyRows && m->wt != WT_INT4);
+        const int act = !tiled ? PF_ACT_PAIR : m->pf_act;
+        const int f16 = act == PF_ACT_F16;
+        pf_launch_embed(m, T, f16);
         const int nch = (D + PF_CHUNK - 1) / PF_CHUNK;
         for (uint32_t l = 0; l < c.nlayers; ++l) {
             const DevLayer &L = m->layers[l];
             const bool fp8 = m->wt == WT_FP8;
             // q/k/v projections, RoPE, cache append
             int N = Q + 2 * KV;
-            int sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.wqkv, L.s_qkv, T, N, D);
+            int sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.wqkv, L.s_qkv, T, N, D, act);
             {
                 const size_t items = (size_t)T * (N / 4);
                 dim3 grid((unsigned)((items + 255) / 256)), block(256);
@@ -654,20 +660,20 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
                 dim3 grid((T + 31) / 32, c.heads), block(64 * PF_ATT_WAVES);
 #define PFATT(KVB, HD)                                                                                             \
     hipLaunchKernelGGL((k_pf_attn<KVB, HD>), grid, block, 0, m->stream, w.q, L.kc, L.vc, w.att_hi, w.att_lo, T, Q, KV, \
-                       gqa, pos0, (int)c.seq, scale)
+                       gqa, pos0, (int)c.seq, scale, f16)
                 if (m->kvbf16) { if (c.hd == 64) PFATT(1, 64); else PFATT(1, 128); }
                 else { if (c.hd == 64) PFATT(0, 64); else PFATT(0, 128); }
 #undef PFATT
             }
             // output projection, residual, second norm
-            sp = pf_gemm(m, m->wt, w.att_hi, w.att_lo, L.wo, L.s_wo, T, D, Q);
-            pf_launch_resid(m, T, sp, L.s_wo, w.x, w.x2, L.g2);
+            sp = pf_gemm(m, m->wt, w.att_hi, w.att_lo, L.wo, L.s_wo, T, D, Q, act);
+            pf_launch_resid(m, T, sp, L.s_wo, w.x, w.x2, L.g2, f16);
             // gate/up, activation
-            sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.w13, L.s_w13, T, 2 * H, D);
-            pf_launch_gate(m, T, sp, L.s_w13);
+            sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.w13, L.s_w13, T, 2 * H, D, act);
+            pf_launch_gate(m, T, sp, L.s_w13, f16);
             // down projection, residual, next layer's first norm
-            sp = pf_gemm(m, m->wt, w.gate_hi, w.gate_lo, L.w2, L.s_w2, T, D, H);
-            pf_launch_resid(m, T, sp, L.s_w2, w.x2, w.x, l + 1 < c.nlayers ? m->layers[l + 1].g1 : nullptr);
+            sp = pf_gemm(m, m->wt, w.gate_hi, w.gate_lo, L.w2, L.s_w2, T, D, H, act);
+            pf_launch_resid(m, T, sp, L.s_w2, w.x2, w.x, l + 1 < c.nlayers ? m->layers[l + 1].g1 : nullptr, f16);
         }
         HCHK(hipGetLastError());
         *x_last = w.x + (size_t)(T - 1) * D;
@@ -1260,10 +1266,24 @@ int hipdec_create(const hipdec_config *cfg, const hipdec_layer_f32 *layers, size
     if (const char *e = getenv("HIPDEC_NO_GRAPH")) if (e[0] == '1') o.flags |= HIPDEC_FLAG_NO_GRAPH;
     if (const char *e = getenv("HIPDEC_PREFILL_STEPS")) if (e[0] == '1') o.flags |= HIPDEC_FLAG_PREFILL_STEPS;
     if (const char *e = getenv("HIPDEC_PREFILL_BF16_ACT")) if (e[0] == '1') o.flags |= HIPDEC_FLAG_PREFILL_BF16_ACT;
+    if (const char *e = getenv("HIPDEC_PREFILL_F16_ACT")) if (e[0] == '1') o.flags |= HIPDEC_FLAG_PREFILL_F16_ACT;
+    if (const char *e = getenv("HIPDEC_PREFILL_PAIR_ACT")) if (e[0] == '1') o.flags |= HIPDEC_FLAG_PREFILL_PAIR_ACT;
     m->opt = o;
     m->wt = (int)o.weight_dtype;
     m->embed_wt = o.weight_dtype == HIPDEC_W_F32 ? WT_F32 : WT_BF16;
     m->kvbf16 = o.kv_dtype == HIPDEC_KV_BF16;
+    // Prefill activations: with 8-bit or 4-bit weights and a bf16 cache the GEMMs take one fp16 number per
+    // activation (half the matrix work of the pair; the weights' own rounding, 2^-4 and coarser, is far above
+    // fp16's 2^-11, and such a model is judged at 5e-2 of the largest logit: measured 3e-3 from the pair at
+    // 5B).  bf16 weights keep the pair whatever the cache: with fp16 activations the 600M greedy stream
+    // left the CPU reference's at its 90th token (a near tie moved by differently rounded cache rows).
+    // The flags override either way.
+    const bool quantised = o.weight_dtype == HIPDEC_W_FP8_E4M3 || o.weight_dtype == HIPDEC_W_INT4_G128;
+    m->pf_act = (o.flags & HIPDEC_FLAG_PREFILL_PAIR_ACT)   ? PF_ACT_PAIR
+                : (o.flags & HIPDEC_FLAG_PREFILL_BF16_ACT) ? PF_ACT_BF16
+                : (o.flags & HIPDEC_FLAG_PREFILL_F16_ACT)  ? PF_ACT_F16
+                : (m->kvbf16 && quantised)                 ? PF_ACT_F16
+                                                           : PF_ACT_PAIR;
     m->alpha = 1.0f / sqrtf(2.0f * (float)c.nlayers);   // lib.rs:201
     int rc = create_impl(m, layers, head);
     if (rc != HIPDEC_OK) {
@@ -1283,10 +1303,10 @@ int hipdec_set_len(hipdec_model *m, size_t len) {
     return HIPDEC_OK;
 }
 
-int hipdec_set_prefill_bf16_act(hipdec_model *m, int on) {
+int hipdec_set_prefill_activations(hipdec_model *m, int mode) {
     if (!m) return HIPDEC_ERR_ARG;
-    if (on) m->opt.flags |= HIPDEC_FLAG_PREFILL_BF16_ACT;
-    else m->opt.flags &= ~HIPDEC_FLAG_PREFILL_BF16_ACT;
+    if (mode < 0 || mode > 2) return fail(m, HIPDEC_ERR_ARG, "prefill activation mode must be 0 (bf16 pair), 1 (bf16) or 2 (fp16)");
+    m->pf_act = mode;
     return HIPDEC_OK;
 }
 

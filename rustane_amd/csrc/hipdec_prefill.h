@@ -33,7 +33,14 @@ typedef float pf_f32x16 __attribute__((ext_vector_type(16)));
 #define PF_LDS_STRIDE 72    // bf16 elements per LDS tile row (144 bytes: 16-byte aligned; 16 consecutive rows
                             // start 36 banks apart, so a 128-bit operand read by 16 lanes touches every bank once)
 
-__device__ __forceinline__ void pf_split(float v, uint16_t &hi, uint16_t &lo) {
+// f16 != 0: the activation as ONE fp16 number in hi (11 mantissa bits, saturating at the fp16 range; lo unused)
+__device__ __forceinline__ void pf_split(float v, uint16_t &hi, uint16_t &lo, int f16 = 0) {
+    if (f16) {
+        const _Float16 h = (_Float16)fminf(fmaxf(v, -65504.0f), 65504.0f);
+        hi = __builtin_bit_cast(uint16_t, h);
+        lo = 0;
+        return;
+    }
     hi = f32_to_bf16_rne(v);
     lo = f32_to_bf16_rne(v - bf16_to_f32(hi));
 }
@@ -66,7 +73,7 @@ template <int EWT>
 __global__ __launch_bounds__(PF_CHUNK) void k_pf_embed(const void *__restrict__ embed, const uint32_t *__restrict__ ids,
                                                        float *__restrict__ x, const float *__restrict__ gamma,
                                                        uint16_t *__restrict__ hi, uint16_t *__restrict__ lo,
-                                                       float *__restrict__ ssq, int D) {
+                                                       float *__restrict__ ssq, int D, int f16) {
     __shared__ float red[8];
     const int t = blockIdx.y, d = blockIdx.x * PF_CHUNK + threadIdx.x;
     float v = 0.0f;
@@ -74,7 +81,7 @@ __global__ __launch_bounds__(PF_CHUNK) void k_pf_embed(const void *__restrict__ 
         const size_t tok = ids[t];
         v = EWT == WT_F32 ? ((const float *)embed)[tok * D + d] : bf16_to_f32(((const uint16_t *)embed)[tok * D + d]);
         x[(size_t)t * D + d] = v;
-        pf_split(v * gamma[d], hi[(size_t)t * D + d], lo[(size_t)t * D + d]);
+        pf_split(v * gamma[d], hi[(size_t)t * D + d], lo[(size_t)t * D + d], f16);
     }
     const float ss = pf_block_sum(v * v, red);
     if (threadIdx.x == 0) ssq[t * gridDim.x + blockIdx.x] = ss;
@@ -86,7 +93,7 @@ __global__ __launch_bounds__(PF_CHUNK) void k_pf_resid(const float *__restrict__
                                                        const float *__restrict__ wscale, const float *__restrict__ resid,
                                                        float alpha, float *__restrict__ out, const float *__restrict__ gamma,
                                                        uint16_t *__restrict__ hi, uint16_t *__restrict__ lo,
-                                                       float *__restrict__ ssq, int D) {
+                                                       float *__restrict__ ssq, int D, int f16) {
     __shared__ float red[8];
     const int t = blockIdx.y, d = blockIdx.x * PF_CHUNK + threadIdx.x;
     float v = 0.0f;
@@ -96,7 +103,7 @@ __global__ __launch_bounds__(PF_CHUNK) void k_pf_resid(const float *__restrict__
         if (wscale) s *= wscale[d];
         v = resid[(size_t)t * D + d] + alpha * s;
         out[(size_t)t * D + d] = v;
-        if (gamma) pf_split(v * gamma[d], hi[(size_t)t * D + d], lo[(size_t)t * D + d]);
+        if (gamma) pf_split(v * gamma[d], hi[(size_t)t * D + d], lo[(size_t)t * D + d], f16);
     }
     const float ss = pf_block_sum(v * v, red);
     if (threadIdx.x == 0) ssq[t * gridDim.x + blockIdx.x] = ss;
@@ -162,7 +169,7 @@ __global__ __launch_bounds__(256) void k_pf_qkv_epi(const float *__restrict__ P,
 __global__ __launch_bounds__(256) void k_pf_gate_epi(const float *__restrict__ P, int splits, size_t plane,
                                                      const float *__restrict__ wscale, uint16_t *__restrict__ hi,
                                                      uint16_t *__restrict__ lo, const float *__restrict__ ssq, int nch,
-                                                     int D, int T, int H, int act) {
+                                                     int D, int T, int H, int act, int f16) {
     const int hq = H >> 2;
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= (size_t)T * hq) return;
@@ -185,7 +192,7 @@ __global__ __launch_bounds__(256) void k_pf_gate_epi(const float *__restrict__ P
         float g;
         if (act == 1) { const float lr = h1 > 0.0f ? h1 : 0.5f * h1; g = lr * lr * h3; }
         else { const float sig = 1.0f / (1.0f + expf(-h1)); g = h1 * sig * h3; }
-        pf_split(g, oh[e], ol[e]);
+        pf_split(g, oh[e], ol[e], f16);
     }
     const size_t o = (size_t)t * H + j;
     *(uint2 *)(hi + o) = make_uint2((uint32_t)oh[0] | ((uint32_t)oh[1] << 16), (uint32_t)oh[2] | ((uint32_t)oh[3] << 16));
@@ -211,9 +218,30 @@ __device__ __forceinline__ pf_bf16x8 pf_frag(const uint16_t *p) {
 // 2 x (PF_BN / 64) MFMA tiles.  Operand layout of v_mfma_f32_32x32x16_bf16: lane l supplies row
 // (l % 32), reduction elements 8 * (l / 32) .. + 7 of both operands; result register i of lane l is
 // C[8 * (i / 4) + 4 * (l / 32) + i % 4][l % 32].
-// LO: multiply by the lo parts of the activations too (false: the hi parts only, half the matrix work)
-template <int WT, bool LO = true>
+// ACT: how the activations arrive.  PF_ACT_PAIR: two bf16 numbers (hi, lo), each weight tile multiplies both;
+// PF_ACT_BF16: the hi parts only (8 mantissa bits, half the matrix work); PF_ACT_F16: one fp16 number in
+// hi (11 mantissa bits, half the matrix work): the weight tile is widened to fp16 on its way into LDS
+// (exact for bf16, e4m3 and 4-bit values down to 2^-24) and the product runs on the fp16 matrix instruction.
+enum { PF_ACT_PAIR = 0, PF_ACT_BF16 = 1, PF_ACT_F16 = 2 };
+typedef _Float16 pf_f16x8 __attribute__((ext_vector_type(8)));
+typedef __fp16 pf_h2 __attribute__((ext_vector_type(2)));
+// two fp32 values that are exactly representable -> packed fp16 (the rounding mode never applies)
+__device__ __forceinline__ uint32_t pf_pack_f16(float a, float b) {
+    const pf_h2 h = __builtin_amdgcn_cvt_pkrtz(a, b);
+    return __builtin_bit_cast(uint32_t, h);
+}
+// a 32-bit word holding two bf16 numbers -> the same two numbers as fp16
+__device__ __forceinline__ uint32_t pf_bf16x2_to_f16x2(uint32_t w) {
+    return pf_pack_f16(__uint_as_float(w << 16), __uint_as_float(w & 0xffff0000u));
+}
+__device__ __forceinline__ pf_f32x16 pf_mma(const uint4 &a, const uint4 &b, pf_f32x16 c, bool f16) {
+    if (f16) return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_f16x8, a), __builtin_bit_cast(pf_f16x8, b), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, a), __builtin_bit_cast(pf_bf16x8, b), c, 0, 0, 0);
+}
+template <int WT, int ACT = PF_ACT_PAIR>
 __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g) {
+    constexpr bool LO = ACT == PF_ACT_PAIR;
+    constexpr bool F16 = ACT == PF_ACT_F16;
     constexpr int PF_BN = PF_BN_OF(WT);
     __shared__ __align__(16) uint16_t sAh[PF_BM * PF_LDS_STRIDE];
     __shared__ __align__(16) uint16_t sAl[PF_BM * PF_LDS_STRIDE];
@@ -302,7 +330,9 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
 #pragma unroll
             for (int j = 0; j < WCH; ++j) {
                 const int c = tid + 256 * j, row = c >> 3, kc = c & 7;
-                *(uint4 *)(sW + row * PF_LDS_STRIDE + kc * 8) = s.w[j];
+                uint4 v = s.w[j];
+                if (F16) v = make_uint4(pf_bf16x2_to_f16x2(v.x), pf_bf16x2_to_f16x2(v.y), pf_bf16x2_to_f16x2(v.z), pf_bf16x2_to_f16x2(v.w));
+                *(uint4 *)(sW + row * PF_LDS_STRIDE + kc * 8) = v;
             }
         }
         if (WT == WT_FP8) {
@@ -315,9 +345,14 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
                 for (int i = 0; i < 4; ++i) {
                     auto lo2 = __builtin_amdgcn_cvt_pk_f32_fp8(u[i], false);
                     auto hi2 = __builtin_amdgcn_cvt_pk_f32_fp8(u[i], true);
-                    // e4m3 values are exact in bf16: keep the upper halves of the fp32 patterns
-                    o[2 * i] = (__float_as_uint(lo2[0]) >> 16) | (__float_as_uint(lo2[1]) & 0xffff0000u);
-                    o[2 * i + 1] = (__float_as_uint(hi2[0]) >> 16) | (__float_as_uint(hi2[1]) & 0xffff0000u);
+                    // e4m3 values are exact in bf16 (keep the upper halves of the fp32 patterns) and in fp16
+                    if (F16) {
+                        o[2 * i] = pf_pack_f16(lo2[0], lo2[1]);
+                        o[2 * i + 1] = pf_pack_f16(hi2[0], hi2[1]);
+                    } else {
+                        o[2 * i] = (__float_as_uint(lo2[0]) >> 16) | (__float_as_uint(lo2[1]) & 0xffff0000u);
+                        o[2 * i + 1] = (__float_as_uint(hi2[0]) >> 16) | (__float_as_uint(hi2[1]) & 0xffff0000u);
+                    }
                 }
                 uint16_t *dst = sW + row * PF_LDS_STRIDE + q * 16;
                 *(uint4 *)dst = make_uint4(o[0], o[1], o[2], o[3]);
@@ -339,7 +374,7 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
                     for (int e = 0; e < 4; ++e) {
                         const float f0 = __uint_as_float(0x4B000000u | ((u[i] >> (8 * e)) & 0xfu)) - 8388616.0f;
                         const float f1 = __uint_as_float(0x4B000000u | ((u[i] >> (8 * e + 4)) & 0xfu)) - 8388616.0f;
-                        o[e] = (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xffff0000u);
+                        o[e] = F16 ? pf_pack_f16(f0, f1) : (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xffff0000u);
                     }
                     *(uint4 *)(dst + 8 * i) = make_uint4(o[0], o[1], o[2], o[3]);
                 }
@@ -350,34 +385,34 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
         const int r = lane & 31, kq = 8 * (lane >> 5);
 #pragma unroll
         for (int j = 0; j < PF_BKL / 16; ++j) {
-            pf_bf16x8 ah[2], al[2];
+            uint4 ah[2], al[2];
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt) {
-                ah[mt] = pf_frag(sAh + (64 * wm + 32 * mt + r) * PF_LDS_STRIDE + 16 * j + kq);
-                if (LO) al[mt] = pf_frag(sAl + (64 * wm + 32 * mt + r) * PF_LDS_STRIDE + 16 * j + kq);
+                ah[mt] = *(const uint4 *)(sAh + (64 * wm + 32 * mt + r) * PF_LDS_STRIDE + 16 * j + kq);
+                if (LO) al[mt] = *(const uint4 *)(sAl + (64 * wm + 32 * mt + r) * PF_LDS_STRIDE + 16 * j + kq);
             }
             // two workgroups per CU: one weight fragment at a time keeps the kernel within 128 registers
             // (the other workgroup covers the LDS latency); alone on the CU, all fragments are requested first
             constexpr bool PRELOAD = (WT == WT_INT4);
-            pf_bf16x8 bpre[PRELOAD ? NT : 1];
+            uint4 bpre[PRELOAD ? NT : 1];
             if (PRELOAD) {
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
-                    bpre[PRELOAD ? nt : 0] = pf_frag(sW + (32 * NT * wn + 32 * nt + r) * PF_LDS_STRIDE + 16 * j + kq);
+                    bpre[PRELOAD ? nt : 0] = *(const uint4 *)(sW + (32 * NT * wn + 32 * nt + r) * PF_LDS_STRIDE + 16 * j + kq);
             }
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const pf_bf16x8 bf = PRELOAD ? bpre[PRELOAD ? nt : 0]
-                                             : pf_frag(sW + (32 * NT * wn + 32 * nt + r) * PF_LDS_STRIDE + 16 * j + kq);
+                const uint4 bf = PRELOAD ? bpre[PRELOAD ? nt : 0]
+                                         : *(const uint4 *)(sW + (32 * NT * wn + 32 * nt + r) * PF_LDS_STRIDE + 16 * j + kq);
 #pragma unroll
                 for (int mt = 0; mt < 2; ++mt) {
                     if (WT == WT_INT4) {
                         pf_f32x16 &t = accg[mt % (WT == WT_INT4 ? 2 : 1)][nt % (WT == WT_INT4 ? NT : 1)];
-                        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mt], bf, t, 0, 0, 0);
-                        if (LO) t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], bf, t, 0, 0, 0);
+                        t = pf_mma(ah[mt], bf, t, F16);
+                        if (LO) t = pf_mma(al[mt], bf, t, F16);
                     } else {
-                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mt], bf, acc[mt][nt], 0, 0, 0);
-                        if (LO) acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mt], bf, acc[mt][nt], 0, 0, 0);
+                        acc[mt][nt] = pf_mma(ah[mt], bf, acc[mt][nt], F16);
+                        if (LO) acc[mt][nt] = pf_mma(al[mt], bf, acc[mt][nt], F16);
                     }
                 }
             }
@@ -573,7 +608,7 @@ template <int KVBF16, int HD>
 __global__ __launch_bounds__(64 * PF_ATT_WAVES) void k_pf_attn(const float *__restrict__ q, const void *__restrict__ kc,
                                                 const void *__restrict__ vc, uint16_t *__restrict__ ohi,
                                                 uint16_t *__restrict__ olo, int T, int Q, int KV, int gqa, int pos0,
-                                                int seq, float scale) {
+                                                int seq, float scale, int f16) {
     constexpr int HK = HD / 2;                 // reduction elements per lane group in S
     constexpr int NT = HD / 32;                // 32-wide column tiles of O
     constexpr int VS = HD + 8;                 // LDS row stride of the V tile (floats)
@@ -717,7 +752,7 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void k_pf_attn(const float *__re
         }
         if (t < T) {
             const size_t o = (size_t)t * Q + h * HD + d;
-            pf_split(den > 0.0f ? num / den : 0.0f, ohi[o], olo[o]);
+            pf_split(den > 0.0f ? num / den : 0.0f, ohi[o], olo[o], f16);
         }
     }
 }

@@ -20,7 +20,7 @@ HEAD_BLOCK = 256
 OK, ERR_ARG, ERR_FULL, ERR_HIP, ERR_UNSUPPORTED = 0, 1, 2, 3, 4
 
 EXPORTS = [
-    "hipdec_create", "hipdec_destroy", "hipdec_last_error", "hipdec_len", "hipdec_set_len", "hipdec_set_prefill_bf16_act",
+    "hipdec_create", "hipdec_destroy", "hipdec_last_error", "hipdec_len", "hipdec_set_len", "hipdec_set_prefill_activations",
     "hipdec_seed_layer_cache_from_channel_first", "hipdec_decode_token", "hipdec_decode_token_from_id",
     "hipdec_decode_token_argmax", "hipdec_decode_token_argmax_from_id", "hipdec_decode_token_topk_from_id",
     "hipdec_decode_token_block_stats_from_id", "hipdec_materialize_current_logits_block",
@@ -105,7 +105,7 @@ def load_library(path=None):
     lib.hipdec_create.argtypes = [C.POINTER(Config), C.POINTER(_Layer), C.c_size_t, C.POINTER(_Head),
                                   C.POINTER(_Options), C.POINTER(C.c_void_p)]
     lib.hipdec_set_len.argtypes = [C.c_void_p, C.c_size_t]
-    lib.hipdec_set_prefill_bf16_act.argtypes = [C.c_void_p, C.c_int]
+    lib.hipdec_set_prefill_activations.argtypes = [C.c_void_p, C.c_int]
     lib.hipdec_seed_layer_cache_from_channel_first.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, fp, fp]
     lib.hipdec_decode_token.argtypes = [C.c_void_p, fp, fp]
     lib.hipdec_decode_token_from_id.argtypes = [C.c_void_p, C.c_uint32, fp]
@@ -295,9 +295,9 @@ class HipDecodeModel:
     def set_len(self, n):
         self._chk(self._lib.hipdec_set_len(self._h, n))
 
-    def set_prefill_bf16_act(self, on):
-        """Prefill GEMMs on the activations rounded to one bf16 number (True) or on the (hi, lo) pair (False)."""
-        self._chk(self._lib.hipdec_set_prefill_bf16_act(self._h, 1 if on else 0))
+    def set_prefill_activations(self, mode):
+        """How the prefill GEMMs take their activations: 0 the (hi, lo) bf16 pair, 1 one bf16 number, 2 one fp16 number."""
+        self._chk(self._lib.hipdec_set_prefill_activations(self._h, int(mode)))
 
     def seed_layer_cache_from_channel_first(self, layer_idx, live_len, k_rope_cf, v_cf):
         n = self.cfg.kv_dim * self.cfg.seq

@@ -1,8 +1,9 @@
 """GPU parity of the chunked matrix-core prompt prefill (hipdec_prefill through the C ABI) against
 the CPU oracle's full-window forward (crates/engine/src/full_model.rs:336-437) and against the
-backend's own token-step prefill.  The prefill keeps activations fp32-grade (two bf16 parts), so
-the fp32-cache tolerance is the reference's 1e-4 on logits (crates/engine/tests/auto_kv_decode.rs:67-215);
-with a bf16 cache a 1-ulp difference can flip a cached value's rounding (2e-3)."""
+backend's own token-step prefill.  By default the prefill keeps activations fp32-grade (two bf16
+parts; one fp16 number for 8-bit / 4-bit weights with a bf16 cache), so the fp32-cache tolerance is
+the reference's 1e-4 on logits (crates/engine/tests/auto_kv_decode.rs:67-215); with a bf16 cache a
+1-ulp difference can flip a cached value's rounding (2e-3)."""
 import numpy as np
 import pytest
 
@@ -128,30 +129,44 @@ def test_prefill_longer_than_one_chunk_and_empty_prefill():
     assert rel_err(dev.decode_logits_from_id(tok), orc.decode_logits_from_id(tok)) < 1e-4
 
 
-FLAG_PREFILL_BF16_ACT = 8
+FLAG_PREFILL_BF16_ACT, FLAG_PREFILL_F16_ACT, FLAG_PREFILL_PAIR_ACT = 8, 16, 32
 
 
+@pytest.mark.parametrize("flag,bound", [(FLAG_PREFILL_BF16_ACT, 2e-2), (FLAG_PREFILL_F16_ACT, 3e-3)])
 @pytest.mark.parametrize("wdt,n_prompt", [(WeightDtype.FP8_E4M3, 140), (WeightDtype.INT4_G128, 140), (WeightDtype.BF16, 70)])
-def test_prefill_with_single_bf16_activations(wdt, n_prompt):
-    """HIPDEC_FLAG_PREFILL_BF16_ACT: the prefill GEMMs multiply the weights by the activations rounded to
-    one bf16 number (8 mantissa bits) instead of the (hi, lo) pair, i.e. half the matrix-core work.  The
-    stated bound is 5e-2 of the largest logit against the oracle; what is measured on this 3-layer model
-    is asserted at 2e-2, the token the prompt logits elect is the same as with the pair, and the caches
-    that prefill leaves carry the following cached steps (whose own arithmetic is unchanged) to the same
-    bound."""
+def test_prefill_with_single_number_activations(wdt, n_prompt, flag, bound):
+    """HIPDEC_FLAG_PREFILL_BF16_ACT / _F16_ACT: the prefill GEMMs multiply the weights by the activations
+    rounded to ONE bf16 (8 mantissa bits) or fp16 (11 bits) number instead of the (hi, lo) bf16 pair, i.e.
+    half the matrix-core work.  Stated bounds against the oracle: 5e-2 of the largest logit for bf16, the
+    bf16-cache tolerance of this file for fp16; what is measured on this 3-layer model is asserted (2e-2,
+    3e-3), the token the prompt logits elect is the same as with the pair, the caches that prefill leaves
+    carry the following cached steps (whose own arithmetic is unchanged) to the same bound, and the mode
+    can be switched on a live model.  (fp16 is what an 8-bit / 4-bit model with a bf16 cache uses unless told
+    otherwise; the pair is requested with its own flag here.)"""
     cfg = Config.make(dim=512, hidden=1024, heads=4, hd=128, seq=192, nlayers=3, vocab=512)
     kw = dict(wdt=wdt, kvdt=KvDtype.BF16, std=0.05)
-    w, orc, dev = make(cfg, flags=FLAG_PREFILL_BF16_ACT, **kw)
-    _, _, ref = make(cfg, **kw)
+    w, orc, dev = make(cfg, flags=flag, **kw)
+    _, _, ref = make(cfg, flags=FLAG_PREFILL_PAIR_ACT, **kw)
     ids = synth.make_prompt(3, cfg.vocab, n_prompt)
     lg_o, _, _ = orc.forward_window(ids)
     lg_d, lg_r = dev.prefill(ids), ref.prefill(ids)
     err, err_pair = rel_err(lg_d, lg_o[0]), rel_err(lg_r, lg_o[0])
-    print("single bf16 activations: %.2e of the largest logit against the oracle (pair: %.2e)" % (err, err_pair))
-    assert err_pair < 3e-3 and err_pair < err < 2e-2
+    print("single-number activations (flag %d): %.2e of the largest logit against the oracle (pair: %.2e)" % (flag, err, err_pair))
+    assert err_pair < 3e-3 and err < bound
+    if flag == FLAG_PREFILL_BF16_ACT:
+        assert err > err_pair
     assert int(np.argmax(lg_d)) == int(np.argmax(lg_r)) == int(O.argmax_lower(lg_o[0]))
     tok = int(O.argmax_lower(lg_o[0]))
     for _ in range(4):
         a = orc.decode_logits_from_id(tok)
-        assert rel_err(dev.decode_logits_from_id(tok), a) < 2e-2
+        assert rel_err(dev.decode_logits_from_id(tok), a) < bound
         tok = int(O.argmax_lower(a))
+    # the same switch at run time: the pair model in this mode gives this model's logits bit for bit, and back
+    ref.set_prefill_activations(1 if flag == FLAG_PREFILL_BF16_ACT else 2)
+    ref.set_len(0)
+    np.testing.assert_array_equal(ref.prefill(ids), lg_d)
+    ref.set_prefill_activations(0)
+    ref.set_len(0)
+    np.testing.assert_array_equal(ref.prefill(ids), lg_r)
+    with pytest.raises(Exception):
+        ref.set_prefill_activations(3)
