@@ -501,7 +501,33 @@ bool prefill_batched_ok(const hipdec_model *m, size_t n) {
 struct PfSplit { int splits, steps_per_split; };
 constexpr int kSkinnyRows = 32;          // at most this many rows: the streaming GEMM without LDS weight tiles
 constexpr int kSkinnyLdsBytes = 40 * 1024;   // dynamic LDS for the staged activation slice
-PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K) {
+// the tiled GEMM whose operands go straight into LDS (k_pf_gemm_dl): bf16 weights, enough rows to fill its
+// 128 x 256 tiles, whole 64-element steps, activations as bf16 (pair or single)
+constexpr int kDlMinRows = 129;
+bool pf_use_dl(int wt, int T, int K, int act) {
+    static const bool off = getenv("HIPDEC_NO_DL_GEMM") != nullptr;
+    return !off && wt == WT_BF16 && T >= kDlMinRows && K % PF_BKL == 0 && act != PF_ACT_F16;
+}
+PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K, bool dl = false) {
+    if (dl) {
+        // One workgroup per CU, so the grid runs in rounds of num_cu workgroups and a partly filled last
+        // round costs a whole one.  K splits change the round count: with s splits the work takes
+        // ceil(tiles * s / num_cu) rounds of 1/s the length, plus the extra planes written and summed
+        // (priced at 5 TB/s against ~1.8 us per 64-element step of a tile).
+        const int tiles = ((N + PF_DL_BN - 1) / PF_DL_BN) * ((T + PF_DL_BM - 1) / PF_DL_BM);
+        const int lsteps = K / PF_BKL;
+        const double t_full = 1.8e-6 * lsteps, t_plane = 2.0 * T * N * 4 / 5e12;
+        int best = 1;
+        double best_cost = 1e30;
+        for (int s = 1; s <= 8 && lsteps / s >= 4; ++s) {
+            const int sps = (lsteps + s - 1) / s, ns = (lsteps + sps - 1) / sps;
+            const double rounds = (double)(((size_t)tiles * ns + m->num_cu - 1) / m->num_cu);
+            const double cost = rounds * t_full * sps / lsteps + (ns - 1) * t_plane;
+            if (cost < best_cost * 0.97) { best_cost = cost; best = ns; }
+        }
+        const int sps = (lsteps + best - 1) / best;
+        return PfSplit{(lsteps + sps - 1) / sps, sps};
+    }
     const int nsteps = K / PF_BK;
     if (T <= kSkinnyRows && wt != WT_INT4) {      // (4-bit weights always take the tiled kernel)
         // 4 waves per workgroup share a K range; aim at ~8 waves per CU over the whole grid
@@ -549,7 +575,11 @@ int pf_ensure(hipdec_model *m, int T, bool with_head = false) {
     }
     size_t need = 0;
     const int dims[4][2] = {{(int)(Q + 2 * KV), (int)D}, {(int)D, (int)Q}, {(int)(2 * H), (int)D}, {(int)D, (int)H}};
-    for (auto &d : dims) need = std::max(need, (size_t)pf_split_k(m, m->wt, T, d[0], d[1]).splits * T * d[0]);
+    for (auto &d : dims) {
+        need = std::max(need, (size_t)pf_split_k(m, m->wt, T, d[0], d[1]).splits * T * d[0]);
+        if (pf_use_dl(m->wt, T, d[1], PF_ACT_PAIR))
+            need = std::max(need, (size_t)pf_split_k(m, m->wt, T, d[0], d[1], true).splits * T * d[0]);
+    }
     if (with_head) need = std::max(need, (size_t)pf_split_k(m, m->embed_wt, T, (int)c.vocab, (int)D).splits * T * c.vocab);
     if (need > w.P_floats) {
         if ((rc = dalloc(m, &w.P, need * 4))) return rc;
@@ -562,6 +592,14 @@ int pf_ensure(hipdec_model *m, int T, bool with_head = false) {
 // act: PF_ACT_* of the activation arrays (the few-row kernel only takes pairs)
 int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, const void *W, const void *scales,
             int T, int N, int K, int act = PF_ACT_PAIR) {
+    if (pf_use_dl(wt, T, K, act)) {
+        const PfSplit sp = pf_split_k(m, wt, T, N, K, true);
+        PfGemm g{Ahi, Alo, W, nullptr, m->pf.P, T, N, K, sp.steps_per_split};
+        dim3 grid((N + PF_DL_BN - 1) / PF_DL_BN, (T + PF_DL_BM - 1) / PF_DL_BM, sp.splits), block(64 * PF_DL_WAVES);
+        if (act == PF_ACT_PAIR) hipLaunchKernelGGL((k_pf_gemm_dl<true, PF_BKL, 2, PF_DL_WAVES, 1>), grid, block, 0, m->stream, g);
+        else hipLaunchKernelGGL((k_pf_gemm_dl<false, PF_BKL, 3, PF_DL_WAVES, 1>), grid, block, 0, m->stream, g);
+        return sp.splits;
+    }
     const PfSplit sp = pf_split_k(m, wt, T, N, K);
     PfGemm g{Ahi, Alo, W, wt == WT_INT4 ? (const uint16_t *)scales : nullptr, m->pf.P, T, N, K, sp.steps_per_split};
     if (T <= kSkinnyRows && wt != WT_INT4) {

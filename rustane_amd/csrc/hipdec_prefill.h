@@ -486,6 +486,172 @@ __global__ __launch_bounds__(256, WT == WT_INT4 ? 1 : 2) void k_pf_gemm(PfGemm g
         }
 }
 
+// ---------------------------------------------------------------- tiled GEMM, operands loaded straight into LDS
+// The kernel above moves every operand global -> registers -> LDS, which costs it 48 staging registers
+// (so its tile cannot grow), a round of LDS store instructions per step, and leaves one step of loads
+// in flight.  For bf16 weights no conversion is needed on the way, so this variant lets the memory
+// system write the tiles into LDS itself (`global_load_lds_dwordx4`: every lane names a 16-byte chunk in
+// global memory, the wave's 64 chunks land side by side at an LDS address the wave gives).  No staging
+// registers: the workgroup tile is 128 rows x 256 channels, eight waves of 64 x 64 each (two per SIMD: one
+// multiplies while the other reads operands and computes addresses; four waves of 64 x 128 with one
+// wave per SIMD ran 10 % slower), two (pair) or three (single) LDS stages of 64 / 48 KB, a step's loads
+// issued one or two steps before its multiply and waited for with `s_waitcnt vmcnt(n)`, one workgroup
+// per CU.  Stand-alone, 1024 x 22016 x 4096 / 1024 x 4096 x 11008 / 1024 x 6144 x 4096, pair: 351 / 172 /
+// 119 us against 429 / 219 / 152 us for the kernel above; single bf16: 234 / 113 / 80 us against 278 / 144 / 81.
+// LDS layout: tile rows without padding -- the hardware writes a wave's chunks contiguously -- with the
+// chunks of a row permuted by an XOR of the row index, so that the rows of an operand read spread over
+// all banks; the lane that loads slot s of row R fetches the chunk that belongs there from global.
+#define PF_DL_BM 128
+#define PF_DL_BN 256
+#define PF_DL_WAVES 8      // waves per workgroup the host launches (64 x 64 of the tile each)
+// One load-to-LDS instruction of a wave: lane l's 16 bytes at gptr land at LDS byte address lds_base + 16 l
+// (lds_base wave-uniform, in M0).  Written as assembly on purpose: through the builtin the compiler knows
+// the instruction writes LDS, and across the loop's back edge it can no longer tell the stage being read
+// from the stage being filled, so it waits for ALL of these loads (vmcnt(0)) before the first operand read
+// of every other step -- which serialises the pipeline.  Here every wait for them is stated by hand
+// (pf_vmcnt); the counter is shared with the compiler's own loads, whose waits can only get stricter
+// by loads it does not know of (they complete in order).
+__device__ __forceinline__ void pf_dl_load16(const uint16_t *gptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :: "v"(gptr), "s"(lds_base) : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t pf_lds_addr(const void *p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
+// s_waitcnt vmcnt(n) alone (n < 64): bits 3:0 and 15:14 hold the count, the other counters stay at their maximum
+__device__ __forceinline__ constexpr int pf_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
+// Workgroup barrier for the LDS stages.  A release fence on local memory would also wait for every
+// outstanding load-to-LDS (they are LDS writes), the next stage's included, which is exactly the
+// overlap this kernel is built for; the waits are stated by hand instead (vmcnt(n) by the caller for
+// the stage it is about to read, lgkmcnt(0) here for its own LDS reads), and the "memory" clobber keeps
+// the compiler from moving LDS accesses across the barrier.
+__device__ __forceinline__ void pf_lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+// BK: reduction elements per stage (32 or 64); STAGES: stages in LDS.  Step i's loads are issued
+// STAGES - 1 steps before they are read: after the barrier of step i - (STAGES - 1), i.e. once every wave
+// is done with the stage they overwrite, so a step needs ONE barrier.
+// WAVES: 4 (each wave 64 x 128 of the tile) or 8 (64 x 64: two waves per SIMD cover each other's operand
+// reads and address arithmetic); WGS: workgroups per CU the registers and LDS are budgeted for.
+template <bool LO, int BK, int STAGES, int WAVES, int WGS>
+__global__ __launch_bounds__(64 * WAVES, WGS) void k_pf_gemm_dl(PfGemm g) {
+    constexpr int NTW = 8 / (WAVES / 2);                      // 32-channel tiles per wave
+    constexpr int CPR = BK / 8;                               // 16-byte chunks per tile row
+    constexpr int RPB = 256 / (BK * 2);                       // tile rows per 256 bytes of LDS (64 banks of 4 bytes)
+    constexpr int A_EL = PF_DL_BM * BK, W_EL = PF_DL_BN * BK;
+    constexpr int W_AT = A_EL * (LO ? 2 : 1);                 // element offset of the weight tile inside a stage
+    constexpr int ST_EL = W_AT + W_EL;
+    constexpr int NA = PF_DL_BM * CPR / (64 * WAVES), NW = PF_DL_BN * CPR / (64 * WAVES);   // load instructions per wave: activation tile, weight tile
+    constexpr int LOADS = NA * (LO ? 2 : 1) + NW;             // per wave and stage
+    static_assert(STAGES >= 2 && STAGES <= 6 && LOADS * (STAGES - 1) < 64, "vmcnt holds 6 bits");
+    __shared__ __align__(16) uint16_t sbuf[STAGES * ST_EL];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / (WAVES / 2), wn = wave % (WAVES / 2);
+    const int n0 = blockIdx.x * PF_DL_BN, t0 = blockIdx.y * PF_DL_BM, z = blockIdx.z;
+    const int nsteps = g.K / BK;
+    const int s_begin = z * g.steps_per_split, s_end = min(nsteps, s_begin + g.steps_per_split);
+
+    pf_f32x16 acc[2][NTW];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < NTW; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.0f;
+
+    // Load instruction q of a tile covers the LDS chunk positions 64 q .. 64 q + 63; wave w issues
+    // q = w, w + WAVES, ...  The global element offset of this lane's chunk is fixed over the K loop (rows past
+    // the end re-read the last valid row; their results are not stored).  Chunk c of row R sits at slot
+    // c ^ ((R / RPB) % CPR): a 128-bit operand read is served 16 lanes (16 consecutive tile rows) at a time
+    // out of 64 banks, and with this the 16 chunks fall into 16 different 16-byte bank groups (measured:
+    // swizzled by R % CPR, as 32 banks would want, half of the LDS cycles were bank conflicts).
+    size_t a_off[NA], w_off[NW];
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+        const int P = 64 * (wave + WAVES * i) + lane, row = P / CPR, c = (P % CPR) ^ ((row / RPB) % CPR);
+        a_off[i] = (size_t)min(t0 + row, g.T - 1) * g.K + c * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+        const int P = 64 * (wave + WAVES * i) + lane, row = P / CPR, c = (P % CPR) ^ ((row / RPB) % CPR);
+        w_off[i] = (size_t)min(n0 + row, g.N - 1) * g.K + c * 8;
+    }
+    const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)pf_lds_addr(sbuf)) + (uint32_t)wave * 1024u;   // bytes
+    auto issue = [&](int slot, int step) {
+        const size_t k0 = (size_t)step * BK;
+        const uint32_t base = lds0 + (uint32_t)slot * (2u * ST_EL);
+#pragma unroll
+        for (int i = 0; i < NA; ++i) pf_dl_load16(g.Ahi + a_off[i] + k0, base + 1024u * WAVES * i);
+        if (LO) {
+#pragma unroll
+            for (int i = 0; i < NA; ++i) pf_dl_load16(g.Alo + a_off[i] + k0, base + 2u * A_EL + 1024u * WAVES * i);
+        }
+#pragma unroll
+        for (int i = 0; i < NW; ++i) pf_dl_load16((const uint16_t *)g.W + w_off[i] + k0, base + 2u * W_AT + 1024u * WAVES * i);
+    };
+    const int r = lane & 31, gq = lane >> 5, sw = (r / RPB) % CPR;
+    auto multiply = [&](const uint16_t *sb) {
+#pragma unroll
+        for (int j = 0; j < BK / 16; ++j) {
+            const int slot = ((2 * j + gq) ^ sw) * 8;          // this lane's chunk of the sub-step, swizzled (the tile bases are multiples of 32 rows)
+            uint4 ah[2], al[2];
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+                const int R = 64 * wm + 32 * mt + r;
+                ah[mt] = *(const uint4 *)(sb + R * BK + slot);
+                if (LO) al[mt] = *(const uint4 *)(sb + A_EL + R * BK + slot);
+            }
+#pragma unroll
+            for (int nt = 0; nt < NTW; ++nt) {
+                const int R = 32 * NTW * wn + 32 * nt + r;
+                const uint4 bf = *(const uint4 *)(sb + W_AT + R * BK + slot);
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt) {
+                    acc[mt][nt] = pf_mma(ah[mt], bf, acc[mt][nt], false);
+                    if (LO) acc[mt][nt] = pf_mma(al[mt], bf, acc[mt][nt], false);
+                }
+            }
+        }
+    };
+    // wait until at most `stages` later stages of this wave's loads are outstanding
+    auto wait_stages = [&](int stages) {
+        switch (stages) {
+            case 0: __builtin_amdgcn_s_waitcnt(pf_vmcnt(0)); break;
+            case 1: __builtin_amdgcn_s_waitcnt(pf_vmcnt(LOADS)); break;
+            case 2: __builtin_amdgcn_s_waitcnt(pf_vmcnt(STAGES > 2 ? 2 * LOADS : 0)); break;
+            case 3: __builtin_amdgcn_s_waitcnt(pf_vmcnt(STAGES > 3 ? 3 * LOADS : 0)); break;
+            default: __builtin_amdgcn_s_waitcnt(pf_vmcnt(STAGES > 4 ? 4 * LOADS : 0)); break;
+        }
+    };
+
+    const int n = s_end - s_begin;
+#pragma unroll
+    for (int p = 0; p < STAGES - 1; ++p)
+        if (p < n) issue(p, s_begin + p);
+    int slot = 0;
+    for (int i = 0; i < n; ++i) {
+        wait_stages(min(STAGES - 2, n - 1 - i));   // this wave's part of step i has landed
+        pf_lds_barrier();                          // everyone's has, and everyone is done with step i - 1
+        if (i + STAGES - 1 < n) issue(slot == 0 ? STAGES - 1 : slot - 1, s_begin + i + STAGES - 1);
+        multiply(sbuf + slot * ST_EL);
+        slot = slot + 1 == STAGES ? 0 : slot + 1;
+    }
+
+    float *Pz = g.P + (size_t)z * g.T * g.N;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NTW; ++nt) {
+            const int col = n0 + 32 * NTW * wn + 32 * nt + r;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int t = t0 + 64 * wm + 32 * mt + 8 * (i >> 2) + 4 * gq + (i & 3);
+                if (t < g.T && col < g.N) Pz[(size_t)t * g.N + col] = acc[mt][nt][i];
+            }
+        }
+}
+
 // GEMM for at most 32 activation rows (multi-sample decode, short prompts): weight streaming, not
 // matrix throughput, bounds it, so there is no LDS tile and no barrier in the loop.  A workgroup
 // owns 32 weight rows; its four waves split the workgroup's K range and each lane streams its own
