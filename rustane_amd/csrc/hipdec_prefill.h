@@ -807,6 +807,29 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void k_pf_attn(const float *__re
             qf[s] = v.x * scale; qf[s + 1] = v.y * scale; qf[s + 2] = v.z * scale; qf[s + 3] = v.w * scale;
         }
     }
+    // bf16 cache: both products run on the bf16 matrix instruction (32x32x16), eight times the rate of the
+    // fp32 one.  Keys and values are bf16 numbers already; the scaled query row and the probabilities
+    // enter as (hi, lo) bf16 pairs, like the activations of the GEMMs, so nothing is rounded to 8 bits.
+    // This lane's half of the query row, in operand chunks of 8 elements:
+    uint4 qh[KVBF16 ? KCH : 1], ql[KVBF16 ? KCH : 1];
+    if constexpr (KVBF16 != 0) {
+#pragma unroll
+        for (int c = 0; c < KCH; ++c) {
+            uint32_t wh[4], wl[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                uint16_t h0, l0, h1, l1;
+                pf_split(qf[8 * c + 2 * e], h0, l0);
+                pf_split(qf[8 * c + 2 * e + 1], h1, l1);
+                wh[e] = (uint32_t)h0 | ((uint32_t)h1 << 16);
+                wl[e] = (uint32_t)l0 | ((uint32_t)l1 << 16);
+            }
+            qh[KVBF16 ? c : 0] = make_uint4(wh[0], wh[1], wh[2], wh[3]);
+            ql[KVBF16 ? c : 0] = make_uint4(wl[0], wl[1], wl[2], wl[3]);
+        }
+    }
+    constexpr int VSB = HD + 16;               // bf16 V tile: elements per LDS row (rows 4 apart fall 32 banks apart)
+    uint16_t *sVb = (uint16_t *)sV;            // (the bf16 tile shares the wave's fp32 tile, which the key loop then does not use)
     pf_f32x16 accO[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
@@ -835,23 +858,41 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void k_pf_attn(const float *__re
         pf_f32x16 accS;
 #pragma unroll
         for (int i = 0; i < 16; ++i) accS[i] = 0.0f;
+        if constexpr (KVBF16 != 0) {
+            // chunk c of this lane's half key row is an operand as it is: reduction slot (g, e) of step c
+            // is element g * HK + 8 c + e of the head dimension for the key and for the query alike
 #pragma unroll
-        for (int c = 0; c < KCH; ++c) {
-            float kf[16 / KESZ];
-            WS<KVBF16 ? WT_BF16 : WT_F32>::decode(kr[c], kf);
+            for (int c = 0; c < KCH; ++c) {
+                accS = pf_mma(kr[c], qh[KVBF16 ? c : 0], accS, false);
+                accS = pf_mma(kr[c], ql[KVBF16 ? c : 0], accS, false);
+            }
+        } else {
 #pragma unroll
-            for (int e = 0; e < 16 / KESZ; ++e)
-                accS = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[c * (16 / KESZ) + e], accS, 0, 0, 0);
+            for (int c = 0; c < KCH; ++c) {
+                float kf[16 / KESZ];
+                WS<KVBF16 ? WT_BF16 : WT_F32>::decode(kr[c], kf);
+#pragma unroll
+                for (int e = 0; e < 16 / KESZ; ++e)
+                    accS = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[c * (16 / KESZ) + e], accS, 0, 0, 0);
+            }
         }
         wave_sync();                           // the previous tile's V reads are done
+        if constexpr (KVBF16 != 0) {
 #pragma unroll
-        for (int c = 0; c < VCH; ++c) {
-            const int ch = lane + 64 * c, vrow = ch / CPR, cc = ch % CPR;
-            float vf[16 / KESZ];
-            WS<KVBF16 ? WT_BF16 : WT_F32>::decode(vr[c], vf);
-            float *dst = sV + vrow * VS + cc * (16 / KESZ);
+            for (int c = 0; c < VCH; ++c) {
+                const int ch = lane + 64 * c, vrow = ch / CPR, cc = ch % CPR;
+                *(uint4 *)(sVb + vrow * VSB + cc * 8) = vr[c];
+            }
+        } else {
 #pragma unroll
-            for (int e = 0; e < 16 / KESZ; e += 4) *(float4 *)(dst + e) = make_float4(vf[e], vf[e + 1], vf[e + 2], vf[e + 3]);
+            for (int c = 0; c < VCH; ++c) {
+                const int ch = lane + 64 * c, vrow = ch / CPR, cc = ch % CPR;
+                float vf[16 / KESZ];
+                WS<KVBF16 ? WT_BF16 : WT_F32>::decode(vr[c], vf);
+                float *dst = sV + vrow * VS + cc * (16 / KESZ);
+#pragma unroll
+                for (int e = 0; e < 16 / KESZ; e += 4) *(float4 *)(dst + e) = make_float4(vf[e], vf[e + 1], vf[e + 2], vf[e + 3]);
+            }
         }
         // online softmax for query row r over this tile's 32 keys (16 here, 16 in lane r ^ 32)
         float tmax = -1e30f;
@@ -886,12 +927,42 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void k_pf_attn(const float *__re
                 accO[nt][4 * j4 + 2] *= f.z; accO[nt][4 * j4 + 3] *= f.w;
             }
         }
+        if constexpr (KVBF16 != 0) {
+            // two steps of 16 keys: reduction slot (g, e) of step t is key 16 t + 8 (e / 4) + 4 g + e % 4, the
+            // key this lane's p[8 t + e] belongs to; the value operand gathers that key's column element
 #pragma unroll
-        for (int s = 0; s < 16; ++s) {
-            const int key = 8 * (s >> 2) + 4 * g + (s & 3);
+            for (int t = 0; t < 2; ++t) {
+                uint32_t ph[4], pl[4];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-                accO[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(p[s], sV[key * VS + 32 * nt + r], accO[nt], 0, 0, 0);
+                for (int e = 0; e < 4; ++e) {
+                    uint16_t h0, l0, h1, l1;
+                    pf_split(p[8 * t + 2 * e], h0, l0);
+                    pf_split(p[8 * t + 2 * e + 1], h1, l1);
+                    ph[e] = (uint32_t)h0 | ((uint32_t)h1 << 16);
+                    pl[e] = (uint32_t)l0 | ((uint32_t)l1 << 16);
+                }
+                const uint4 Ph = make_uint4(ph[0], ph[1], ph[2], ph[3]), Pl = make_uint4(pl[0], pl[1], pl[2], pl[3]);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    uint32_t vb[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int key = 16 * t + 8 * (e >> 1) + 4 * g + 2 * (e & 1);      // slots 2 e and 2 e + 1: this key and the next
+                        vb[e] = (uint32_t)sVb[key * VSB + 32 * nt + r] | ((uint32_t)sVb[(key + 1) * VSB + 32 * nt + r] << 16);
+                    }
+                    const uint4 Vb = make_uint4(vb[0], vb[1], vb[2], vb[3]);
+                    accO[nt] = pf_mma(Ph, Vb, accO[nt], false);
+                    accO[nt] = pf_mma(Pl, Vb, accO[nt], false);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < 16; ++s) {
+                const int key = 8 * (s >> 2) + 4 * g + (s & 3);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    accO[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(p[s], sV[key * VS + 32 * nt + r], accO[nt], 0, 0, 0);
+            }
         }
     }
     // merge the waves' partial results: O = sum_w e_w O_w / sum_w e_w l_w with e_w = exp(m_w - max m)
