@@ -95,6 +95,13 @@ int hipdec_create(const hipdec_config *cfg, const hipdec_layer_f32 *layers, size
                   const hipdec_head_f32 *head, const hipdec_options *opts, hipdec_model **out);
 void hipdec_destroy(hipdec_model *m);
 
+/* A second model on the weights `base` already holds on its device: same configuration and weight
+ * format, KV caches, step state and workspaces of its own, no upload.  The weights stay alive until the
+ * last model using them is destroyed (in any order).  (No counterpart in the reference, where every
+ * Model::new uploads its own copy, lib.rs:147-207; a server that keeps several prompts' sessions resident
+ * pays the weights once with this.) */
+int hipdec_create_shared(const hipdec_model *base, uint32_t kv_dtype, uint32_t flags, hipdec_model **out);
+
 /* Text of the last error on this model (or of the last failed hipdec_create when m is NULL). */
 const char *hipdec_last_error(const hipdec_model *m);
 

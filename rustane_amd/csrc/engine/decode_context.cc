@@ -80,6 +80,17 @@ DecodeContext::DecodeContext(const ModelConfig &cfg, const ModelWeights &weights
     int rc = hipdec_create(&c, layers.data(), layers.size(), &head, &o, &m_);
     if (rc != HIPDEC_OK)
         throw std::runtime_error(std::string("failed to initialize hip decode: ") + hipdec_last_error(nullptr));
+    init_buffers(cfg);
+}
+
+DecodeContext::DecodeContext(const ModelConfig &cfg, const DecodeContext &weights_of, KvDtype kvdt, uint32_t flags) {
+    int rc = hipdec_create_shared(weights_of.m_, (uint32_t)kvdt, flags, &m_);
+    if (rc != HIPDEC_OK)
+        throw std::runtime_error(std::string("failed to initialize hip decode: ") + hipdec_last_error(nullptr));
+    init_buffers(cfg);
+}
+
+void DecodeContext::init_buffers(const ModelConfig &cfg) {
     vocab_ = cfg.vocab;
     blocks_ = (cfg.vocab + HIPDEC_HEAD_BLOCK - 1) / HIPDEC_HEAD_BLOCK;
     // decode.rs:200-216

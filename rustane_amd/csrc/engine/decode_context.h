@@ -28,6 +28,9 @@ public:
     // decode.rs:34-71 (throws std::runtime_error where the reference `expect`s)
     DecodeContext(const ModelConfig &cfg, const ModelWeights &weights, WeightDtype wdt = WeightDtype::F32,
                   KvDtype kvdt = KvDtype::F32, int device = 0, uint32_t flags = 0);
+    // a context on the device weights another context already holds (hipdec_create_shared): no upload,
+    // KV caches and step state of its own; the weights live as long as any context that uses them
+    DecodeContext(const ModelConfig &cfg, const DecodeContext &weights_of, KvDtype kvdt, uint32_t flags);
     ~DecodeContext();
     DecodeContext(const DecodeContext &) = delete;
     DecodeContext &operator=(const DecodeContext &) = delete;
@@ -88,6 +91,7 @@ public:
 
 private:
     void check(int rc, const char *what) const;
+    void init_buffers(const ModelConfig &cfg);
     hipdec_model *m_ = nullptr;
     size_t vocab_ = 0, blocks_ = 0;
     // decode.rs:19-31 DecodeWorkspace

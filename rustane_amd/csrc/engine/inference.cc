@@ -196,7 +196,7 @@ size_t fill_input_window(const std::vector<uint32_t> &generated, size_t seq, std
 
 InferenceSession::InferenceSession(const ModelConfig &cfg, const ModelWeights &weights,
                                    const std::vector<uint32_t> &prompt_ids, float softcap, const SessionOptions &opts,
-                                   std::string *err)
+                                   std::string *err, InferenceSession *share_weights_with)
     : cfg_(cfg), prompt_ids_(prompt_ids), softcap_(softcap), device_sampling_(opts.device_sampling),
       batch_samples_(opts.batch_samples) {
     err->clear();
@@ -204,7 +204,10 @@ InferenceSession::InferenceSession(const ModelConfig &cfg, const ModelWeights &w
     *err = validate_token_ids(prompt_ids.data(), prompt_ids.size(), cfg.vocab, "prompt");
     if (!err->empty()) return;
     try {
-        ctx_.reset(new DecodeContext(cfg, weights, opts.weight_dtype, opts.kv_dtype, opts.device, opts.flags));
+        if (share_weights_with && share_weights_with->ctx_)
+            ctx_.reset(new DecodeContext(cfg, *share_weights_with->ctx_, opts.kv_dtype, opts.flags));
+        else
+            ctx_.reset(new DecodeContext(cfg, weights, opts.weight_dtype, opts.kv_dtype, opts.device, opts.flags));
         prompt_len_ = fill_input_window(prompt_ids, cfg.seq, &input_);
         const double t0 = now_s();
         prompt_logits_ = ctx_->prefill(input_.data(), prompt_len_, softcap);                         // :139-144

@@ -97,8 +97,11 @@ struct SessionOptions {
 // (empty on success); construction failure leaves ok() false.
 class InferenceSession {
 public:
+    // share_weights_with: a live session of the same model whose device weights this one uses instead of
+    // uploading its own (the session cache keeps several prompts resident on one copy of the weights)
     InferenceSession(const ModelConfig &cfg, const ModelWeights &weights, const std::vector<uint32_t> &prompt_ids,
-                     float softcap, const SessionOptions &opts, std::string *err);
+                     float softcap, const SessionOptions &opts, std::string *err,
+                     InferenceSession *share_weights_with = nullptr);
     bool ok() const { return ctx_ != nullptr; }
     const std::vector<uint32_t> &prompt_ids() const { return prompt_ids_; }
     size_t prompt_len() const { return prompt_len_; }

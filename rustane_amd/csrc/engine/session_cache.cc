@@ -42,7 +42,9 @@ void SessionCache::evict_lru() {
 }
 
 long SessionCache::insert(const std::vector<uint32_t> &p, std::string *err) {
-    std::unique_ptr<InferenceSession> s(new InferenceSession(cfg_, weights_, p, softcap_, opts_, err));
+    // every entry after the first runs on the device weights of an entry that is already there
+    InferenceSession *donor = entries_.empty() ? nullptr : entries_.front().session.get();
+    std::unique_ptr<InferenceSession> s(new InferenceSession(cfg_, weights_, p, softcap_, opts_, err, donor));
     if (!s->ok()) return -1;
     if (entries_.size() >= max_entries_) evict_lru();
     Entry e;

@@ -14,6 +14,7 @@
 #include <vector>
 #include <algorithm>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <thread>
 
@@ -21,6 +22,8 @@ namespace {
 
 // V_TOPK_S / V_STATS_S: the same step followed by the on-device draw (hipdec_sample.h)
 enum Variant { V_X = 0, V_ARGMAX, V_TOPK, V_STATS, V_LOGITS, V_TOPK_S, V_STATS_S, V_COUNT };
+
+struct WeightStore;
 
 struct DevLayer {
     void *wqkv = nullptr, *wo = nullptr, *w13 = nullptr, *w2 = nullptr;
@@ -114,6 +117,7 @@ struct hipdec_model {
     uint64_t *d_rng = nullptr;                        // [32], one state per row
     SampleHost *h_samp = nullptr;                     // pinned
     std::vector<void *> allocs;
+    std::shared_ptr<WeightStore> wstore;   // the weights (read-only after creation), possibly shared with other models
     std::string err;
 };
 
@@ -169,10 +173,30 @@ void uncached_give(int device, size_t cap, void *p) {
     pool.idle.insert({{device, cap}, p});
 }
 
+// device memory of a model's weights: shared (reference-counted) by the models created from one another
+// with hipdec_create_shared, freed with the last of them
+struct WeightStore {
+    int device = 0;
+    std::vector<void *> allocs;
+    ~WeightStore() {
+        (void)hipSetDevice(device);
+        for (void *p : allocs) (void)hipFree(p);
+    }
+};
+
+template <typename T> int walloc(hipdec_model *m, T **p, size_t bytes);
 template <typename T> int dalloc(hipdec_model *m, T **p, size_t bytes) {
     void *v = nullptr;
     HCHK(hipMalloc(&v, bytes ? bytes : 16));
     m->allocs.push_back(v);
+    *p = (T *)v;
+    return HIPDEC_OK;
+}
+
+template <typename T> int walloc(hipdec_model *m, T **p, size_t bytes) {
+    void *v = nullptr;
+    HCHK(hipMalloc(&v, bytes ? bytes : 16));
+    m->wstore->allocs.push_back(v);
     *p = (T *)v;
     return HIPDEC_OK;
 }
@@ -1065,7 +1089,9 @@ void hipdec_destroy(hipdec_model *m) {
     delete m;
 }
 
-static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hipdec_head_f32 *head) {
+// base != null: the new model takes base's weights (same configuration and weight format) instead of uploading any
+static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hipdec_head_f32 *head,
+                       const hipdec_model *base = nullptr) {
     const hipdec_config &c = m->cfg;
     const size_t D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden, V = c.vocab, S = c.seq;
     HCHK(hipSetDevice(m->opt.device));
@@ -1082,8 +1108,14 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
     if (D * H > max_elems) max_elems = D * H;
     if (D * Q > max_elems) max_elems = D * Q;
     float *stage_a = nullptr, *stage_b = nullptr;
-    HCHK(hipMalloc((void **)&stage_a, max_elems * sizeof(float)));
-    HCHK(hipMalloc((void **)&stage_b, max_elems * sizeof(float)));
+    if (base) {
+        m->wstore = base->wstore;
+    } else {
+        m->wstore = std::make_shared<WeightStore>();
+        m->wstore->device = m->opt.device;
+        HCHK(hipMalloc((void **)&stage_a, max_elems * sizeof(float)));
+        HCHK(hipMalloc((void **)&stage_b, max_elems * sizeof(float)));
+    }
     int rc = HIPDEC_OK;
     auto done = [&](int code) { (void)hipFree(stage_a); (void)hipFree(stage_b); return code; };
 
@@ -1092,24 +1124,29 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
     m->layers.resize(c.nlayers);
     for (uint32_t l = 0; l < c.nlayers && rc == HIPDEC_OK; ++l) {
         DevLayer &L = m->layers[l];
-        const hipdec_layer_f32 &src = layers[l];
-        if (!src.wq || !src.wk || !src.wv || !src.wo || !src.w1 || !src.w3 || !src.w2 || !src.gamma1 || !src.gamma2)
-            return done(fail(m, HIPDEC_ERR_ARG, "null layer weight pointer"));
 #define TRY(x) do { rc = (x); if (rc != HIPDEC_OK) return done(rc); } while (0)
-        TRY(dalloc(m, &L.wqkv, wt_row_bytes(wt, D) * (Q + 2 * KV)));
-        TRY(dalloc(m, &L.wo, wt_row_bytes(wt, Q) * D));
-        TRY(dalloc(m, &L.w13, wt_row_bytes(wt, D) * 2 * H));
-        TRY(dalloc(m, &L.w2, wt_row_bytes(wt, H) * D));
-        TRY(dalloc(m, &L.s_qkv, wt_scale_bytes(wt, Q + 2 * KV, D)));
-        TRY(dalloc(m, &L.s_wo, wt_scale_bytes(wt, D, Q)));
-        TRY(dalloc(m, &L.s_w13, wt_scale_bytes(wt, 2 * H, D)));
-        TRY(dalloc(m, &L.s_w2, wt_scale_bytes(wt, D, H)));
-        TRY(dalloc(m, &L.g1, D * 4));
-        TRY(dalloc(m, &L.g2, D * 4));
+        if (base) {
+            L = base->layers[l];                       // weight, scale and norm pointers; the caches are this model's own
+            L.kc = nullptr; L.vc = nullptr;
+        }
         TRY(dalloc(m, &L.kc, S * KV * kvsz));
         TRY(dalloc(m, &L.vc, S * KV * kvsz));
         HCHK(hipMemsetAsync(L.kc, 0, S * KV * kvsz, m->stream));
         HCHK(hipMemsetAsync(L.vc, 0, S * KV * kvsz, m->stream));
+        if (base) continue;
+        const hipdec_layer_f32 &src = layers[l];
+        if (!src.wq || !src.wk || !src.wv || !src.wo || !src.w1 || !src.w3 || !src.w2 || !src.gamma1 || !src.gamma2)
+            return done(fail(m, HIPDEC_ERR_ARG, "null layer weight pointer"));
+        TRY(walloc(m, &L.wqkv, wt_row_bytes(wt, D) * (Q + 2 * KV)));
+        TRY(walloc(m, &L.wo, wt_row_bytes(wt, Q) * D));
+        TRY(walloc(m, &L.w13, wt_row_bytes(wt, D) * 2 * H));
+        TRY(walloc(m, &L.w2, wt_row_bytes(wt, H) * D));
+        TRY(walloc(m, &L.s_qkv, wt_scale_bytes(wt, Q + 2 * KV, D)));
+        TRY(walloc(m, &L.s_wo, wt_scale_bytes(wt, D, Q)));
+        TRY(walloc(m, &L.s_w13, wt_scale_bytes(wt, 2 * H, D)));
+        TRY(walloc(m, &L.s_w2, wt_scale_bytes(wt, D, H)));
+        TRY(walloc(m, &L.g1, D * 4));
+        TRY(walloc(m, &L.g2, D * 4));
         TRY(load_matrix(m, wt, src.wq, Q, D, true, stage_a, stage_b, L.wqkv, L.s_qkv, 1, 0));
         TRY(load_matrix(m, wt, src.wk, KV, D, true, stage_a, stage_b, L.wqkv, L.s_qkv, 1, (int)Q));
         TRY(load_matrix(m, wt, src.wv, KV, D, true, stage_a, stage_b, L.wqkv, L.s_qkv, 1, (int)(Q + KV)));
@@ -1120,10 +1157,15 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
         HCHK(hipMemcpy(L.g1, src.gamma1, D * 4, hipMemcpyHostToDevice));
         HCHK(hipMemcpy(L.g2, src.gamma2, D * 4, hipMemcpyHostToDevice));
     }
-    TRY(dalloc(m, &m->embed, wt_row_bytes(m->embed_wt, D) * V));
-    TRY(load_matrix(m, m->embed_wt, head->embed, V, D, false, stage_a, stage_b, m->embed, nullptr, 1, 0));
-    TRY(dalloc(m, &m->gfinal, D * 4));
-    HCHK(hipMemcpy(m->gfinal, head->gamma_final, D * 4, hipMemcpyHostToDevice));
+    if (base) {
+        m->embed = base->embed;
+        m->gfinal = base->gfinal;
+    } else {
+        TRY(walloc(m, &m->embed, wt_row_bytes(m->embed_wt, D) * V));
+        TRY(load_matrix(m, m->embed_wt, head->embed, V, D, false, stage_a, stage_b, m->embed, nullptr, 1, 0));
+        TRY(walloc(m, &m->gfinal, D * 4));
+        HCHK(hipMemcpy(m->gfinal, head->gamma_final, D * 4, hipMemcpyHostToDevice));
+    }
 
     m->blocks = (int)((V + HIPDEC_HEAD_BLOCK - 1) / HIPDEC_HEAD_BLOCK);
     int ns = (int)(256 / c.heads);
@@ -1324,6 +1366,38 @@ int hipdec_create(const hipdec_config *cfg, const hipdec_layer_f32 *layers, size
                                                            : PF_ACT_PAIR;
     m->alpha = 1.0f / sqrtf(2.0f * (float)c.nlayers);   // lib.rs:201
     int rc = create_impl(m, layers, head);
+    if (rc != HIPDEC_OK) {
+        g_create_error = m->err;
+        hipdec_destroy(m);
+        return rc;
+    }
+    *out = m;
+    return HIPDEC_OK;
+}
+
+int hipdec_create_shared(const hipdec_model *base, uint32_t kv_dtype, uint32_t flags, hipdec_model **out) {
+    if (!base || !out) return fail(nullptr, HIPDEC_ERR_ARG, "null argument");
+    *out = nullptr;
+    if (kv_dtype > HIPDEC_KV_BF16) return fail(nullptr, HIPDEC_ERR_ARG, "unknown kv_dtype");
+    hipdec_model *m = new hipdec_model();
+    m->cfg = base->cfg;
+    hipdec_options o = base->opt;
+    o.kv_dtype = kv_dtype;
+    o.flags = flags;
+    if (const char *e = getenv("HIPDEC_NO_GRAPH")) if (e[0] == '1') o.flags |= HIPDEC_FLAG_NO_GRAPH;
+    if (const char *e = getenv("HIPDEC_PREFILL_STEPS")) if (e[0] == '1') o.flags |= HIPDEC_FLAG_PREFILL_STEPS;
+    m->opt = o;
+    m->wt = base->wt;
+    m->embed_wt = base->embed_wt;
+    m->kvbf16 = kv_dtype == HIPDEC_KV_BF16;
+    const bool quantised = o.weight_dtype == HIPDEC_W_FP8_E4M3 || o.weight_dtype == HIPDEC_W_INT4_G128;
+    m->pf_act = (o.flags & HIPDEC_FLAG_PREFILL_PAIR_ACT)   ? PF_ACT_PAIR
+                : (o.flags & HIPDEC_FLAG_PREFILL_BF16_ACT) ? PF_ACT_BF16
+                : (o.flags & HIPDEC_FLAG_PREFILL_F16_ACT)  ? PF_ACT_F16
+                : (m->kvbf16 && quantised)                 ? PF_ACT_F16
+                                                           : PF_ACT_PAIR;
+    m->alpha = base->alpha;
+    const int rc = create_impl(m, nullptr, nullptr, base);
     if (rc != HIPDEC_OK) {
         g_create_error = m->err;
         hipdec_destroy(m);

@@ -20,7 +20,7 @@ HEAD_BLOCK = 256
 OK, ERR_ARG, ERR_FULL, ERR_HIP, ERR_UNSUPPORTED = 0, 1, 2, 3, 4
 
 EXPORTS = [
-    "hipdec_create", "hipdec_destroy", "hipdec_last_error", "hipdec_len", "hipdec_set_len", "hipdec_set_prefill_activations",
+    "hipdec_create", "hipdec_create_shared", "hipdec_destroy", "hipdec_last_error", "hipdec_len", "hipdec_set_len", "hipdec_set_prefill_activations",
     "hipdec_seed_layer_cache_from_channel_first", "hipdec_decode_token", "hipdec_decode_token_from_id",
     "hipdec_decode_token_argmax", "hipdec_decode_token_argmax_from_id", "hipdec_decode_token_topk_from_id",
     "hipdec_decode_token_block_stats_from_id", "hipdec_materialize_current_logits_block",
@@ -272,6 +272,20 @@ class HipDecodeModel:
             raise HipDecodeError(rc, (self._lib.hipdec_last_error(None) or b"").decode())
         self.blocks = (V + HEAD_BLOCK - 1) // HEAD_BLOCK
         self._rows = 0
+
+    def create_shared(self, kv_dtype=KvDtype.F32, flags=0):
+        """A second model on this model's device weights (no upload): own KV caches and step state."""
+        other = object.__new__(HipDecodeModel)
+        other._lib = self._lib
+        other._h = C.c_void_p()
+        other.cfg = self.cfg
+        self._lib.hipdec_create_shared.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(C.c_void_p)]
+        rc = self._lib.hipdec_create_shared(self._h, int(kv_dtype), int(flags), C.byref(other._h))
+        if rc != OK:
+            raise HipDecodeError(rc, (self._lib.hipdec_last_error(None) or b"").decode())
+        other.blocks = self.blocks
+        other._rows = 0
+        return other
 
     def close(self):
         if getattr(self, "_h", None) and self._h.value:

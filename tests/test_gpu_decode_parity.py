@@ -328,3 +328,56 @@ def test_graph_replay_equals_eager_launch_and_runs_repeat_bit_for_bit(wdt, kvdt)
     for x, y, z in zip(a, b, c):
         np.testing.assert_array_equal(x.view(np.uint32), y.view(np.uint32))
         np.testing.assert_array_equal(x.view(np.uint32), z.view(np.uint32))
+
+
+def _free_device_bytes():
+    import ctypes as C
+    rt = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(), C.c_size_t()
+    assert rt.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
+@pytest.mark.gpu
+def test_models_sharing_one_copy_of_the_weights():
+    """hipdec_create_shared: a second model on the first one's device weights (the reference uploads per
+    Model::new, crates/metal-decode/src/lib.rs:147-207).  Both give the logits of an independently created
+    model, bit for bit, with their own caches and positions; the second costs caches and workspaces, not
+    weights; the weights outlive the model that uploaded them."""
+    cfg = Config.make(dim=512, hidden=2048, heads=4, hd=128, seq=64, nlayers=4, vocab=4096)
+    w = synth.make_weights(cfg, seed=21, std=0.06, round_bf16=True)
+    weight_bytes = 2 * (cfg.nlayers * (4 * cfg.dim * cfg.dim + 3 * cfg.dim * cfg.hidden) + cfg.vocab * cfg.dim)
+    ids_a = synth.make_prompt(5, cfg.vocab, 12)
+    ids_b = synth.make_prompt(6, cfg.vocab, 20)
+    ref = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.F32)
+    want_a, want_b = ref.prefill(ids_a), None
+    ref.set_len(0)
+    want_b = ref.prefill(ids_b)
+    ref.close()
+
+    before = _free_device_bytes()
+    base = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.F32)
+    after_base = _free_device_bytes()
+    twin = base.create_shared(kv_dtype=KvDtype.F32)
+    after_twin = _free_device_bytes()
+    assert before - after_base >= weight_bytes                         # the first model holds the weights ...
+    assert after_base - after_twin < weight_bytes // 4                 # ... the second one only caches and workspaces
+    np.testing.assert_array_equal(base.prefill(ids_a), want_a)
+    np.testing.assert_array_equal(twin.prefill(ids_b), want_b)         # interleaved use, separate caches
+    assert (base.len(), twin.len()) == (12, 20)
+    ta, tb = int(np.argmax(want_a)), int(np.argmax(want_b))
+    la, lb = base.decode_logits_from_id(ta), twin.decode_logits_from_id(tb)
+    base.close()                                                       # the uploader goes first
+    ref2 = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.F32)
+    ref2.prefill(ids_b)
+    np.testing.assert_array_equal(ref2.decode_logits_from_id(tb), lb)
+    np.testing.assert_array_equal(twin.decode_greedy_run(int(np.argmax(lb)), 8), ref2.decode_greedy_run(int(np.argmax(lb)), 8))
+    ref2.set_len(0)
+    ref2.prefill(ids_a)
+    np.testing.assert_array_equal(ref2.decode_logits_from_id(ta), la)
+    # a bf16 cache on the same weights
+    twin16 = twin.create_shared(kv_dtype=KvDtype.BF16)
+    solo16 = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.BF16)
+    np.testing.assert_array_equal(twin16.prefill(ids_a), solo16.prefill(ids_a))
+    twin.close()
+    np.testing.assert_array_equal(twin16.decode_logits_from_id(ta), solo16.decode_logits_from_id(ta))
