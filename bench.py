@@ -49,7 +49,7 @@ ALL_CONFIG_STEPS = {"c1_tiny_fp32": 31, "c2_600m_bf16_bs1": 255, "c3_600m_bf16_8
 # (per step, i.e. the LM-head GEMV included where it is a launch of its own, at the KV length of the
 # profiled run); a benchmark run cannot collect it itself.
 TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries under profiles/, not measured in this run"
-MEASURED_TRAFFIC_BYTES = {"c1_tiny_fp32": 1.267e8, "c2_600m_bf16_bs1": 1.5068e9, "c4_5b_bf16_bs1": 1.3874e10,
+MEASURED_TRAFFIC_BYTES = {"c1_tiny_fp32": 1.267e8, "c2_600m_bf16_bs1": 1.5083e9, "c4_5b_bf16_bs1": 1.3874e10,
                           "c5_5b_fp8_bs1": 7.118e9, "c5_5b_int4_bs1": 4.008e9}
 
 
