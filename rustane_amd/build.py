@@ -8,6 +8,7 @@ LIBDIR = os.path.join(ROOT, "lib")
 HIPDECODE_SO = os.path.join(LIBDIR, "libhipdecode.so")
 ENGINE_SO = os.path.join(LIBDIR, "librustane_engine.so")
 GENERATE_BIN = os.path.join(LIBDIR, "generate")
+SERVE_BIN = os.path.join(LIBDIR, "serve")
 
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -39,9 +40,8 @@ def build_engine():
     inc = os.path.join(os.path.dirname(ROOT), "include")
     _run(["g++"] + CXX_FLAGS + ["-shared", "-I", inc] + engine_sources() +
          ["-o", ENGINE_SO, "-L", LIBDIR, "-lhipdecode", "-Wl,-rpath,$ORIGIN"])
-    main = os.path.join(CSRC, "engine", "generate_main.cc")
-    if os.path.exists(main):
-        _run(["g++"] + CXX_FLAGS + ["-I", inc, main, "-o", GENERATE_BIN, "-L", LIBDIR,
+    for src, out in (("generate_main.cc", GENERATE_BIN), ("serve_main.cc", SERVE_BIN)):
+        _run(["g++"] + CXX_FLAGS + ["-I", inc, os.path.join(CSRC, "engine", src), "-o", out, "-L", LIBDIR,
                                     "-lrustane_engine", "-lhipdecode", "-Wl,-rpath,$ORIGIN"])
     return ENGINE_SO
 

@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "checkpoint.h"
+#include "http_server.h"
 #include "inference.h"
 #include "jsonl_session.h"
 #include "session_cache.h"
@@ -309,6 +310,47 @@ int rs_jsonl_parse(const char *line, const rs_request *defaults, rs_request *out
     out->top_k = req.top_k; out->samples = req.samples; out->seed = req.seed;
     *n_suffix = sfx.size();
     for (size_t i = 0; i < sfx.size() && i < cap; ++i) suffix[i] = sfx[i];
+    return 0;
+}
+
+// ---- the HTTP front end (bin/serve.rs) without a model behind it
+// Reads one request from a connected socket.  0 = ok, 1 = refused (err holds the message of the 400 answer).
+int rs_http_parse_request(int fd, uint64_t max_body, char *method, size_t mcap, char *path, size_t pcap, char *body,
+                          size_t bcap, uint64_t *body_len, char *err, size_t errcap) {
+    HttpRequest req;
+    std::string e;
+    if (!parse_http_request(fd, &req, &e, (size_t)max_body)) { put_err(err, errcap, e); return 1; }
+    put_err(method, mcap, req.method);
+    put_err(path, pcap, req.path);
+    *body_len = req.body.size();
+    if (body && bcap) memcpy(body, req.body.data(), req.body.size() < bcap ? req.body.size() : bcap);
+    return 0;
+}
+// The body of POST /v1/completions (chat = 0) or /v1/chat/completions (chat = 1) turned into prompt ids and a
+// generation request, as the server does before it generates.  0 = ok, 1 = refused by validation, 2 = invalid JSON.
+int rs_http_prepare(const char *body, int chat, const char *model_name, uint64_t vocab, uint32_t default_backend,
+                    rs_request *out, int *stream, uint32_t *ids, size_t cap, uint64_t *n_ids, char *err, size_t errcap) {
+    CompletionRequest parsed;
+    std::string e;
+    if (!parse_completion_request(body, chat != 0, &parsed, &e)) { put_err(err, errcap, e); return 2; }
+    ModelConfig cfg = ModelConfig::make(128, 256, 1, 1, 128, 16, 1, vocab);
+    HttpServer server(cfg, nullptr, model_name, (DecodeBackendRequest)default_backend);
+    std::vector<uint32_t> prompt;
+    GenerationRequest req;
+    if (!server.prepare(parsed, chat != 0, &prompt, &req, &e)) { put_err(err, errcap, e); return 1; }
+    out->backend = (uint32_t)req.decode_backend; out->steps = req.steps; out->temperature = req.temperature;
+    out->top_k = req.top_k; out->samples = req.samples; out->seed = req.seed;
+    *stream = parsed.has_stream && parsed.stream;
+    *n_ids = prompt.size();
+    for (size_t i = 0; i < prompt.size() && i < cap; ++i) ids[i] = prompt[i];
+    return 0;
+}
+// bin/serve.rs:616-633 over the "messages" of a chat request body.  0 = ok, 2 = invalid JSON.
+int rs_http_render_chat_prompt(const char *body, char *out, size_t cap, char *err, size_t errcap) {
+    CompletionRequest parsed;
+    std::string e;
+    if (!parse_completion_request(body, true, &parsed, &e)) { put_err(err, errcap, e); return 2; }
+    put_err(out, cap, render_chat_prompt(parsed.messages));
     return 0;
 }
 

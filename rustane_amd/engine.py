@@ -71,6 +71,11 @@ def lib():
         L.rs_checkpoint_write.argtypes = [C.c_char_p, C.POINTER(RsConfig), C.c_void_p, C.c_uint32, C.c_char_p, C.c_size_t]
         L.rs_jsonl_parse.argtypes = [C.c_char_p, C.POINTER(RsRequest), C.POINTER(RsRequest), u32p, C.c_size_t, u64p,
                                      C.c_char_p, C.c_size_t]
+        L.rs_http_parse_request.argtypes = [C.c_int, C.c_uint64, C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t, C.c_char_p,
+                                            C.c_size_t, u64p, C.c_char_p, C.c_size_t]
+        L.rs_http_prepare.argtypes = [C.c_char_p, C.c_int, C.c_char_p, C.c_uint64, C.c_uint32, C.POINTER(RsRequest),
+                                      C.POINTER(C.c_int), u32p, C.c_size_t, u64p, C.c_char_p, C.c_size_t]
+        L.rs_http_render_chat_prompt.argtypes = [C.c_char_p, C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t]
         L.rs_weights_tensor.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.POINTER(fp), u64p]
         L.rs_session_new.restype = C.c_void_p
         L.rs_session_new.argtypes = [C.POINTER(RsConfig), C.c_void_p, u32p, C.c_size_t, C.c_float, C.c_uint32,
@@ -479,3 +484,51 @@ def parse_jsonl_request(line, defaults=None):
         raise JsonlRequestError(err.value.decode())
     req = GenerationRequest(DecodeBackendRequest(out.backend), out.steps, out.temperature, out.top_k, out.samples, out.seed)
     return req, buf[:n.value].copy()
+
+
+# ---------------------------------------------------------------- HTTP front end (bin/serve.rs), the parts that need no model
+class HttpRequestError(ValueError):
+    """A request the server answers with status 400; `invalid_json` tells a body that does not parse from one
+    that parses and is refused by validation."""
+
+    def __init__(self, message, invalid_json=False):
+        super().__init__(message)
+        self.invalid_json = invalid_json
+
+
+def http_parse_request(fd, max_body=64 << 20):
+    """Reads one HTTP request from a connected socket -> (method, path, body bytes)."""
+    L = lib()
+    method, path, err = C.create_string_buffer(64), C.create_string_buffer(4096), C.create_string_buffer(512)
+    cap = 1 << 20
+    body, n = C.create_string_buffer(cap), C.c_uint64()
+    if L.rs_http_parse_request(fd, max_body, method, 64, path, 4096, body, cap, C.byref(n), err, 512):
+        raise HttpRequestError(err.value.decode())
+    return method.value.decode(), path.value.decode(), body.raw[:min(n.value, cap)]
+
+
+def http_prepare(body, chat=False, model_name="rustane", vocab=8192, default_backend=DecodeBackendRequest.AUTO):
+    """The body of a (chat) completion request -> (prompt ids, GenerationRequest, stream flag), as the server
+    derives them before generating (bin/serve.rs:635-725)."""
+    L = lib()
+    out, n, stream, err = RsRequest(), C.c_uint64(), C.c_int(), C.create_string_buffer(512)
+    buf = np.zeros(4096, np.uint32)
+    if isinstance(body, str):
+        body = body.encode()
+    rc = L.rs_http_prepare(body, int(chat), model_name.encode(), vocab, int(default_backend), C.byref(out), C.byref(stream),
+                           buf.ctypes.data_as(C.POINTER(C.c_uint32)), buf.size, C.byref(n), err, 512)
+    if rc:
+        raise HttpRequestError(err.value.decode(), invalid_json=rc == 2)
+    req = GenerationRequest(DecodeBackendRequest(out.backend), out.steps, out.temperature, out.top_k, out.samples, out.seed)
+    return buf[:n.value].copy(), req, bool(stream.value)
+
+
+def http_render_chat_prompt(body):
+    """The flattened prompt text of a chat request's messages (bin/serve.rs:616-633)."""
+    L = lib()
+    out, err = C.create_string_buffer(1 << 16), C.create_string_buffer(512)
+    if isinstance(body, str):
+        body = body.encode()
+    if L.rs_http_render_chat_prompt(body, out, 1 << 16, err, 512):
+        raise HttpRequestError(err.value.decode(), invalid_json=True)
+    return out.value.decode()
