@@ -553,15 +553,17 @@ PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K, bool dl =
         return PfSplit{(lsteps + sps - 1) / sps, sps};
     }
     const int nsteps = K / PF_BK;
-    if (T <= kSkinnyRows && wt != WT_INT4) {      // (4-bit weights always take the tiled kernel)
+    if (T <= kSkinnyRows) {
         // 4 waves per workgroup share a K range; aim at ~8 waves per CU over the whole grid
         const int tiles = (N + 31) / 32;
         int s = std::max(1, (2 * m->num_cu) / tiles);
         s = std::min(s, std::max(1, nsteps / 8));
         // the workgroup's slice of the activation rows (hi + lo) has to fit its LDS budget
-        const int max_steps = std::max(1, ((kSkinnyLdsBytes / (4 * T)) - PF_SK_PAD) / PF_BK);
+        int max_steps = std::max(1, ((kSkinnyLdsBytes / (4 * T)) - PF_SK_PAD) / PF_BK);
+        if (wt == WT_INT4) max_steps = std::max(4, max_steps & ~3);   // a split covers whole scale groups (four steps each)
         s = std::max(s, (nsteps + max_steps - 1) / max_steps);
-        const int sps = (nsteps + s - 1) / s;
+        int sps = (nsteps + s - 1) / s;
+        if (wt == WT_INT4) sps = std::min(max_steps, (sps + 3) & ~3);
         return PfSplit{(nsteps + sps - 1) / sps, sps};
     }
     const int bn = PF_BN_OF(wt);
@@ -626,11 +628,12 @@ int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, c
     }
     const PfSplit sp = pf_split_k(m, wt, T, N, K);
     PfGemm g{Ahi, Alo, W, wt == WT_INT4 ? (const uint16_t *)scales : nullptr, m->pf.P, T, N, K, sp.steps_per_split};
-    if (T <= kSkinnyRows && wt != WT_INT4) {
+    if (T <= kSkinnyRows) {
         dim3 grid((N + 31) / 32, sp.splits), block(256);
         const size_t lds = (size_t)2 * T * (sp.steps_per_split * PF_BK + PF_SK_PAD) * 2;
         if (wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_BF16>, grid, block, lds, m->stream, g);
-        else hipLaunchKernelGGL(k_pf_gemm_skinny<WT_FP8>, grid, block, lds, m->stream, g);
+        else if (wt == WT_FP8) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_FP8>, grid, block, lds, m->stream, g);
+        else hipLaunchKernelGGL(k_pf_gemm_skinny<WT_INT4>, grid, block, lds, m->stream, g);
         return sp.splits;
     }
     const int bn = PF_BN_OF(wt);
@@ -694,7 +697,7 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
         memcpy(w.h_ids, ids + done, (size_t)T * 4);
         HCHK(hipMemcpyAsync(w.ids, w.h_ids, (size_t)T * 4, hipMemcpyHostToDevice, m->stream));
         // how this chunk's activations travel between its kernels (the few-row GEMM only takes pairs)
-        const bool tiled = !(T <= kSkinnyRows && m->wt != WT_INT4);
+        const bool tiled = T > kSkinnyRows;
         const int act = !tiled ? PF_ACT_PAIR : m->pf_act;
         const int f16 = act == PF_ACT_F16;
         pf_launch_embed(m, T, f16);

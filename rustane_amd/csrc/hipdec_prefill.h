@@ -659,6 +659,9 @@ __global__ __launch_bounds__(64 * WAVES, WGS) void k_pf_gemm_dl(PfGemm g) {
 // workgroup's slice of the few activation rows (hi and lo parts) is staged once in LDS while the
 // first weight loads are in flight; rows past T read row T-1 and are not stored.  The four partial
 // tiles are summed through LDS in wave order.
+// 4-bit weights: a lane's 16 elements of a step are 8 bytes; the PF_SK_UNROLL = 4 steps issued together are
+// exactly one scale group of 128 elements (the host makes every K split, and the kernel every wave's part,
+// a whole number of groups), whose products are summed unscaled and enter the result times the row's scale.
 #define PF_SK_UNROLL 4     // 32-element steps whose loads are issued together
 #define PF_SK_PAD 8        // bf16 elements of padding per staged activation row
 template <int WT>
@@ -670,13 +673,15 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
     const int n0 = blockIdx.x * 32, z = blockIdx.y;
     const int nsteps = g.K / PF_BK;
     const int zb = z * g.steps_per_split, ze = min(nsteps, zb + g.steps_per_split);
-    const int per_wave = (ze - zb + 3) / 4;
+    const int per_wave = WT == WT_INT4 ? (((ze - zb + 3) / 4 + PF_SK_UNROLL - 1) / PF_SK_UNROLL) * PF_SK_UNROLL : (ze - zb + 3) / 4;
     const int s_begin = min(ze, zb + wave * per_wave), s_end = min(ze, s_begin + per_wave);
     const size_t na = (size_t)min(n0 + r, g.N - 1);
     const int krange = (ze - zb) * PF_BK, astride = g.steps_per_split * PF_BK + PF_SK_PAD;
     const uint16_t *ah = s_act + min(r, g.T - 1) * astride + 16 * gq;
     const uint16_t *al = ah + g.T * astride;
-    const char *wp = (const char *)g.W + na * (WT == WT_BF16 ? (size_t)g.K * 2 : (size_t)g.K) + (WT == WT_BF16 ? 32 : 16) * gq;
+    // bytes of a weight row, and of this lane's 16 elements of a step
+    const char *wp = (const char *)g.W + na * (WT == WT_BF16 ? (size_t)g.K * 2 : WT == WT_INT4 ? (size_t)g.K / 2 : (size_t)g.K) +
+                     (WT == WT_BF16 ? 32 : WT == WT_INT4 ? 8 : 16) * gq;
 
     uint4 w[PF_SK_UNROLL][2];
     auto wload = [&](int s0) {
@@ -687,6 +692,9 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
             if (WT == WT_BF16) {
                 w[u][0] = *(const uint4 *)(wp + k0 * 2);
                 w[u][1] = *(const uint4 *)(wp + k0 * 2 + 16);
+            } else if (WT == WT_INT4) {
+                const uint2 v = *(const uint2 *)(wp + k0 / 2);
+                w[u][0] = make_uint4(v.x, v.y, 0u, 0u);
             } else {
                 w[u][0] = *(const uint4 *)(wp + k0);
             }
@@ -705,11 +713,13 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
     }
     __syncthreads();
 
-    pf_f32x16 acc;
+    pf_f32x16 acc, accg;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    for (int i = 0; i < 16; ++i) { acc[i] = 0.0f; accg[i] = 0.0f; }
     for (int s0 = s_begin; s0 < s_end; s0 += PF_SK_UNROLL) {
         uint4 wc[PF_SK_UNROLL][2], xh[PF_SK_UNROLL][2], xl[PF_SK_UNROLL][2];
+        float gscale = 0.0f;
+        if (WT == WT_INT4) gscale = __uint_as_float((uint32_t)g.S[na * (size_t)(g.K / 128) + s0 / PF_SK_UNROLL] << 16);
 #pragma unroll
         for (int u = 0; u < PF_SK_UNROLL; ++u) { wc[u][0] = w[u][0]; wc[u][1] = w[u][1]; }
         if (s0 + PF_SK_UNROLL < s_end) wload(s0 + PF_SK_UNROLL);   // next group in flight while this one multiplies
@@ -724,7 +734,20 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
             if (s0 + u < s_end) {
                 uint4 b0, b1;
                 if (WT == WT_BF16) { b0 = wc[u][0]; b1 = wc[u][1]; }
-                else {
+                else if (WT == WT_INT4) {
+                    // nibble n (offset-binary, element 2j = low nibble of byte j) -> bf16 bits of the integer n - 8
+                    const uint32_t q[2] = {wc[u][0].x, wc[u][0].y};
+                    uint32_t o[8];
+#pragma unroll
+                    for (int i = 0; i < 2; ++i)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float f0 = __uint_as_float(0x4B000000u | ((q[i] >> (8 * e)) & 0xfu)) - 8388616.0f;
+                            const float f1 = __uint_as_float(0x4B000000u | ((q[i] >> (8 * e + 4)) & 0xfu)) - 8388616.0f;
+                            o[4 * i + e] = (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xffff0000u);
+                        }
+                    b0 = make_uint4(o[0], o[1], o[2], o[3]); b1 = make_uint4(o[4], o[5], o[6], o[7]);
+                } else {
                     const uint32_t q[4] = {wc[u][0].x, wc[u][0].y, wc[u][0].z, wc[u][0].w};
                     uint32_t o[8];
 #pragma unroll
@@ -737,11 +760,16 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
                     b0 = make_uint4(o[0], o[1], o[2], o[3]); b1 = make_uint4(o[4], o[5], o[6], o[7]);
                 }
                 const pf_bf16x8 B0 = __builtin_bit_cast(pf_bf16x8, b0), B1 = __builtin_bit_cast(pf_bf16x8, b1);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xh[u][0]), B0, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xl[u][0]), B0, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xh[u][1]), B1, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xl[u][1]), B1, acc, 0, 0, 0);
+                pf_f32x16 &t = WT == WT_INT4 ? accg : acc;
+                t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xh[u][0]), B0, t, 0, 0, 0);
+                t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xl[u][0]), B0, t, 0, 0, 0);
+                t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xh[u][1]), B1, t, 0, 0, 0);
+                t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xl[u][1]), B1, t, 0, 0, 0);
             }
+        }
+        if (WT == WT_INT4) {       // result columns are weight rows (lane % 32): one scale per lane and group
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { acc[i] = fmaf(accg[i], gscale, acc[i]); accg[i] = 0.0f; }
         }
     }
 #pragma unroll

@@ -58,6 +58,24 @@ def test_batched_logits_rows_match_sequential_oracles(rows, n_prompt):
     assert rel_err(dev.decode_logits_from_id(5), fresh.decode_logits_from_id(5)) < 1e-4
 
 
+@pytest.mark.parametrize("rows", [5, 32])
+def test_batched_4bit_weights_are_fp32_grade(rows):
+    # 4-bit weights enter the few-row GEMM as exact integers and are scaled per 128-element group in fp32,
+    # so every row is fp32-grade against the oracle run on the de-quantised weights.  3 and 9 scale groups
+    # per weight row: the K splits and the four waves of a workgroup get uneven numbers of groups.
+    cfg = Config.make(dim=384, hidden=1152, heads=3, hd=128, seq=64, nlayers=2, vocab=640)
+    w, dev, orcs, ids = setup(cfg, rows, 12, wdt=WeightDtype.INT4_G128, std=0.05)
+    dev.batch_begin(rows)
+    toks = np.array([(11 * r + 3) % cfg.vocab for r in range(rows)], np.uint32)
+    for step in range(4):
+        got = dev.decode_logits_from_ids_batch(toks)
+        want = np.stack([orcs[r].decode_logits_from_id(int(toks[r])) for r in range(rows)])
+        for r in range(rows):
+            assert rel_err(got[r], want[r]) < 1e-4, (step, r)
+        toks = np.array([np.argsort(-want[r], kind="stable")[r % 3] for r in range(rows)], np.uint32)
+    dev.batch_end()
+
+
 def test_batched_head_variants_match_oracle():
     cfg = Config.make(dim=256, hidden=384, heads=4, hd=64, seq=64, nlayers=2, vocab=600, kv_heads=2)
     rows = 4
