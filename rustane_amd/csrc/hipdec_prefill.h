@@ -791,73 +791,109 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
 // One workgroup of PF_ATT_WAVES waves per (32 query rows, head); wave w takes the key tiles w,
 // w + PF_ATT_WAVES, ... with its own running maximum, sum and output tile, and the partial results
 // are merged through LDS at the end (a single wave walking up to T/32 tiles one after the other is
-// the critical path of the whole kernel under the causal mask).  S^T = K . Q^T on the fp32 MFMA (32x32x2: lane l supplies
-// row l % 32 and reduction element l / 32 of both operands), so lane (q = l % 32, g = l / 32) ends
-// up with the scores of query q against keys 8 * (i / 4) + 4 * g + i % 4, i = 0..15 -- exactly the
-// operand layout P needs in O += P . V.  Softmax statistics are per lane (+ one exchange with lane
-// l ^ 32); the rescale factors of the O rows travel through LDS.
+// the critical path of the whole kernel under the causal mask).  S^T = K . Q^T, so lane
+// (q = l % 32, g = l / 32) ends up with the scores of query q against keys 8 * (i / 4) + 4 * g + i % 4,
+// i = 0..15 -- exactly the operand layout P needs in O += P . V.  Softmax statistics are per lane (+ one
+// exchange with lane l ^ 32); the rescale factors of the O rows travel through LDS, and only in the
+// tiles where some row's maximum grew; the causal mask is applied only in tiles that reach past the
+// block's first query.  Scores carry a factor log2(e), so the exponentials are bare v_exp_f32.
+// fp32 cache: both products on the fp32 MFMA (32x32x2: lane l supplies row l % 32 and reduction element
+// l / 32 of both operands).  bf16 cache: both on the bf16 MFMA (32x32x16) -- keys and values are bf16
+// numbers already; the scaled query rows and the probabilities enter as (hi, lo) bf16 pairs, like the
+// activations of the GEMMs, so nothing is rounded to 8 bits.  The query pair tile is shared by the
+// four waves and lives in LDS (chunks of a row permuted by the row index, so that 16 rows' reads of
+// one chunk spread over all banks); in registers it cost 64 per lane and the loop spilled.
 // (kernels/sdpa_fwd.rs:325-354: softmax(q . k^T / sqrt(hd) + causal mask) . v)
 #define PF_ATT_WAVES 4
+typedef __bf16 pf_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float pf_f32x2 __attribute__((ext_vector_type(2)));
+// two floats as packed bf16 (round to nearest even, in hardware), and as a (hi, lo) pair of such words
+__device__ __forceinline__ uint32_t pf_pack_bf16(float a, float b) {
+    const pf_f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, pf_bf16x2));
+}
+__device__ __forceinline__ void pf_split2(float a, float b, uint32_t &hi, uint32_t &lo) {
+    hi = pf_pack_bf16(a, b);
+    lo = pf_pack_bf16(a - __uint_as_float(hi << 16), b - __uint_as_float(hi & 0xffff0000u));
+}
 template <int KVBF16, int HD>
-__global__ __launch_bounds__(64 * PF_ATT_WAVES) void k_pf_attn(const float *__restrict__ q, const void *__restrict__ kc,
+__global__ __launch_bounds__(64 * PF_ATT_WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_pf_attn(const float *__restrict__ q, const void *__restrict__ kc,
                                                 const void *__restrict__ vc, uint16_t *__restrict__ ohi,
                                                 uint16_t *__restrict__ olo, int T, int Q, int KV, int gqa, int pos0,
                                                 int seq, float scale, int f16) {
     constexpr int HK = HD / 2;                 // reduction elements per lane group in S
     constexpr int NT = HD / 32;                // 32-wide column tiles of O
-    constexpr int VS = HD + 8;                 // LDS row stride of the V tile (floats)
+    constexpr int VS = HD + 8;                 // LDS row stride of the fp32 V tile (floats)
+    constexpr int VSB = HD + 16;               // bf16 V tile: elements per LDS row (rows 4 apart fall 32 banks apart)
     constexpr int KESZ = KVBF16 ? 2 : 4;
     constexpr int CPR = HD * KESZ / 16;        // 16-byte chunks per cache row
     constexpr int KCH = HK * KESZ / 16;        // chunks of this lane's half row
     constexpr int VCH = 32 * CPR / 64;         // V-tile chunks per lane
-    __shared__ __align__(16) float sVw[PF_ATT_WAVES][32 * VS];
-    __shared__ __align__(16) float sfacw[PF_ATT_WAVES][32];
+    constexpr int QCH = HD / 8;                // 16-byte chunks of a bf16 query row
+    // LDS.  fp32 cache: a V tile per wave, which also takes the wave's output tile for the merge.  bf16 cache:
+    // the query pair tile and a V tile per wave; the merge (two output tiles at a time) reuses that space.
+    constexpr int Q_BYTES = 2 * 32 * HD * 2, VB_BYTES = 32 * VSB * 2, MERGE_BYTES = 2 * 16 * NT * 64 * 4;
+    constexpr int LOOP_BYTES = Q_BYTES + PF_ATT_WAVES * VB_BYTES;
+    constexpr int LDS_BYTES = KVBF16 ? (LOOP_BYTES > MERGE_BYTES ? LOOP_BYTES : MERGE_BYTES) : PF_ATT_WAVES * 32 * VS * 4;
+    __shared__ __align__(16) char smem[LDS_BYTES];
+    __shared__ __align__(16) float sfacw[PF_ATT_WAVES][32], sfow[PF_ATT_WAVES][32];
     __shared__ float s_m[PF_ATT_WAVES][32], s_l[PF_ATT_WAVES][32];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, g = lane >> 5;
-    float *sV = sVw[wave], *sfac = sfacw[wave];
+    float *sV = (float *)smem + wave * 32 * VS, *sfac = sfacw[wave];
+    uint16_t *sQh = (uint16_t *)smem, *sQl = sQh + 32 * HD;
+    uint16_t *sVb = (uint16_t *)(smem + (KVBF16 ? Q_BYTES + wave * VB_BYTES : 0));
     // LDS traffic inside the key loop stays within one wave (its own tile and factors): program order
-    // is enough for the hardware, the fence keeps the compiler from reordering across it
+    // is enough for the hardware, the fence keeps the compiler from reordering LDS accesses across it
+    // (a fence over every address space also made it write the loaded V chunks to scratch and back)
     auto wave_sync = [&]() {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
         __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
     };
-    const int q0 = blockIdx.x * 32, h = blockIdx.y, kvh = h / gqa;
+    // Which (query block, head) this workgroup takes.  Workgroups are dealt to the 8 XCDs round-robin by their
+    // linear index, and each XCD has its own L2: with whole heads per XCD (heads a multiple of 8) a head's keys
+    // and values are fetched into one L2 instead of all eight, and within an XCD the query blocks run from
+    // the last (most keys) to the first, so the long ones do not end up as the tail of the launch.
+    int qb = blockIdx.x, h = blockIdx.y;
+    if ((gridDim.y & 7) == 0) {
+        const int L = blockIdx.x + gridDim.x * blockIdx.y, xcd = L & 7, j = L >> 3;
+        h = xcd * (gridDim.y >> 3) + j / gridDim.x;
+        qb = gridDim.x - 1 - j % gridDim.x;
+    }
+    const int q0 = qb * 32, kvh = h / gqa;
     const int tq = min(q0 + r, T - 1);
     const int qpos = pos0 + q0 + r;            // position of this lane's query row
+    const float sc2 = scale * 1.44269504088896341f;
 
-    float qf[HK];
-    {
+    float qf[KVBF16 ? 1 : HK];
+    int qoff[KVBF16 ? KCH : 1];                // element offsets of this lane's operand chunks inside its query row
+    if constexpr (KVBF16 != 0) {
+        // this lane's half of the query row in operand chunks of 8 elements; the four waves share the work
+        const int rx = r & (QCH - 1);
+#pragma unroll
+        for (int c = 0; c < KCH; ++c) qoff[c] = r * HD + (((g * KCH + c) ^ rx) << 3);
+        for (int c = wave; c < KCH; c += PF_ATT_WAVES) {
+            const float *qp = q + (size_t)tq * Q + h * HD + HK * g + 8 * c;
+            const float4 a = *(const float4 *)qp, b = *(const float4 *)(qp + 4);
+            uint32_t wh[4], wl[4];
+            pf_split2(a.x * sc2, a.y * sc2, wh[0], wl[0]);
+            pf_split2(a.z * sc2, a.w * sc2, wh[1], wl[1]);
+            pf_split2(b.x * sc2, b.y * sc2, wh[2], wl[2]);
+            pf_split2(b.z * sc2, b.w * sc2, wh[3], wl[3]);
+            const int o = r * HD + (((g * KCH + c) ^ rx) << 3);
+            *(uint4 *)(sQh + o) = make_uint4(wh[0], wh[1], wh[2], wh[3]);
+            *(uint4 *)(sQl + o) = make_uint4(wl[0], wl[1], wl[2], wl[3]);
+        }
+        __syncthreads();
+    } else {
         const float *qp = q + (size_t)tq * Q + h * HD + HK * g;
 #pragma unroll
         for (int s = 0; s < HK; s += 4) {
             const float4 v = *(const float4 *)(qp + s);
-            qf[s] = v.x * scale; qf[s + 1] = v.y * scale; qf[s + 2] = v.z * scale; qf[s + 3] = v.w * scale;
+            qf[KVBF16 ? 0 : s] = v.x * sc2; qf[KVBF16 ? 0 : s + 1] = v.y * sc2;
+            qf[KVBF16 ? 0 : s + 2] = v.z * sc2; qf[KVBF16 ? 0 : s + 3] = v.w * sc2;
         }
     }
-    // bf16 cache: both products run on the bf16 matrix instruction (32x32x16), eight times the rate of the
-    // fp32 one.  Keys and values are bf16 numbers already; the scaled query row and the probabilities
-    // enter as (hi, lo) bf16 pairs, like the activations of the GEMMs, so nothing is rounded to 8 bits.
-    // This lane's half of the query row, in operand chunks of 8 elements:
-    uint4 qh[KVBF16 ? KCH : 1], ql[KVBF16 ? KCH : 1];
-    if constexpr (KVBF16 != 0) {
-#pragma unroll
-        for (int c = 0; c < KCH; ++c) {
-            uint32_t wh[4], wl[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                uint16_t h0, l0, h1, l1;
-                pf_split(qf[8 * c + 2 * e], h0, l0);
-                pf_split(qf[8 * c + 2 * e + 1], h1, l1);
-                wh[e] = (uint32_t)h0 | ((uint32_t)h1 << 16);
-                wl[e] = (uint32_t)l0 | ((uint32_t)l1 << 16);
-            }
-            qh[KVBF16 ? c : 0] = make_uint4(wh[0], wh[1], wh[2], wh[3]);
-            ql[KVBF16 ? c : 0] = make_uint4(wl[0], wl[1], wl[2], wl[3]);
-        }
-    }
-    constexpr int VSB = HD + 16;               // bf16 V tile: elements per LDS row (rows 4 apart fall 32 banks apart)
-    uint16_t *sVb = (uint16_t *)sV;            // (the bf16 tile shares the wave's fp32 tile, which the key loop then does not use)
     pf_f32x16 accO[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
@@ -870,6 +906,7 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void k_pf_attn(const float *__re
     const char *vbase = (const char *)vc + (size_t)kvh * HD * KESZ;
     const size_t rowb = (size_t)KV * KESZ;
     for (int kt0 = 32 * wave; kt0 <= last_pos; kt0 += 32 * PF_ATT_WAVES) {
+        wave_sync();                           // the previous tile's reads of the V tile are done
         // this lane's key row (its half of the head dimension) and its share of the V tile
         uint4 kr[KCH], vr[VCH];
         {
@@ -883,28 +920,8 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void k_pf_attn(const float *__re
                 vr[c] = *(const uint4 *)(vbase + (size_t)vrow * rowb + cc * 16);
             }
         }
-        pf_f32x16 accS;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) accS[i] = 0.0f;
-        if constexpr (KVBF16 != 0) {
-            // chunk c of this lane's half key row is an operand as it is: reduction slot (g, e) of step c
-            // is element g * HK + 8 c + e of the head dimension for the key and for the query alike
-#pragma unroll
-            for (int c = 0; c < KCH; ++c) {
-                accS = pf_mma(kr[c], qh[KVBF16 ? c : 0], accS, false);
-                accS = pf_mma(kr[c], ql[KVBF16 ? c : 0], accS, false);
-            }
-        } else {
-#pragma unroll
-            for (int c = 0; c < KCH; ++c) {
-                float kf[16 / KESZ];
-                WS<KVBF16 ? WT_BF16 : WT_F32>::decode(kr[c], kf);
-#pragma unroll
-                for (int e = 0; e < 16 / KESZ; ++e)
-                    accS = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[c * (16 / KESZ) + e], accS, 0, 0, 0);
-            }
-        }
-        wave_sync();                           // the previous tile's V reads are done
+        // the V tile goes to LDS first, so that its registers are free during the products (and no fence
+        // stands between its loads and its stores: across one the compiler parks the chunks in scratch)
         if constexpr (KVBF16 != 0) {
 #pragma unroll
             for (int c = 0; c < VCH; ++c) {
@@ -922,37 +939,73 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void k_pf_attn(const float *__re
                 for (int e = 0; e < 16 / KESZ; e += 4) *(float4 *)(dst + e) = make_float4(vf[e], vf[e + 1], vf[e + 2], vf[e + 3]);
             }
         }
-        // online softmax for query row r over this tile's 32 keys (16 here, 16 in lane r ^ 32)
-        float tmax = -1e30f;
-        bool valid[16];
+        pf_f32x16 accS;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int kpos = kt0 + 8 * (i >> 2) + 4 * g + (i & 3);
-            valid[i] = kpos <= qpos;
-            if (valid[i]) tmax = fmaxf(tmax, accS[i]);
+        for (int i = 0; i < 16; ++i) accS[i] = 0.0f;
+        if constexpr (KVBF16 != 0) {
+            // chunk c of this lane's half key row is an operand as it is: reduction slot (g, e) of step c
+            // is element g * HK + 8 c + e of the head dimension for the key and for the query alike
+#pragma unroll
+            for (int c = 0; c < KCH; ++c) {
+                const uint4 qh = *(const uint4 *)(sQh + qoff[KVBF16 ? c : 0]), ql = *(const uint4 *)(sQl + qoff[KVBF16 ? c : 0]);
+                accS = pf_mma(kr[c], qh, accS, false);
+                accS = pf_mma(kr[c], ql, accS, false);
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < KCH; ++c) {
+                float kf[16 / KESZ];
+                WS<KVBF16 ? WT_BF16 : WT_F32>::decode(kr[c], kf);
+#pragma unroll
+                for (int e = 0; e < 16 / KESZ; ++e)
+                    accS = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[e], qf[KVBF16 ? 0 : c * (16 / KESZ) + e], accS, 0, 0, 0);
+            }
+        }
+        // online softmax for query row r over this tile's 32 keys (16 here, 16 in lane r ^ 32); a tile that
+        // ends at or before the block's first query needs no mask
+        const bool full = kt0 + 31 <= pos0 + q0;
+        float tmax = -1e30f;
+        if (full) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, accS[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                if (kt0 + 8 * (i >> 2) + 4 * g + (i & 3) <= qpos) tmax = fmaxf(tmax, accS[i]);
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
         const float m_new = fmaxf(m_run, tmax);
-        const float corr = __expf(m_run - m_new);
+        const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
+        const bool grew = __any(m_new > m_run) != 0;      // some row of this wave moved its maximum: the O rows need rescaling
         float psum = 0.0f;
         float p[16];
+        if (full) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            p[i] = valid[i] ? __expf(accS[i] - m_new) : 0.0f;
-            psum += p[i];
+            for (int i = 0; i < 16; ++i) {
+                p[i] = __builtin_amdgcn_exp2f(accS[i] - m_new);
+                psum += p[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                p[i] = kt0 + 8 * (i >> 2) + 4 * g + (i & 3) <= qpos ? __builtin_amdgcn_exp2f(accS[i] - m_new) : 0.0f;
+                psum += p[i];
+            }
         }
         psum += __shfl_xor(psum, 32, 64);
         l_run = l_run * corr + psum;
         m_run = m_new;
-        if (g == 0) sfac[r] = corr;
+        if (grew && g == 0) sfac[r] = corr;
         wave_sync();                           // V tile and rescale factors are in LDS
+        if (grew) {
 #pragma unroll
-        for (int j4 = 0; j4 < 4; ++j4) {
-            const float4 f = *(const float4 *)(sfac + 8 * j4 + 4 * g);
+            for (int j4 = 0; j4 < 4; ++j4) {
+                const float4 f = *(const float4 *)(sfac + 8 * j4 + 4 * g);
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                accO[nt][4 * j4] *= f.x; accO[nt][4 * j4 + 1] *= f.y;
-                accO[nt][4 * j4 + 2] *= f.z; accO[nt][4 * j4 + 3] *= f.w;
+                for (int nt = 0; nt < NT; ++nt) {
+                    accO[nt][4 * j4] *= f.x; accO[nt][4 * j4 + 1] *= f.y;
+                    accO[nt][4 * j4 + 2] *= f.z; accO[nt][4 * j4 + 3] *= f.w;
+                }
             }
         }
         if constexpr (KVBF16 != 0) {
@@ -962,13 +1015,7 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void k_pf_attn(const float *__re
             for (int t = 0; t < 2; ++t) {
                 uint32_t ph[4], pl[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    uint16_t h0, l0, h1, l1;
-                    pf_split(p[8 * t + 2 * e], h0, l0);
-                    pf_split(p[8 * t + 2 * e + 1], h1, l1);
-                    ph[e] = (uint32_t)h0 | ((uint32_t)h1 << 16);
-                    pl[e] = (uint32_t)l0 | ((uint32_t)l1 << 16);
-                }
+                for (int e = 0; e < 4; ++e) pf_split2(p[8 * t + 2 * e], p[8 * t + 2 * e + 1], ph[e], pl[e]);
                 const uint4 Ph = make_uint4(ph[0], ph[1], ph[2], ph[3]), Pl = make_uint4(pl[0], pl[1], pl[2], pl[3]);
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
@@ -993,31 +1040,87 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void k_pf_attn(const float *__re
             }
         }
     }
-    // merge the waves' partial results: O = sum_w e_w O_w / sum_w e_w l_w with e_w = exp(m_w - max m)
-    wave_sync();
+    // merge the waves' partial results: O = sum_w e_w O_w / sum_w e_w l_w with e_w = 2^(m_w - max m)
+    if constexpr (KVBF16 != 0) {
+        // in registers, as a tree: waves 2 and 3 hand their tiles to waves 0 and 1, then wave 1 to wave 0 (every
+        // wave holds its tile in the same layout, so a tile crosses LDS lane by lane)
+        __syncthreads();                       // every wave is done with the query tile and its own V tile
+        float *mb = (float *)smem;
+        auto put = [&](int slot) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int qi = 8 * (i >> 2) + 4 * g + (i & 3);
+            for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) sV[qi * VS + 32 * nt + r] = accO[nt][i];
-    }
-    if (g == 0) { s_m[wave][r] = m_run; s_l[wave][r] = l_run; }
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < 32 * HD; idx += 64 * PF_ATT_WAVES) {
-        const int qi = idx / HD, d = idx - qi * HD, t = q0 + qi;
-        float M = -1e30f;
+                for (int i = 0; i < 16; ++i) mb[((slot * NT + nt) * 16 + i) * 64 + lane] = accO[nt][i];
+            if (g == 0) { s_m[wave][r] = m_run; s_l[wave][r] = l_run; }
+        };
+        auto take = [&](int slot, int other) {
+            const float mo = s_m[other][r], lo = s_l[other][r];
+            const float M = fmaxf(m_run, mo);
+            const float fs = __builtin_amdgcn_exp2f(m_run - M), fo = __builtin_amdgcn_exp2f(mo - M);
+            l_run = fs * l_run + fo * lo;
+            m_run = M;
+            if (g == 0) { sfacw[wave][r] = fs; sfow[wave][r] = fo; }
+            wave_sync();
 #pragma unroll
-        for (int w = 0; w < PF_ATT_WAVES; ++w) M = fmaxf(M, s_m[w][qi]);
-        float num = 0.0f, den = 0.0f;
+            for (int i = 0; i < 16; ++i) {
+                const int qi = 8 * (i >> 2) + 4 * g + (i & 3);
+                const float a = sfacw[wave][qi], b = sfow[wave][qi];
 #pragma unroll
-        for (int w = 0; w < PF_ATT_WAVES; ++w) {
-            const float e = __expf(s_m[w][qi] - M);
-            den += e * s_l[w][qi];
-            num += e * sVw[w][qi * VS + d];
+                for (int nt = 0; nt < NT; ++nt)
+                    accO[nt][i] = accO[nt][i] * a + mb[((slot * NT + nt) * 16 + i) * 64 + lane] * b;
+            }
+            wave_sync();                       // the factors are read before the next merge overwrites them
+        };
+        if (wave >= 2) put(wave - 2);
+        __syncthreads();
+        if (wave < 2) take(wave, wave + 2);
+        __syncthreads();
+        if (wave == 1) put(0);
+        __syncthreads();
+        if (wave == 0) {
+            take(0, 1);
+            if (g == 0) sfacw[0][r] = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+            wave_sync();
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int qi = 8 * (i >> 2) + 4 * g + (i & 3), t = q0 + qi;
+                const float inv = sfacw[0][qi];
+                if (t < T) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        const size_t o = (size_t)t * Q + h * HD + 32 * nt + r;
+                        pf_split(accO[nt][i] * inv, ohi[o], olo[o], f16);
+                    }
+                }
+            }
         }
-        if (t < T) {
-            const size_t o = (size_t)t * Q + h * HD + d;
-            pf_split(den > 0.0f ? num / den : 0.0f, ohi[o], olo[o], f16);
+    } else {
+        wave_sync();
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int qi = 8 * (i >> 2) + 4 * g + (i & 3);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) sV[qi * VS + 32 * nt + r] = accO[nt][i];
+        }
+        if (g == 0) { s_m[wave][r] = m_run; s_l[wave][r] = l_run; }
+        __syncthreads();
+        const float *sVall = (const float *)smem;
+        for (int idx = threadIdx.x; idx < 32 * HD; idx += 64 * PF_ATT_WAVES) {
+            const int qi = idx / HD, d = idx - qi * HD, t = q0 + qi;
+            float M = -1e30f;
+#pragma unroll
+            for (int w = 0; w < PF_ATT_WAVES; ++w) M = fmaxf(M, s_m[w][qi]);
+            float num = 0.0f, den = 0.0f;
+#pragma unroll
+            for (int w = 0; w < PF_ATT_WAVES; ++w) {
+                const float e = __builtin_amdgcn_exp2f(s_m[w][qi] - M);
+                den += e * s_l[w][qi];
+                num += e * sVall[w * 32 * VS + qi * VS + d];
+            }
+            if (t < T) {
+                const size_t o = (size_t)t * Q + h * HD + d;
+                pf_split(den > 0.0f ? num / den : 0.0f, ohi[o], olo[o], f16);
+            }
         }
     }
 }
