@@ -102,8 +102,12 @@ struct Reader {
         if (*end) return fail("malformed number");
         return true;
     }
-    // skips any value (fields the protocol does not know)
+    // skips any value (fields the protocol does not know); nesting is bounded, so that a request made of
+    // brackets cannot run the stack out
+    int depth = 0;
     bool skip() {
+        struct Level { int &d; explicit Level(int &x) : d(x) { ++d; } ~Level() { --d; } } level(depth);
+        if (depth > 128) return fail("value nested too deeply");
         ws();
         if (i >= s.size()) return fail("unexpected end of input");
         std::string tmp;

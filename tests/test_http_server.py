@@ -92,6 +92,10 @@ def test_completion_rejections():
                  '{"prompt_ids":[1]} x', '{"stream":"yes","prompt_ids":[1]}', '{"prompt_ids":{"a":1}}', '[1]'):
         m, invalid = msg(body)
         assert invalid and m.startswith("invalid JSON: "), body
+    m, invalid = msg('{"x":' + "[" * 100000 + "]" * 100000 + ',"prompt_ids":[1]}')      # (skipping an unknown field recurses)
+    assert invalid and "nested too deeply" in m
+    ids, _, _ = engine.http_prepare('{"x":' + "[" * 100 + "]" * 100 + ',"prompt_ids":[1]}')
+    assert ids.tolist() == [1]
     assert msg('{"model":"other","prompt_ids":[1]}') == ("requested model other does not match loaded model rustane", False)
     assert msg('{"prompt":"a","prompt_ids":[1]}')[0] == "pass either prompt or prompt_ids, not both"
     assert msg('{}')[0] == "one of prompt or prompt_ids is required"
