@@ -664,16 +664,16 @@ void pf_launch_resid(hipdec_model *m, int T, int splits, const void *wscale, con
                      const float *gamma, int f16 = 0) {
     PrefillWork &w = m->pf;
     const int D = (int)m->cfg.dim;
-    dim3 grid((D + PF_CHUNK - 1) / PF_CHUNK, T), block(PF_CHUNK);
+    const int nch = (D + PF_CHUNK - 1) / PF_CHUNK;
+    dim3 grid((nch + 3) / 4, T), block(256);
     hipLaunchKernelGGL(k_pf_resid, grid, block, 0, m->stream, w.P, splits, (size_t)T * D,
                        m->wt == WT_FP8 ? (const float *)wscale : nullptr, resid, m->alpha, out, gamma, w.xn_hi, w.xn_lo,
-                       w.ssq, D, f16);
+                       w.ssq, D, nch, f16);
 }
 void pf_launch_gate(hipdec_model *m, int T, int splits, const void *wscale, int f16 = 0) {
     PrefillWork &w = m->pf;
     const int D = (int)m->cfg.dim, H = (int)m->cfg.hidden;
-    const size_t items = (size_t)T * (H / 4);
-    hipLaunchKernelGGL(k_pf_gate_epi, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, m->stream, w.P, splits,
+    hipLaunchKernelGGL(k_pf_gate_epi, dim3((unsigned)((H / 4 + 255) / 256), (unsigned)T), dim3(256), 0, m->stream, w.P, splits,
                        (size_t)T * 2 * H, m->wt == WT_FP8 ? (const float *)wscale : nullptr, w.gate_hi, w.gate_lo, w.ssq,
                        (D + PF_CHUNK - 1) / PF_CHUNK, D, T, H, (int)m->opt.ffn_activation, f16);
 }
@@ -709,8 +709,7 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
             int N = Q + 2 * KV;
             int sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.wqkv, L.s_qkv, T, N, D, act);
             {
-                const size_t items = (size_t)T * (N / 4);
-                dim3 grid((unsigned)((items + 255) / 256)), block(256);
+                dim3 grid((unsigned)((N / 4 + 255) / 256), (unsigned)T), block(256);
                 if (m->kvbf16)
                     hipLaunchKernelGGL(k_pf_qkv_epi<1>, grid, block, 0, m->stream, w.P, sp, (size_t)T * N,
                                        fp8 ? (const float *)L.s_qkv : nullptr, w.q, L.kc, L.vc, m->rope_cos, m->rope_sin,

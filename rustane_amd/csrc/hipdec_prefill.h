@@ -67,6 +67,14 @@ __device__ __forceinline__ float pf_row_inv(const float *__restrict__ ssq, int t
     return 1.0f / sqrtf(s * (1.0f / (float)D) + 1e-5f);
 }
 
+// The same for a workgroup whose threads all work on row t: one lane of each wave adds up the row's sums and
+// hands the factor to the others, instead of every thread reading all of them.
+__device__ __forceinline__ float pf_row_inv_wave(const float *__restrict__ ssq, int t, int nch, int D) {
+    float mine = 0.0f;
+    if ((threadIdx.x & 63) == 0) mine = pf_row_inv(ssq, t, nch, D);
+    return __shfl(mine, 0, 64);
+}
+
 // x[t] = embed[ids[t]] (cpu/embedding.rs:8-16); hi/lo = x * gamma1 of the first layer; chunk sums of squares.
 // grid (chunks, rows)
 template <int EWT>
@@ -89,24 +97,41 @@ __global__ __launch_bounds__(PF_CHUNK) void k_pf_embed(const void *__restrict__ 
 
 // out[t][d] = resid[t][d] + alpha * scale[d] * sum_z P[z][t][d]   (layer.rs:1397-1405, :1300);
 // hi/lo = out * gamma for the next GEMM (gamma == nullptr: none); chunk sums of squares.  grid (chunks, rows)
-__global__ __launch_bounds__(PF_CHUNK) void k_pf_resid(const float *__restrict__ P, int splits, size_t plane,
-                                                       const float *__restrict__ wscale, const float *__restrict__ resid,
-                                                       float alpha, float *__restrict__ out, const float *__restrict__ gamma,
-                                                       uint16_t *__restrict__ hi, uint16_t *__restrict__ lo,
-                                                       float *__restrict__ ssq, int D, int f16) {
-    __shared__ float red[8];
-    const int t = blockIdx.y, d = blockIdx.x * PF_CHUNK + threadIdx.x;
-    float v = 0.0f;
+__global__ __launch_bounds__(256) void k_pf_resid(const float *__restrict__ P, int splits, size_t plane,
+                                                 const float *__restrict__ wscale, const float *__restrict__ resid,
+                                                 float alpha, float *__restrict__ out, const float *__restrict__ gamma,
+                                                 uint16_t *__restrict__ hi, uint16_t *__restrict__ lo,
+                                                 float *__restrict__ ssq, int D, int nch, int f16) {
+    // a wave per 256-element chunk, four neighbouring elements per lane (D is a multiple of 4); grid (ceil(nch / 4), rows)
+    const int t = blockIdx.y, chunk = blockIdx.x * 4 + (threadIdx.x >> 6), d = chunk * PF_CHUNK + 4 * (threadIdx.x & 63);
+    if (chunk >= nch) return;
+    float ss = 0.0f;
     if (d < D) {
-        float s = 0.0f;
-        for (int z = 0; z < splits; ++z) s += P[z * plane + (size_t)t * D + d];
-        if (wscale) s *= wscale[d];
-        v = resid[(size_t)t * D + d] + alpha * s;
-        out[(size_t)t * D + d] = v;
-        if (gamma) pf_split(v * gamma[d], hi[(size_t)t * D + d], lo[(size_t)t * D + d], f16);
+        const size_t o = (size_t)t * D + d;
+        float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        for (int z = 0; z < splits; ++z) {
+            const float4 p = *(const float4 *)(P + z * plane + o);
+            s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
+        }
+        if (wscale) {
+            const float4 ws = *(const float4 *)(wscale + d);
+            s.x *= ws.x; s.y *= ws.y; s.z *= ws.z; s.w *= ws.w;
+        }
+        const float4 rs = *(const float4 *)(resid + o);
+        const float4 v = make_float4(rs.x + alpha * s.x, rs.y + alpha * s.y, rs.z + alpha * s.z, rs.w + alpha * s.w);
+        *(float4 *)(out + o) = v;
+        if (gamma) {
+            const float4 gm = *(const float4 *)(gamma + d);
+            uint16_t h0, l0, h1, l1, h2, l2, h3, l3;
+            pf_split(v.x * gm.x, h0, l0, f16); pf_split(v.y * gm.y, h1, l1, f16);
+            pf_split(v.z * gm.z, h2, l2, f16); pf_split(v.w * gm.w, h3, l3, f16);
+            *(uint2 *)(hi + o) = make_uint2((uint32_t)h0 | ((uint32_t)h1 << 16), (uint32_t)h2 | ((uint32_t)h3 << 16));
+            *(uint2 *)(lo + o) = make_uint2((uint32_t)l0 | ((uint32_t)l1 << 16), (uint32_t)l2 | ((uint32_t)l3 << 16));
+        }
+        ss = (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
     }
-    const float ss = pf_block_sum(v * v, red);
-    if (threadIdx.x == 0) ssq[t * gridDim.x + blockIdx.x] = ss;
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) ssq[t * nch + chunk] = ss;
 }
 
 // q/k/v rows of the chunk: sum the split planes, scale (8-bit weights), RoPE on interleaved pairs
@@ -120,10 +145,10 @@ __global__ __launch_bounds__(256) void k_pf_qkv_epi(const float *__restrict__ P,
                                                     const float *__restrict__ rope_cos, const float *__restrict__ rope_sin,
                                                     const float *__restrict__ ssq, int nch, int D,
                                                     int T, int Q, int KV, int hd, int pos0) {
-    const int N = Q + 2 * KV, nquads = N >> 2;
-    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (gid >= (size_t)T * nquads) return;
-    const int t = (int)(gid / nquads), row0 = 4 * (int)(gid - (size_t)t * nquads);
+    // grid (ceil(N / 4 / 256), rows): no division to find the row, and one row factor per workgroup
+    const int N = Q + 2 * KV, t = blockIdx.y, row0 = 4 * (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    const float inv = pf_row_inv_wave(ssq, t, nch, D);
+    if (row0 >= N) return;
     float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     for (int z = 0; z < splits; ++z) {
         const float4 v = *(const float4 *)(P + z * plane + (size_t)t * N + row0);
@@ -133,13 +158,12 @@ __global__ __launch_bounds__(256) void k_pf_qkv_epi(const float *__restrict__ P,
 #pragma unroll
         for (int e = 0; e < 4; ++e) s[e] *= wscale[row0 + e];
     }
-    const float inv = pf_row_inv(ssq, t, nch, D);
 #pragma unroll
     for (int e = 0; e < 4; ++e) s[e] *= inv;
     const int pos = pos0 + t;
     if (row0 < Q + KV) {
         const int rr = row0 < Q ? row0 : row0 - Q;
-        const int pi2 = (rr % hd) >> 1;
+        const int pi2 = (rr & (hd - 1)) >> 1;          // (hd is 64 or 128)
         const float2 c = *(const float2 *)(rope_cos + (size_t)pos * (hd / 2) + pi2);
         const float2 sn = *(const float2 *)(rope_sin + (size_t)pos * (hd / 2) + pi2);
         const float e0 = s[0] * c.x - s[1] * sn.x, o0 = s[1] * c.x + s[0] * sn.x;
@@ -170,10 +194,10 @@ __global__ __launch_bounds__(256) void k_pf_gate_epi(const float *__restrict__ P
                                                      const float *__restrict__ wscale, uint16_t *__restrict__ hi,
                                                      uint16_t *__restrict__ lo, const float *__restrict__ ssq, int nch,
                                                      int D, int T, int H, int act, int f16) {
-    const int hq = H >> 2;
-    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (gid >= (size_t)T * hq) return;
-    const int t = (int)(gid / hq), j = 4 * (int)(gid - (size_t)t * hq);
+    // grid (ceil(H / 4 / 256), rows)
+    const int t = blockIdx.y, j = 4 * (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    const float inv = pf_row_inv_wave(ssq, t, nch, D);
+    if (j >= H) return;
     float h[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     for (int z = 0; z < splits; ++z) {
         const float4 a = *(const float4 *)(P + z * plane + (size_t)t * 2 * H + 2 * j);
@@ -184,7 +208,6 @@ __global__ __launch_bounds__(256) void k_pf_gate_epi(const float *__restrict__ P
 #pragma unroll
         for (int e = 0; e < 8; ++e) h[e] *= wscale[2 * j + e];
     }
-    const float inv = pf_row_inv(ssq, t, nch, D);
     uint16_t oh[4], ol[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
