@@ -166,8 +166,8 @@ int hipdec_prefill(hipdec_model *m, const uint32_t *ids, size_t n, float softcap
  * every batched call returns what the single-row call of the same name would return for a model
  * that had decoded row r's tokens alone.  Between begin and end only the *_batch calls may be
  * used; hipdec_batch_end leaves len and the shared positions as they were.  1 <= n_rows <= 32;
- * needs bf16, e4m3 or 4-bit weights and model dimensions that are multiples of 32 (128 with
- * 4-bit weights); HIPDEC_ERR_UNSUPPORTED otherwise. */
+ * needs model dimensions that are multiples of 32 (128 with 4-bit weights);
+ * HIPDEC_ERR_UNSUPPORTED otherwise. */
 int hipdec_batch_begin(hipdec_model *m, size_t n_rows);
 int hipdec_batch_end(hipdec_model *m);
 /* steps taken since hipdec_batch_begin (each row is at position len + steps) */

@@ -515,7 +515,7 @@ bool prefill_batched_ok(const hipdec_model *m, size_t n) {
     const hipdec_config &c = m->cfg;
     if (m->opt.flags & HIPDEC_FLAG_PREFILL_STEPS) return false;
     if (n < (size_t)kPrefillMinRows) return false;
-    if (m->wt == WT_F32) return false;                               // fp32 weights: token steps
+    // (fp32 weights: chunks of at most kSkinnyRows rows, the one matrix-core GEMM that takes them)
     if (c.dim % PF_BK || c.q_dim % PF_BK || c.hidden % PF_BK) return false;
     if (m->wt == WT_INT4 && (c.dim % 128 || c.q_dim % 128 || c.hidden % 128)) return false;   // whole scale groups
     if (c.hd != 64 && c.hd != 128) return false;
@@ -631,7 +631,8 @@ int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, c
     if (T <= kSkinnyRows) {
         dim3 grid((N + 31) / 32, sp.splits), block(256);
         const size_t lds = (size_t)2 * T * (sp.steps_per_split * PF_BK + PF_SK_PAD) * 2;
-        if (wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_BF16>, grid, block, lds, m->stream, g);
+        if (wt == WT_F32) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_F32>, grid, block, lds, m->stream, g);
+        else if (wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_BF16>, grid, block, lds, m->stream, g);
         else if (wt == WT_FP8) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_FP8>, grid, block, lds, m->stream, g);
         else hipLaunchKernelGGL(k_pf_gemm_skinny<WT_INT4>, grid, block, lds, m->stream, g);
         return sp.splits;
@@ -688,7 +689,7 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
     const float scale = 1.0f / sqrtf((float)c.hd);
     size_t done = 0;
     while (done < n) {
-        const int T = (int)std::min<size_t>(n - done, kPrefillMaxRows);
+        const int T = (int)std::min<size_t>(n - done, m->wt == WT_F32 ? kSkinnyRows : kPrefillMaxRows);
         const int pos0 = (int)(m->len + done);
         int rc = pf_ensure(m, T);
         if (rc) return rc;
@@ -1618,7 +1619,7 @@ int hipdec_batch_begin(hipdec_model *m, size_t n_rows) {
     if (!m) return HIPDEC_ERR_ARG;
     if (n_rows == 0 || n_rows > (size_t)kBatchMaxRows) return fail(m, HIPDEC_ERR_ARG, "n_rows must be in 1..32");
     if (!prefill_batched_ok(m, kPrefillMinRows))
-        return fail(m, HIPDEC_ERR_UNSUPPORTED, "multi-row decode needs bf16, e4m3 or 4-bit weights and dimensions that are multiples of 32 (128 with 4-bit weights)");
+        return fail(m, HIPDEC_ERR_UNSUPPORTED, "multi-row decode needs dimensions that are multiples of 32 (128 with 4-bit weights) and a head dimension of 64 or 128");
     if (m->len >= m->cfg.seq) return fail(m, HIPDEC_ERR_FULL, "decode only supports lengths within cfg.seq");
     int rc = batch_alloc(m, (int)n_rows);
     if (rc) return rc;

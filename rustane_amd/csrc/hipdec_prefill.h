@@ -45,6 +45,18 @@ __device__ __forceinline__ void pf_split(float v, uint16_t &hi, uint16_t &lo, in
     lo = f32_to_bf16_rne(v - bf16_to_f32(hi));
 }
 
+typedef __bf16 pf_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float pf_f32x2 __attribute__((ext_vector_type(2)));
+// two floats as packed bf16 (round to nearest even, in hardware), and as a (hi, lo) pair of such words
+__device__ __forceinline__ uint32_t pf_pack_bf16(float a, float b) {
+    const pf_f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, pf_bf16x2));
+}
+__device__ __forceinline__ void pf_split2(float a, float b, uint32_t &hi, uint32_t &lo) {
+    hi = pf_pack_bf16(a, b);
+    lo = pf_pack_bf16(a - __uint_as_float(hi << 16), b - __uint_as_float(hi & 0xffff0000u));
+}
+
 __device__ __forceinline__ float pf_block_sum(float v, float *red) {
     v = wave_sum(v);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
@@ -685,6 +697,9 @@ __global__ __launch_bounds__(64 * WAVES, WGS) void k_pf_gemm_dl(PfGemm g) {
 // 4-bit weights: a lane's 16 elements of a step are 8 bytes; the PF_SK_UNROLL = 4 steps issued together are
 // exactly one scale group of 128 elements (the host makes every K split, and the kernel every wave's part,
 // a whole number of groups), whose products are summed unscaled and enter the result times the row's scale.
+// fp32 weights: a lane's 16 elements of a step are 64 bytes; each is split in registers into a (hi, lo) pair
+// of bf16 numbers like the activations, and x w = xh wh + xl wh + xh wl on the matrix cores (the dropped
+// xl wl and the weight's third part are 2^-16 of a product and less): fp32-grade, three instructions.
 #define PF_SK_UNROLL 4     // 32-element steps whose loads are issued together
 #define PF_SK_PAD 8        // bf16 elements of padding per staged activation row
 template <int WT>
@@ -703,16 +718,21 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
     const uint16_t *ah = s_act + min(r, g.T - 1) * astride + 16 * gq;
     const uint16_t *al = ah + g.T * astride;
     // bytes of a weight row, and of this lane's 16 elements of a step
-    const char *wp = (const char *)g.W + na * (WT == WT_BF16 ? (size_t)g.K * 2 : WT == WT_INT4 ? (size_t)g.K / 2 : (size_t)g.K) +
-                     (WT == WT_BF16 ? 32 : WT == WT_INT4 ? 8 : 16) * gq;
+    const char *wp = (const char *)g.W +
+                     na * (WT == WT_F32 ? (size_t)g.K * 4 : WT == WT_BF16 ? (size_t)g.K * 2 : WT == WT_INT4 ? (size_t)g.K / 2 : (size_t)g.K) +
+                     (WT == WT_F32 ? 64 : WT == WT_BF16 ? 32 : WT == WT_INT4 ? 8 : 16) * gq;
+    constexpr int WREG = WT == WT_F32 ? 4 : 2;             // 16-byte registers per step and lane
 
-    uint4 w[PF_SK_UNROLL][2];
+    uint4 w[PF_SK_UNROLL][WREG];
     auto wload = [&](int s0) {
 #pragma unroll
         for (int u = 0; u < PF_SK_UNROLL; ++u) {
             const int s = min(s0 + u, s_end - 1);             // a padded step re-reads the last one (and is skipped below)
             const size_t k0 = (size_t)s * PF_BK;
-            if (WT == WT_BF16) {
+            if (WT == WT_F32) {
+#pragma unroll
+                for (int c = 0; c < WREG; ++c) w[u][c] = *(const uint4 *)(wp + k0 * 4 + 16 * c);
+            } else if (WT == WT_BF16) {
                 w[u][0] = *(const uint4 *)(wp + k0 * 2);
                 w[u][1] = *(const uint4 *)(wp + k0 * 2 + 16);
             } else if (WT == WT_INT4) {
@@ -740,11 +760,13 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) { acc[i] = 0.0f; accg[i] = 0.0f; }
     for (int s0 = s_begin; s0 < s_end; s0 += PF_SK_UNROLL) {
-        uint4 wc[PF_SK_UNROLL][2], xh[PF_SK_UNROLL][2], xl[PF_SK_UNROLL][2];
+        uint4 wc[PF_SK_UNROLL][WREG], xh[PF_SK_UNROLL][2], xl[PF_SK_UNROLL][2];
         float gscale = 0.0f;
         if (WT == WT_INT4) gscale = __uint_as_float((uint32_t)g.S[na * (size_t)(g.K / 128) + s0 / PF_SK_UNROLL] << 16);
 #pragma unroll
-        for (int u = 0; u < PF_SK_UNROLL; ++u) { wc[u][0] = w[u][0]; wc[u][1] = w[u][1]; }
+        for (int u = 0; u < PF_SK_UNROLL; ++u)
+#pragma unroll
+            for (int c = 0; c < WREG; ++c) wc[u][c] = w[u][c];
         if (s0 + PF_SK_UNROLL < s_end) wload(s0 + PF_SK_UNROLL);   // next group in flight while this one multiplies
 #pragma unroll
         for (int u = 0; u < PF_SK_UNROLL; ++u) {
@@ -755,8 +777,18 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
 #pragma unroll
         for (int u = 0; u < PF_SK_UNROLL; ++u) {
             if (s0 + u < s_end) {
-                uint4 b0, b1;
-                if (WT == WT_BF16) { b0 = wc[u][0]; b1 = wc[u][1]; }
+                uint4 b0, b1, c0 = make_uint4(0u, 0u, 0u, 0u), c1 = c0;      // (c0, c1: the lo parts of fp32 weights)
+                if (WT == WT_F32) {
+                    uint32_t oh[8], ol[8];
+#pragma unroll
+                    for (int c = 0; c < WREG; ++c) {
+                        const uint4 v = wc[u][WT == WT_F32 ? c : 0];
+                        pf_split2(__uint_as_float(v.x), __uint_as_float(v.y), oh[2 * c], ol[2 * c]);
+                        pf_split2(__uint_as_float(v.z), __uint_as_float(v.w), oh[2 * c + 1], ol[2 * c + 1]);
+                    }
+                    b0 = make_uint4(oh[0], oh[1], oh[2], oh[3]); b1 = make_uint4(oh[4], oh[5], oh[6], oh[7]);
+                    c0 = make_uint4(ol[0], ol[1], ol[2], ol[3]); c1 = make_uint4(ol[4], ol[5], ol[6], ol[7]);
+                } else if (WT == WT_BF16) { b0 = wc[u][0]; b1 = wc[u][1]; }
                 else if (WT == WT_INT4) {
                     // nibble n (offset-binary, element 2j = low nibble of byte j) -> bf16 bits of the integer n - 8
                     const uint32_t q[2] = {wc[u][0].x, wc[u][0].y};
@@ -788,6 +820,10 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
                 t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xl[u][0]), B0, t, 0, 0, 0);
                 t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xh[u][1]), B1, t, 0, 0, 0);
                 t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xl[u][1]), B1, t, 0, 0, 0);
+                if (WT == WT_F32) {
+                    t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xh[u][0]), __builtin_bit_cast(pf_bf16x8, c0), t, 0, 0, 0);
+                    t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, xh[u][1]), __builtin_bit_cast(pf_bf16x8, c1), t, 0, 0, 0);
+                }
             }
         }
         if (WT == WT_INT4) {       // result columns are weight rows (lane % 32): one scale per lane and group
@@ -828,17 +864,6 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
 // one chunk spread over all banks); in registers it cost 64 per lane and the loop spilled.
 // (kernels/sdpa_fwd.rs:325-354: softmax(q . k^T / sqrt(hd) + causal mask) . v)
 #define PF_ATT_WAVES 4
-typedef __bf16 pf_bf16x2 __attribute__((ext_vector_type(2)));
-typedef float pf_f32x2 __attribute__((ext_vector_type(2)));
-// two floats as packed bf16 (round to nearest even, in hardware), and as a (hi, lo) pair of such words
-__device__ __forceinline__ uint32_t pf_pack_bf16(float a, float b) {
-    const pf_f32x2 v = {a, b};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, pf_bf16x2));
-}
-__device__ __forceinline__ void pf_split2(float a, float b, uint32_t &hi, uint32_t &lo) {
-    hi = pf_pack_bf16(a, b);
-    lo = pf_pack_bf16(a - __uint_as_float(hi << 16), b - __uint_as_float(hi & 0xffff0000u));
-}
 template <int KVBF16, int HD>
 __global__ __launch_bounds__(64 * PF_ATT_WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_pf_attn(const float *__restrict__ q, const void *__restrict__ kc,
                                                 const void *__restrict__ vc, uint16_t *__restrict__ ohi,

@@ -17,8 +17,8 @@ def rel_err(a, b):
     return float(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64)).max() / max(np.abs(b).max(), 1e-30))
 
 
-def setup(cfg, rows, n_prompt, wdt=WeightDtype.BF16, kvdt=KvDtype.F32, std=0.07, seed=17):
-    w = synth.make_weights(cfg, seed=seed, std=std, round_bf16=True)
+def setup(cfg, rows, n_prompt, wdt=WeightDtype.BF16, kvdt=KvDtype.F32, std=0.07, seed=17, round_bf16=True):
+    w = synth.make_weights(cfg, seed=seed, std=std, round_bf16=round_bf16)
     wo = w
     if wdt == WeightDtype.FP8_E4M3:
         wo = O.dequantised_weights(cfg, w, "fp8")[0]
@@ -56,6 +56,22 @@ def test_batched_logits_rows_match_sequential_oracles(rows, n_prompt):
     fresh = O.Oracle(cfg, w)
     fresh.forward_window(ids)
     assert rel_err(dev.decode_logits_from_id(5), fresh.decode_logits_from_id(5)) < 1e-4
+
+
+def test_batched_f32_weights():
+    # (the reference's own format: its samples run one after the other; here they step together like the others)
+    cfg = Config.make(dim=256, hidden=384, heads=4, hd=64, seq=64, nlayers=2, vocab=600, kv_heads=2)
+    rows = 6
+    w, dev, orcs, ids = setup(cfg, rows, 11, wdt=WeightDtype.F32, round_bf16=False)     # weights with all 24 bits in use
+    dev.batch_begin(rows)
+    toks = np.array([(13 * r + 2) % cfg.vocab for r in range(rows)], np.uint32)
+    for step in range(5):
+        got = dev.decode_logits_from_ids_batch(toks)
+        want = np.stack([orcs[r].decode_logits_from_id(int(toks[r])) for r in range(rows)])
+        for r in range(rows):
+            assert rel_err(got[r], want[r]) < 1e-4, (step, r)
+        toks = np.array([np.argsort(-want[r], kind="stable")[r % 3] for r in range(rows)], np.uint32)
+    dev.batch_end()
 
 
 @pytest.mark.parametrize("rows", [5, 32])
@@ -151,7 +167,9 @@ def test_batched_error_codes():
         dev.decode_token_argmax_from_ids_batch([1, 2])
     assert e.value.status == ERR_FULL                     # 10 + 2 == seq
     dev.batch_end()
-    f32 = HipDecodeModel(cfg, synth.make_weights(cfg, seed=2, std=0.05), weight_dtype=WeightDtype.F32)
+    # dimensions the few-row GEMM cannot tile (not multiples of 32): no multi-row step, the caller falls back
+    odd = Config.make(dim=144, hidden=208, heads=1, hd=128, seq=12, nlayers=1, vocab=64)
+    f32 = HipDecodeModel(odd, synth.make_weights(odd, seed=2, std=0.05), weight_dtype=WeightDtype.F32)
     with pytest.raises(HipDecodeError) as e:
         f32.batch_begin(2)
     assert e.value.status == ERR_UNSUPPORTED

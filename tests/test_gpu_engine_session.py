@@ -170,6 +170,20 @@ def test_samples_stepped_together_equal_sequential_samples(T, k, softcap):
     assert together.total_decode_elapsed > 0
 
 
+def test_f32_weight_samples_step_together_too():
+    cfg = tiny_cfg(vocab=1000)
+    prompt = [5, 6, 7, 8, 9, 10, 11, 12, 13]
+    w = synth.make_weights(cfg, seed=33, std=0.08, round_bf16=False)
+    req = E.GenerationRequest(E.DecodeBackendRequest.HIP, steps=8, temperature=0.8, top_k=8, samples=3, seed=4)
+    together = E.InferenceSession(cfg, w, prompt, weight_dtype=0).generate(req)
+    one_by_one = E.InferenceSession(cfg, w, prompt, weight_dtype=0, flags=0x100).generate(req)
+    want = oracle_streams(cfg, w, prompt, req, 0.0)
+    for a, b, (sampled, gen) in zip(together.results, one_by_one.results, want):
+        np.testing.assert_array_equal(a.sampled, b.sampled)
+        np.testing.assert_array_equal(a.sampled, sampled)
+        np.testing.assert_array_equal(a.generated, gen)
+
+
 def test_samples_stepped_together_after_a_suffix():
     cfg = tiny_cfg()
     w = synth.make_weights(cfg, seed=31, std=0.08, round_bf16=True)

@@ -20,8 +20,8 @@ def rel_err(a, b):
     return float(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64)).max() / max(np.abs(b).max(), 1e-30))
 
 
-def make(cfg, wdt=WeightDtype.BF16, kvdt=KvDtype.F32, std=0.06, seed=31, act=0, flags=0):
-    w = synth.make_weights(cfg, seed=seed, std=std, round_bf16=True)
+def make(cfg, wdt=WeightDtype.BF16, kvdt=KvDtype.F32, std=0.06, seed=31, act=0, flags=0, round_bf16=True):
+    w = synth.make_weights(cfg, seed=seed, std=std, round_bf16=round_bf16)
     wo = w
     if wdt == WeightDtype.FP8_E4M3:
         wo, _ = O.dequantised_weights(cfg, w, "fp8")
@@ -52,6 +52,14 @@ def check_prefill_then_decode(cfg, n_prompt, tol, n_decode=4, **kw):
 def test_prefill_bf16_weights_f32_cache(n_prompt):
     cfg = Config.make(dim=256, hidden=640, heads=2, hd=128, seq=160, nlayers=2, vocab=320)
     check_prefill_then_decode(cfg, n_prompt, 1e-4)
+
+
+@pytest.mark.parametrize("n_prompt", [8, 40, 97])
+def test_prefill_f32_weights(n_prompt):
+    # fp32 weights go through the few-row GEMM in chunks of 32 rows (40 = 32 + 8, 97 = 3 x 32 + 1 token step):
+    # every weight as a (hi, lo) pair of bf16 numbers, three matrix instructions per product
+    cfg = Config.make(dim=256, hidden=640, heads=2, hd=128, seq=160, nlayers=2, vocab=320)
+    check_prefill_then_decode(cfg, n_prompt, 1e-4, wdt=WeightDtype.F32, round_bf16=False)   # weights with all 24 bits in use
 
 
 def test_prefill_hd64_gqa_and_leaky_relu():
