@@ -79,12 +79,16 @@ __device__ __forceinline__ float pf_row_inv(const float *__restrict__ ssq, int t
     return 1.0f / sqrtf(s * (1.0f / (float)D) + 1e-5f);
 }
 
-// The same for a workgroup whose threads all work on row t: one lane of each wave adds up the row's sums and
-// hands the factor to the others, instead of every thread reading all of them.
-__device__ __forceinline__ float pf_row_inv_wave(const float *__restrict__ ssq, int t, int nch, int D) {
-    float mine = 0.0f;
-    if ((threadIdx.x & 63) == 0) mine = pf_row_inv(ssq, t, nch, D);
-    return __shfl(mine, 0, 64);
+// The same for a wave whose lanes all work on row t, in two halves: lane c requests chunk sum c (one load,
+// issued beside the kernel's own loads instead of nch dependent ones per thread), and once those have
+// come back the wave adds them up with shuffles.
+__device__ __forceinline__ float pf_row_part(const float *__restrict__ ssq, int t, int nch) {
+    float s = 0.0f;
+    for (int c = threadIdx.x & 63; c < nch; c += 64) s += ssq[t * nch + c];
+    return s;
+}
+__device__ __forceinline__ float pf_row_finish(float part, int D) {
+    return 1.0f / sqrtf(wave_sum(part) * (1.0f / (float)D) + 1e-5f);
 }
 
 // x[t] = embed[ids[t]] (cpu/embedding.rs:8-16); hi/lo = x * gamma1 of the first layer; chunk sums of squares.
@@ -159,13 +163,16 @@ __global__ __launch_bounds__(256) void k_pf_qkv_epi(const float *__restrict__ P,
                                                     int T, int Q, int KV, int hd, int pos0) {
     // grid (ceil(N / 4 / 256), rows): no division to find the row, and one row factor per workgroup
     const int N = Q + 2 * KV, t = blockIdx.y, row0 = 4 * (int)(blockIdx.x * blockDim.x + threadIdx.x);
-    const float inv = pf_row_inv_wave(ssq, t, nch, D);
-    if (row0 >= N) return;
+    const float part = pf_row_part(ssq, t, nch);
     float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int z = 0; z < splits; ++z) {
-        const float4 v = *(const float4 *)(P + z * plane + (size_t)t * N + row0);
-        s[0] += v.x; s[1] += v.y; s[2] += v.z; s[3] += v.w;
+    if (row0 < N) {
+        for (int z = 0; z < splits; ++z) {
+            const float4 v = *(const float4 *)(P + z * plane + (size_t)t * N + row0);
+            s[0] += v.x; s[1] += v.y; s[2] += v.z; s[3] += v.w;
+        }
     }
+    const float inv = pf_row_finish(part, D);
+    if (row0 >= N) return;
     if (wscale) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) s[e] *= wscale[row0 + e];
@@ -208,14 +215,17 @@ __global__ __launch_bounds__(256) void k_pf_gate_epi(const float *__restrict__ P
                                                      int D, int T, int H, int act, int f16) {
     // grid (ceil(H / 4 / 256), rows)
     const int t = blockIdx.y, j = 4 * (int)(blockIdx.x * blockDim.x + threadIdx.x);
-    const float inv = pf_row_inv_wave(ssq, t, nch, D);
-    if (j >= H) return;
+    const float part = pf_row_part(ssq, t, nch);
     float h[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-    for (int z = 0; z < splits; ++z) {
-        const float4 a = *(const float4 *)(P + z * plane + (size_t)t * 2 * H + 2 * j);
-        const float4 b = *(const float4 *)(P + z * plane + (size_t)t * 2 * H + 2 * j + 4);
-        h[0] += a.x; h[1] += a.y; h[2] += a.z; h[3] += a.w; h[4] += b.x; h[5] += b.y; h[6] += b.z; h[7] += b.w;
+    if (j < H) {
+        for (int z = 0; z < splits; ++z) {
+            const float4 a = *(const float4 *)(P + z * plane + (size_t)t * 2 * H + 2 * j);
+            const float4 b = *(const float4 *)(P + z * plane + (size_t)t * 2 * H + 2 * j + 4);
+            h[0] += a.x; h[1] += a.y; h[2] += a.z; h[3] += a.w; h[4] += b.x; h[5] += b.y; h[6] += b.z; h[7] += b.w;
+        }
     }
+    const float inv = pf_row_finish(part, D);
+    if (j >= H) return;
     if (wscale) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) h[e] *= wscale[2 * j + e];
