@@ -229,6 +229,33 @@ int hipdec_last_device_ms(const hipdec_model *m, float *out_ms);
  * bandwidth roofline is computed from. */
 int hipdec_bytes_per_token(const hipdec_model *m, size_t kv_len, uint64_t *out_bytes);
 
+/* Offline conversion.  The reference's loader reads fp32 RSTK files (engine/src/checkpoint.rs:25-242) and the
+ * model converts them when it is created (lib.rs:159-202 uploads fp32; here also bf16 / e4m3 / 4-bit).  These
+ * entry points, which have no counterpart in the reference, let a caller do that conversion once: copy the
+ * stored weights of a model out (exactly the bytes the kernels read: fused q/k/v rows, interleaved gate/up
+ * rows, every matrix [rows][k] in the weight format, then its scales), keep them in a file, and create later
+ * models from them with plain copies -- an eighth of the fp32 bytes for 4-bit weights, and no staging.
+ * hipdec_packed_sizes_of needs no GPU; sizes are bytes per layer array and for the embedding. */
+typedef struct hipdec_packed_sizes {
+    uint64_t wqkv, wo, w13, w2, s_qkv, s_wo, s_w13, s_w2, gamma, embed;
+} hipdec_packed_sizes;
+typedef struct hipdec_packed_layer {
+    const void *wqkv, *wo, *w13, *w2;          /* hipdec_packed_sizes bytes each */
+    const void *s_qkv, *s_wo, *s_w13, *s_w2;   /* scales; unused (size 0) for fp32 and bf16 weights */
+    const float *gamma1, *gamma2;
+} hipdec_packed_layer;
+typedef struct hipdec_packed_head {
+    const float *gamma_final;
+    const void *embed;                         /* fp32 with fp32 weights, bf16 otherwise */
+} hipdec_packed_head;
+int hipdec_packed_sizes_of(const hipdec_config *cfg, uint32_t weight_dtype, hipdec_packed_sizes *out);
+int hipdec_export_packed_layer(hipdec_model *m, size_t layer_idx, void *wqkv, void *wo, void *w13, void *w2, void *s_qkv,
+                               void *s_wo, void *s_w13, void *s_w2, float *gamma1, float *gamma2);
+int hipdec_export_packed_head(hipdec_model *m, float *gamma_final, void *embed);
+/* As hipdec_create, from stored weights in the format opts->weight_dtype names. */
+int hipdec_create_packed(const hipdec_config *cfg, const hipdec_packed_layer *layers, size_t n_layers,
+                         const hipdec_packed_head *head, const hipdec_options *opts, hipdec_model **out);
+
 /* Debug/verification: copy one stored weight matrix back as fp32 after de-quantisation, in
  * out-major [rows][k] order.  which: 0 wqkv (rows q_dim+2*kv_dim, k dim), 1 wo (dim, q_dim),
  * 2 w13 (2*hidden interleaved gate/up rows, dim), 3 w2 (dim, hidden), 4 embed (vocab, dim). */

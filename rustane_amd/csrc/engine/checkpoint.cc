@@ -1,5 +1,7 @@
 #include "checkpoint.h"
 
+#include "hip_decode.h"
+
 #include <errno.h>
 #include <fcntl.h>
 #include <string.h>
@@ -150,9 +152,92 @@ bool load_checkpoint(const std::string &path, Checkpoint *out, std::string *err)
     void *p = mmap(nullptr, len, PROT_READ, MAP_PRIVATE, fd, 0);
     close(fd);
     if (p == MAP_FAILED) return bad(err, "cannot map " + path + ": " + strerror(errno));
-    const bool ok = parse_checkpoint((const uint8_t *)p, len, out, err, have_shape ? &shape : nullptr);
+    const bool packed = len >= 4 && memcmp(p, "RSTQ", 4) == 0;
+    const bool ok = packed ? parse_packed_checkpoint((const uint8_t *)p, len, out, err)
+                           : parse_checkpoint((const uint8_t *)p, len, out, err, have_shape ? &shape : nullptr);
     munmap(p, len);
     return ok;
+}
+
+namespace {
+constexpr uint32_t kPackedVersion = 1;
+constexpr size_t kPackedHeader = 4 + 12 * 4;
+hipdec_config to_hipdec_config(const ModelConfig &c) {
+    hipdec_config h{};
+    h.dim = (uint32_t)c.dim; h.hidden = (uint32_t)c.hidden; h.heads = (uint32_t)c.heads; h.kv_heads = (uint32_t)c.kv_heads;
+    h.hd = (uint32_t)c.hd; h.seq = (uint32_t)c.seq; h.nlayers = (uint32_t)c.nlayers; h.vocab = (uint32_t)c.vocab;
+    h.q_dim = (uint32_t)c.q_dim; h.kv_dim = (uint32_t)c.kv_dim; h.gqa_ratio = (uint32_t)c.gqa_ratio;
+    return h;
+}
+}  // namespace
+
+bool parse_packed_checkpoint(const uint8_t *bytes, size_t len, Checkpoint *out, std::string *err) {
+    if (len < kPackedHeader) return bad(err, "converted checkpoint too small for header");
+    if (memcmp(bytes, "RSTQ", 4) != 0) return bad(err, "bad converted checkpoint magic");
+    uint32_t h[12];
+    memcpy(h, bytes + 4, sizeof h);
+    if (h[0] != kPackedVersion) return bad(err, "unsupported converted checkpoint version " + std::to_string(h[0]));
+    if (h[2] > 3) return bad(err, "unknown weight format " + std::to_string(h[2]) + " in converted checkpoint");
+    if (h[3] > 1) return bad(err, "unknown ffn activation " + std::to_string(h[3]) + " in converted checkpoint");
+    const uint32_t dim = h[4], hidden = h[5], heads = h[6], kv_heads = h[7], hd = h[8], seq = h[9], nlayers = h[10], vocab = h[11];
+    if (!dim || !hidden || !heads || !kv_heads || !hd || !seq || !nlayers || !vocab || heads % kv_heads != 0)
+        return bad(err, "converted checkpoint header describes no model");
+    out->cfg = ModelConfig::make(dim, hidden, heads, kv_heads, hd, seq, nlayers, vocab, (FfnActivation)h[3]);
+    out->step = h[1];
+    const hipdec_config hc = to_hipdec_config(out->cfg);
+    hipdec_packed_sizes z;
+    if (hipdec_packed_sizes_of(&hc, h[2], &z) != HIPDEC_OK)
+        return bad(err, std::string("converted checkpoint: ") + hipdec_last_error(nullptr));
+    const uint64_t per_layer = z.wqkv + z.s_qkv + z.wo + z.s_wo + z.w13 + z.s_w13 + z.w2 + z.s_w2 + 2 * z.gamma;
+    const uint64_t want = kPackedHeader + z.gamma + z.embed + (uint64_t)nlayers * per_layer;
+    if ((uint64_t)len != want)
+        return bad(err, "converted checkpoint size " + std::to_string(len) + " does not match its header (" + std::to_string(want) + ")");
+    auto pw = std::make_shared<PackedWeights>();
+    pw->dtype = (WeightDtype)h[2];
+    size_t cur = kPackedHeader;
+    auto take = [&](std::vector<uint8_t> *v, uint64_t n) { v->assign(bytes + cur, bytes + cur + n); cur += n; };
+    auto take_f = [&](std::vector<float> *v, uint64_t n) { v->resize(n / 4); memcpy(v->data(), bytes + cur, n); cur += n; };
+    take_f(&pw->gamma_final, z.gamma);
+    take(&pw->embed, z.embed);
+    pw->layers.resize(nlayers);
+    for (PackedLayer &L : pw->layers) {
+        take(&L.wqkv, z.wqkv); take(&L.s_qkv, z.s_qkv); take(&L.wo, z.wo); take(&L.s_wo, z.s_wo);
+        take(&L.w13, z.w13); take(&L.s_w13, z.s_w13); take(&L.w2, z.w2); take(&L.s_w2, z.s_w2);
+        take_f(&L.gamma1, z.gamma); take_f(&L.gamma2, z.gamma);
+    }
+    out->weights = ModelWeights();
+    out->weights.packed = pw;
+    return true;
+}
+
+bool write_packed_checkpoint(const std::string &path, const ModelConfig &c, const PackedWeights &w, uint32_t step,
+                             std::string *err) {
+    const hipdec_config hc = to_hipdec_config(c);
+    hipdec_packed_sizes z;
+    if (hipdec_packed_sizes_of(&hc, (uint32_t)w.dtype, &z) != HIPDEC_OK)
+        return bad(err, std::string("converted checkpoint: ") + hipdec_last_error(nullptr));
+    if (w.layers.size() != c.nlayers) return bad(err, "layer count does not match the configuration");
+    FILE *f = fopen(path.c_str(), "wb");
+    if (!f) return bad(err, "cannot create " + path + ": " + strerror(errno));
+    const uint32_t head[12] = {kPackedVersion, step, (uint32_t)w.dtype, (uint32_t)c.ffn_activation, (uint32_t)c.dim,
+                               (uint32_t)c.hidden, (uint32_t)c.heads, (uint32_t)c.kv_heads, (uint32_t)c.hd, (uint32_t)c.seq,
+                               (uint32_t)c.nlayers, (uint32_t)c.vocab};
+    bool ok = fwrite("RSTQ", 1, 4, f) == 4 && fwrite(head, 4, 12, f) == 12;
+    auto put = [&](const void *p, size_t have, uint64_t want) {
+        ok = ok && have == want && (want == 0 || fwrite(p, 1, want, f) == want);
+    };
+    put(w.gamma_final.data(), w.gamma_final.size() * 4, z.gamma);
+    put(w.embed.data(), w.embed.size(), z.embed);
+    for (const PackedLayer &L : w.layers) {
+        put(L.wqkv.data(), L.wqkv.size(), z.wqkv); put(L.s_qkv.data(), L.s_qkv.size(), z.s_qkv);
+        put(L.wo.data(), L.wo.size(), z.wo); put(L.s_wo.data(), L.s_wo.size(), z.s_wo);
+        put(L.w13.data(), L.w13.size(), z.w13); put(L.s_w13.data(), L.s_w13.size(), z.s_w13);
+        put(L.w2.data(), L.w2.size(), z.w2); put(L.s_w2.data(), L.s_w2.size(), z.s_w2);
+        put(L.gamma1.data(), L.gamma1.size() * 4, z.gamma); put(L.gamma2.data(), L.gamma2.size() * 4, z.gamma);
+    }
+    ok = (fclose(f) == 0) && ok;
+    if (!ok) return bad(err, "short write or array size mismatch writing " + path);
+    return true;
 }
 
 bool write_checkpoint(const std::string &path, const ModelConfig &c, const ModelWeights &w, uint32_t step,

@@ -67,6 +67,26 @@ DecodeContext::DecodeContext(const ModelConfig &cfg, const ModelWeights &weights
     c.kv_heads = (uint32_t)cfg.kv_heads; c.hd = (uint32_t)cfg.hd; c.seq = (uint32_t)cfg.seq;
     c.nlayers = (uint32_t)cfg.nlayers; c.vocab = (uint32_t)cfg.vocab; c.q_dim = (uint32_t)cfg.q_dim;
     c.kv_dim = (uint32_t)cfg.kv_dim; c.gqa_ratio = (uint32_t)cfg.gqa_ratio;
+    hipdec_options o{};
+    o.weight_dtype = (uint32_t)wdt; o.kv_dtype = (uint32_t)kvdt; o.device = device;
+    o.ffn_activation = (uint32_t)cfg.ffn_activation; o.flags = flags;
+    if (weights.packed) {
+        // a checkpoint converted ahead of time: the stored bytes go to the device as they are
+        const PackedWeights &p = *weights.packed;
+        if (p.dtype != wdt) throw std::runtime_error("failed to initialize hip decode: the checkpoint holds converted weights of another format than the one asked for");
+        std::vector<hipdec_packed_layer> pl(p.layers.size());
+        for (size_t l = 0; l < pl.size(); ++l) {
+            const PackedLayer &L = p.layers[l];
+            pl[l] = hipdec_packed_layer{L.wqkv.data(), L.wo.data(), L.w13.data(), L.w2.data(), L.s_qkv.data(), L.s_wo.data(),
+                                        L.s_w13.data(), L.s_w2.data(), L.gamma1.data(), L.gamma2.data()};
+        }
+        hipdec_packed_head ph{p.gamma_final.data(), p.embed.data()};
+        int prc = hipdec_create_packed(&c, pl.data(), pl.size(), &ph, &o, &m_);
+        if (prc != HIPDEC_OK)
+            throw std::runtime_error(std::string("failed to initialize hip decode: ") + hipdec_last_error(nullptr));
+        init_buffers(cfg);
+        return;
+    }
     std::vector<hipdec_layer_f32> layers(weights.layers.size());
     for (size_t l = 0; l < layers.size(); ++l) {
         const LayerWeights &L = weights.layers[l];
@@ -74,9 +94,6 @@ DecodeContext::DecodeContext(const ModelConfig &cfg, const ModelWeights &weights
                                      L.w3.data(), L.w2.data(), L.gamma1.data(), L.gamma2.data()};
     }
     hipdec_head_f32 head{weights.gamma_final.data(), weights.embed.data()};
-    hipdec_options o{};
-    o.weight_dtype = (uint32_t)wdt; o.kv_dtype = (uint32_t)kvdt; o.device = device;
-    o.ffn_activation = (uint32_t)cfg.ffn_activation; o.flags = flags;
     int rc = hipdec_create(&c, layers.data(), layers.size(), &head, &o, &m_);
     if (rc != HIPDEC_OK)
         throw std::runtime_error(std::string("failed to initialize hip decode: ") + hipdec_last_error(nullptr));
@@ -88,6 +105,30 @@ DecodeContext::DecodeContext(const ModelConfig &cfg, const DecodeContext &weight
     if (rc != HIPDEC_OK)
         throw std::runtime_error(std::string("failed to initialize hip decode: ") + hipdec_last_error(nullptr));
     init_buffers(cfg);
+}
+
+void DecodeContext::export_packed(const ModelConfig &cfg, WeightDtype wdt, PackedWeights *out) const {
+    hipdec_config c{};
+    c.dim = (uint32_t)cfg.dim; c.hidden = (uint32_t)cfg.hidden; c.heads = (uint32_t)cfg.heads;
+    c.kv_heads = (uint32_t)cfg.kv_heads; c.hd = (uint32_t)cfg.hd; c.seq = (uint32_t)cfg.seq;
+    c.nlayers = (uint32_t)cfg.nlayers; c.vocab = (uint32_t)cfg.vocab; c.q_dim = (uint32_t)cfg.q_dim;
+    c.kv_dim = (uint32_t)cfg.kv_dim; c.gqa_ratio = (uint32_t)cfg.gqa_ratio;
+    hipdec_packed_sizes z;
+    check(hipdec_packed_sizes_of(&c, (uint32_t)wdt, &z), "packed sizes");
+    out->dtype = wdt;
+    out->layers.resize(cfg.nlayers);
+    for (size_t l = 0; l < cfg.nlayers; ++l) {
+        PackedLayer &L = out->layers[l];
+        L.wqkv.resize(z.wqkv); L.wo.resize(z.wo); L.w13.resize(z.w13); L.w2.resize(z.w2);
+        L.s_qkv.resize(z.s_qkv); L.s_wo.resize(z.s_wo); L.s_w13.resize(z.s_w13); L.s_w2.resize(z.s_w2);
+        L.gamma1.resize(z.gamma / 4); L.gamma2.resize(z.gamma / 4);
+        check(hipdec_export_packed_layer(m_, l, L.wqkv.data(), L.wo.data(), L.w13.data(), L.w2.data(), L.s_qkv.data(),
+                                         L.s_wo.data(), L.s_w13.data(), L.s_w2.data(), L.gamma1.data(), L.gamma2.data()),
+              "export layer");
+    }
+    out->gamma_final.resize(z.gamma / 4);
+    out->embed.resize(z.embed);
+    check(hipdec_export_packed_head(m_, out->gamma_final.data(), out->embed.data()), "export head");
 }
 
 void DecodeContext::init_buffers(const ModelConfig &cfg) {

@@ -32,6 +32,8 @@ public:
     // KV caches and step state of its own; the weights live as long as any context that uses them
     DecodeContext(const ModelConfig &cfg, const DecodeContext &weights_of, KvDtype kvdt, uint32_t flags);
     ~DecodeContext();
+    // the weights as this context's model stores them on the device (for a checkpoint converted ahead of time)
+    void export_packed(const ModelConfig &cfg, WeightDtype wdt, PackedWeights *out) const;
     DecodeContext(const DecodeContext &) = delete;
     DecodeContext &operator=(const DecodeContext &) = delete;
 

@@ -98,6 +98,18 @@ rs_weights *rs_checkpoint_load(const char *path, rs_config *cfg_out, uint32_t *s
     if (!load_checkpoint(path, &ck, &e)) { put_err(err, errcap, e); return nullptr; }
     return take_checkpoint(ck, cfg_out, step);
 }
+// A converted checkpoint's header and size check (no device needed): 0 = ok; cfg, step and the weight format
+// (0 fp32, 1 bf16, 2 e4m3, 3 4-bit) filled; 1 = rejected with the loader's message.
+int rs_packed_checkpoint_parse(const uint8_t *bytes, size_t n, rs_config *cfg_out, uint32_t *step, uint32_t *dtype, char *err,
+                               size_t errcap) {
+    Checkpoint ck;
+    std::string e;
+    if (!parse_packed_checkpoint(bytes, n, &ck, &e)) { put_err(err, errcap, e); return 1; }
+    from_cfg(ck.cfg, cfg_out);
+    *step = ck.step;
+    *dtype = (uint32_t)ck.weights.packed->dtype;
+    return 0;
+}
 int rs_checkpoint_write(const char *path, const rs_config *c, const rs_weights *w, uint32_t step, char *err, size_t errcap) {
     std::string e;
     if (!write_checkpoint(path, to_cfg(c), w->w, step, &e)) { put_err(err, errcap, e); return 1; }

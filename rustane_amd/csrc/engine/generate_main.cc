@@ -6,11 +6,13 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <stdexcept>
 #include <string>
 #include <vector>
 
 #include "checkpoint.h"
 #include "cli_common.h"
+#include "decode_context.h"
 #include "inference.h"
 #include "jsonl_session.h"
 #include "synth.h"
@@ -25,6 +27,7 @@ void usage() {
            "  [--steps N] [--temperature T] [--top-k K] [--softcap C] [--samples N] [--seed S]\n"
            "  [--decode-backend auto|naive|hip] [--kv-cache] [--weight-dtype f32|bf16|fp8|int4] [--kv-dtype f32|bf16]\n"
            "  [--weight-seed S] [--weight-std X] [--random-prompt N] [--jsonl-session]\n"
+           "  [--convert-to OUT: write the model's weights in the --weight-dtype format as a converted checkpoint and exit]\n"
            "presets: %s\n", kPresets);
 }
 
@@ -53,7 +56,8 @@ std::string format_ids(const std::vector<uint32_t> &ids) {
 }  // namespace
 
 int main(int argc, char **argv) {
-    std::string model = "gpt_1024", checkpoint, prompt_ids_raw, wdt = "f32", kvdt = "f32";
+    std::string model = "gpt_1024", checkpoint, prompt_ids_raw, wdt = "f32", kvdt = "f32", convert_to;
+    bool wdt_given = false;
     GenerationRequest req;
     float softcap = 0.0f, weight_std = 0.02f;
     uint64_t weight_seed = 1234;
@@ -74,7 +78,8 @@ int main(int argc, char **argv) {
         else if (a == "--seed") req.seed = strtoull(val().c_str(), nullptr, 10);
         else if (a == "--weight-seed") weight_seed = strtoull(val().c_str(), nullptr, 10);
         else if (a == "--weight-std") weight_std = strtof(val().c_str(), nullptr);
-        else if (a == "--weight-dtype") wdt = val();
+        else if (a == "--weight-dtype") { wdt = val(); wdt_given = true; }
+        else if (a == "--convert-to") convert_to = val();
         else if (a == "--kv-dtype") kvdt = val();
         else if (a == "--jsonl-session") jsonl_session = true;                          // generate.rs:236-238
         else if (a == "--kv-cache") req.decode_backend = DecodeBackendRequest::Hip;     // generate.rs:189-192
@@ -102,6 +107,30 @@ int main(int argc, char **argv) {
     } else if (!model_from_name(model, &cfg)) fail("unknown --model " + model);
     SessionOptions opts;
     parse_formats(wdt, kvdt, &opts);
+    if (ckpt.weights.packed) {
+        // a checkpoint converted ahead of time carries its weight format
+        if (!wdt_given) opts.weight_dtype = ckpt.weights.packed->dtype;
+        else if (opts.weight_dtype != ckpt.weights.packed->dtype)
+            fail("--weight-dtype " + wdt + " does not match the format this converted checkpoint holds");
+    }
+    if (!convert_to.empty()) {
+        // offline conversion: build the model once in the asked weight format, write its stored weights
+        if (ckpt.weights.packed) fail("--convert-to needs the fp32 checkpoint, this one is converted already");
+        try {
+            const ModelWeights src = checkpoint.empty()
+                                         ? ModelWeights::synthetic(cfg, weight_seed, weight_std, opts.weight_dtype != WeightDtype::F32)
+                                         : std::move(ckpt.weights);
+            DecodeContext ctx(cfg, src, opts.weight_dtype, KvDtype::F32, 0, 0);
+            PackedWeights packed;
+            ctx.export_packed(cfg, opts.weight_dtype, &packed);
+            std::string werr;
+            if (!write_packed_checkpoint(convert_to, cfg, packed, ckpt.step, &werr)) fail(werr);
+        } catch (const std::exception &e) {
+            fail(e.what());
+        }
+        printf("converted_checkpoint=%s weight_dtype=%s step=%u\n", convert_to.c_str(), wdt.c_str(), ckpt.step);
+        return 0;
+    }
 
     std::vector<uint32_t> prompt = parse_ids(prompt_ids_raw);
     if (prompt.empty() && random_prompt) {

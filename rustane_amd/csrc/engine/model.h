@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include <string>
+#include <memory>
 #include <vector>
 
 namespace rustane {
@@ -49,16 +50,31 @@ struct ModelConfig {
 struct LayerWeights {
     std::vector<float> wq, wk, wv, wo, w1, w3, w2, gamma1, gamma2;
 };
+enum class WeightDtype : uint32_t { F32 = 0, BF16 = 1, FP8_E4M3 = 2, INT4_G128 = 3 };
+enum class KvDtype : uint32_t { F32 = 0, BF16 = 1 };
+
+// Weights as the decode library stores them on the device (converted ahead of time, checkpoint.h): per layer
+// the fused q/k/v, wo, interleaved gate/up and w2 matrices in the weight format, their scales, the norm gains.
+struct PackedLayer {
+    std::vector<uint8_t> wqkv, wo, w13, w2, s_qkv, s_wo, s_w13, s_w2;
+    std::vector<float> gamma1, gamma2;
+};
+struct PackedWeights {
+    WeightDtype dtype = WeightDtype::F32;
+    std::vector<PackedLayer> layers;
+    std::vector<float> gamma_final;
+    std::vector<uint8_t> embed;              // fp32 with fp32 weights, bf16 otherwise
+};
+
 // full_model.rs:19-23
 struct ModelWeights {
     std::vector<float> embed, gamma_final;
     std::vector<LayerWeights> layers;
+    // set instead of the fp32 tensors above by a checkpoint that was converted ahead of time
+    std::shared_ptr<const PackedWeights> packed;
 
     // every matrix N(0, std) from the counter-based generator, norm gains 1
     static ModelWeights synthetic(const ModelConfig &cfg, uint64_t seed, float std, bool round_bf16);
 };
-
-enum class WeightDtype : uint32_t { F32 = 0, BF16 = 1, FP8_E4M3 = 2, INT4_G128 = 3 };
-enum class KvDtype : uint32_t { F32 = 0, BF16 = 1 };
 
 }  // namespace rustane

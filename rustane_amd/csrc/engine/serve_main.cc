@@ -32,6 +32,7 @@ int main(int argc, char **argv) {
     float softcap = 0.0f, weight_std = 0.02f;
     uint64_t weight_seed = 1234;
     size_t max_cache_sessions = 32;
+    bool wdt_given = false;
     for (int i = 1; i < argc; ++i) {
         std::string a = argv[i];
         auto val = [&]() -> std::string { if (i + 1 >= argc) fail(a + " needs a value"); return argv[++i]; };
@@ -49,7 +50,7 @@ int main(int argc, char **argv) {
             if (!parse_decode_backend(raw, &backend)) fail("--decode-backend must be one of: auto, naive, hip");
         } else if (a == "--softcap") softcap = strtof(val().c_str(), nullptr);
         else if (a == "--max-cache-sessions") max_cache_sessions = count("an integer");
-        else if (a == "--weight-dtype") wdt = val();
+        else if (a == "--weight-dtype") { wdt = val(); wdt_given = true; }
         else if (a == "--kv-dtype") kvdt = val();
         else if (a == "--weight-seed") weight_seed = count("an integer");
         else if (a == "--weight-std") weight_std = strtof(val().c_str(), nullptr);
@@ -76,6 +77,11 @@ int main(int argc, char **argv) {
         std::string cerr;
         if (!load_checkpoint(checkpoint, &ckpt, &cerr)) fail("failed to load checkpoint: " + cerr);
         cfg = ckpt.cfg;
+        if (ckpt.weights.packed) {               // a checkpoint converted ahead of time carries its weight format
+            if (!wdt_given) opts.weight_dtype = ckpt.weights.packed->dtype;
+            else if (opts.weight_dtype != ckpt.weights.packed->dtype)
+                fail("--weight-dtype " + wdt + " does not match the format this converted checkpoint holds");
+        }
     } else if (!model_from_name(model, &cfg)) fail("unknown --model " + model);
     const ModelWeights weights = checkpoint.empty()
                                      ? ModelWeights::synthetic(cfg, weight_seed, weight_std, opts.weight_dtype != WeightDtype::F32)

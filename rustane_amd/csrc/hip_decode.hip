@@ -1094,7 +1094,8 @@ void hipdec_destroy(hipdec_model *m) {
 
 // base != null: the new model takes base's weights (same configuration and weight format) instead of uploading any
 static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hipdec_head_f32 *head,
-                       const hipdec_model *base = nullptr) {
+                       const hipdec_model *base = nullptr, const hipdec_packed_layer *packed = nullptr,
+                       const hipdec_packed_head *phead = nullptr) {
     const hipdec_config &c = m->cfg;
     const size_t D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden, V = c.vocab, S = c.seq;
     HCHK(hipSetDevice(m->opt.device));
@@ -1116,8 +1117,10 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
     } else {
         m->wstore = std::make_shared<WeightStore>();
         m->wstore->device = m->opt.device;
-        HCHK(hipMalloc((void **)&stage_a, max_elems * sizeof(float)));
-        HCHK(hipMalloc((void **)&stage_b, max_elems * sizeof(float)));
+        if (!packed) {                                   // (stored weights are copied as they are: nothing to stage)
+            HCHK(hipMalloc((void **)&stage_a, max_elems * sizeof(float)));
+            HCHK(hipMalloc((void **)&stage_b, max_elems * sizeof(float)));
+        }
     }
     int rc = HIPDEC_OK;
     auto done = [&](int code) { (void)hipFree(stage_a); (void)hipFree(stage_b); return code; };
@@ -1137,6 +1140,29 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
         HCHK(hipMemsetAsync(L.kc, 0, S * KV * kvsz, m->stream));
         HCHK(hipMemsetAsync(L.vc, 0, S * KV * kvsz, m->stream));
         if (base) continue;
+        if (packed) {
+            // weights as an earlier model stored them (hipdec_export_packed_*): copied, not converted
+            const hipdec_packed_layer &p = packed[l];
+            const size_t wb[4] = {wt_row_bytes(wt, D) * (Q + 2 * KV), wt_row_bytes(wt, Q) * D, wt_row_bytes(wt, D) * 2 * H,
+                                  wt_row_bytes(wt, H) * D};
+            const size_t sb[4] = {wt_scale_bytes(wt, Q + 2 * KV, D), wt_scale_bytes(wt, D, Q), wt_scale_bytes(wt, 2 * H, D),
+                                  wt_scale_bytes(wt, D, H)};
+            const void *wsrc[4] = {p.wqkv, p.wo, p.w13, p.w2}, *ssrc[4] = {p.s_qkv, p.s_wo, p.s_w13, p.s_w2};
+            void **wdst[4] = {&L.wqkv, &L.wo, &L.w13, &L.w2}, **sdst[4] = {&L.s_qkv, &L.s_wo, &L.s_w13, &L.s_w2};
+            if (!p.gamma1 || !p.gamma2) return done(fail(m, HIPDEC_ERR_ARG, "null layer weight pointer"));
+            for (int i = 0; i < 4; ++i) {
+                if (!wsrc[i] || (sb[i] && !ssrc[i])) return done(fail(m, HIPDEC_ERR_ARG, "null layer weight pointer"));
+                TRY(walloc(m, wdst[i], wb[i]));
+                HCHK(hipMemcpy(*wdst[i], wsrc[i], wb[i], hipMemcpyHostToDevice));
+                TRY(walloc(m, sdst[i], sb[i]));
+                if (sb[i]) HCHK(hipMemcpy(*sdst[i], ssrc[i], sb[i], hipMemcpyHostToDevice));
+            }
+            TRY(walloc(m, &L.g1, D * 4));
+            TRY(walloc(m, &L.g2, D * 4));
+            HCHK(hipMemcpy(L.g1, p.gamma1, D * 4, hipMemcpyHostToDevice));
+            HCHK(hipMemcpy(L.g2, p.gamma2, D * 4, hipMemcpyHostToDevice));
+            continue;
+        }
         const hipdec_layer_f32 &src = layers[l];
         if (!src.wq || !src.wk || !src.wv || !src.wo || !src.w1 || !src.w3 || !src.w2 || !src.gamma1 || !src.gamma2)
             return done(fail(m, HIPDEC_ERR_ARG, "null layer weight pointer"));
@@ -1163,6 +1189,11 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
     if (base) {
         m->embed = base->embed;
         m->gfinal = base->gfinal;
+    } else if (packed) {
+        TRY(walloc(m, &m->embed, wt_row_bytes(m->embed_wt, D) * V));
+        HCHK(hipMemcpy(m->embed, phead->embed, wt_row_bytes(m->embed_wt, D) * V, hipMemcpyHostToDevice));
+        TRY(walloc(m, &m->gfinal, D * 4));
+        HCHK(hipMemcpy(m->gfinal, phead->gamma_final, D * 4, hipMemcpyHostToDevice));
     } else {
         TRY(walloc(m, &m->embed, wt_row_bytes(m->embed_wt, D) * V));
         TRY(load_matrix(m, m->embed_wt, head->embed, V, D, false, stage_a, stage_b, m->embed, nullptr, 1, 0));
@@ -1320,28 +1351,105 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
     return done(HIPDEC_OK);
 }
 
-int hipdec_create(const hipdec_config *cfg, const hipdec_layer_f32 *layers, size_t n_layers,
-                  const hipdec_head_f32 *head, const hipdec_options *opts, hipdec_model **out) {
-    if (out) *out = nullptr;
-    if (!cfg || !layers || !head || !out) return fail(nullptr, HIPDEC_ERR_ARG, "null argument");
-    if (!head->embed || !head->gamma_final) return fail(nullptr, HIPDEC_ERR_ARG, "null head weight pointer");
-    if (n_layers != cfg->nlayers) return fail(nullptr, HIPDEC_ERR_ARG, "layer count does not match cfg.nlayers");
-    const hipdec_config &c = *cfg;
+// the checks on a configuration that need no device (shared by model creation and hipdec_packed_sizes_of)
+static int check_config(const hipdec_config &c, uint32_t weight_dtype) {
     if (!c.dim || !c.hidden || !c.heads || !c.kv_heads || !c.hd || !c.seq || !c.nlayers || !c.vocab)
         return fail(nullptr, HIPDEC_ERR_ARG, "zero-sized config field");
     if (c.q_dim != c.heads * c.hd || c.kv_dim != c.kv_heads * c.hd || c.heads % c.kv_heads != 0 ||
         (c.gqa_ratio ? c.gqa_ratio : 1) != c.heads / c.kv_heads)
         return fail(nullptr, HIPDEC_ERR_ARG, "inconsistent head geometry");
-    hipdec_options o{};
-    if (opts) o = *opts;
-    if (o.weight_dtype > HIPDEC_W_INT4_G128 || o.kv_dtype > HIPDEC_KV_BF16 || o.ffn_activation > 1)
-        return fail(nullptr, HIPDEC_ERR_ARG, "unknown option value");
+    if (weight_dtype > HIPDEC_W_INT4_G128) return fail(nullptr, HIPDEC_ERR_ARG, "unknown option value");
     if (c.hd != 64 && c.hd != 128) return fail(nullptr, HIPDEC_ERR_UNSUPPORTED, "head dim must be 64 or 128");
-    uint32_t kmul = o.weight_dtype == HIPDEC_W_INT4_G128 ? 128 : (o.weight_dtype == HIPDEC_W_FP8_E4M3 ? 16 : 8);
+    const uint32_t kmul = weight_dtype == HIPDEC_W_INT4_G128 ? 128 : (weight_dtype == HIPDEC_W_FP8_E4M3 ? 16 : 8);
     if (c.dim % kmul || c.hidden % kmul || c.q_dim % kmul || c.kv_dim % 8)
         return fail(nullptr, HIPDEC_ERR_UNSUPPORTED, "dim / hidden / q_dim must be multiples of the weight load width");
     if ((size_t)(c.hidden > c.dim ? c.hidden : c.dim) * 4 > 150 * 1024)
         return fail(nullptr, HIPDEC_ERR_UNSUPPORTED, "reduction axis does not fit LDS");
+    return HIPDEC_OK;
+}
+
+static int create_front(const hipdec_config *cfg, const hipdec_layer_f32 *layers, const hipdec_head_f32 *head,
+                        const hipdec_packed_layer *packed, const hipdec_packed_head *phead, size_t n_layers,
+                        const hipdec_options *opts, hipdec_model **out);
+
+int hipdec_create(const hipdec_config *cfg, const hipdec_layer_f32 *layers, size_t n_layers,
+                  const hipdec_head_f32 *head, const hipdec_options *opts, hipdec_model **out) {
+    if (out) *out = nullptr;
+    if (!cfg || !layers || !head || !out) return fail(nullptr, HIPDEC_ERR_ARG, "null argument");
+    if (!head->embed || !head->gamma_final) return fail(nullptr, HIPDEC_ERR_ARG, "null head weight pointer");
+    return create_front(cfg, layers, head, nullptr, nullptr, n_layers, opts, out);
+}
+
+int hipdec_create_packed(const hipdec_config *cfg, const hipdec_packed_layer *layers, size_t n_layers,
+                         const hipdec_packed_head *head, const hipdec_options *opts, hipdec_model **out) {
+    if (out) *out = nullptr;
+    if (!cfg || !layers || !head || !out) return fail(nullptr, HIPDEC_ERR_ARG, "null argument");
+    if (!head->embed || !head->gamma_final) return fail(nullptr, HIPDEC_ERR_ARG, "null head weight pointer");
+    return create_front(cfg, nullptr, nullptr, layers, head, n_layers, opts, out);
+}
+
+int hipdec_packed_sizes_of(const hipdec_config *cfg, uint32_t weight_dtype, hipdec_packed_sizes *out) {
+    if (!cfg || !out) return fail(nullptr, HIPDEC_ERR_ARG, "null argument");
+    const int rc = check_config(*cfg, weight_dtype);
+    if (rc != HIPDEC_OK) return rc;
+    const hipdec_config &c = *cfg;
+    const int wt = (int)weight_dtype, ewt = weight_dtype == HIPDEC_W_F32 ? WT_F32 : WT_BF16;
+    const size_t D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden;
+    out->wqkv = wt_row_bytes(wt, D) * (Q + 2 * KV); out->s_qkv = wt_scale_bytes(wt, Q + 2 * KV, D);
+    out->wo = wt_row_bytes(wt, Q) * D;              out->s_wo = wt_scale_bytes(wt, D, Q);
+    out->w13 = wt_row_bytes(wt, D) * 2 * H;         out->s_w13 = wt_scale_bytes(wt, 2 * H, D);
+    out->w2 = wt_row_bytes(wt, H) * D;              out->s_w2 = wt_scale_bytes(wt, D, H);
+    out->gamma = D * 4;
+    out->embed = wt_row_bytes(ewt, D) * c.vocab;
+    return HIPDEC_OK;
+}
+
+int hipdec_export_packed_layer(hipdec_model *m, size_t layer_idx, void *wqkv, void *wo, void *w13, void *w2, void *s_qkv,
+                               void *s_wo, void *s_w13, void *s_w2, float *gamma1, float *gamma2) {
+    if (!m) return HIPDEC_ERR_ARG;
+    if (layer_idx >= m->layers.size()) return fail(m, HIPDEC_ERR_ARG, "layer index out of range");
+    hipdec_packed_sizes z;
+    int rc = hipdec_packed_sizes_of(&m->cfg, (uint32_t)m->wt, &z);
+    if (rc != HIPDEC_OK) return rc;
+    const DevLayer &L = m->layers[layer_idx];
+    const void *src[10] = {L.wqkv, L.wo, L.w13, L.w2, L.s_qkv, L.s_wo, L.s_w13, L.s_w2, L.g1, L.g2};
+    void *dst[10] = {wqkv, wo, w13, w2, s_qkv, s_wo, s_w13, s_w2, gamma1, gamma2};
+    const uint64_t bytes[10] = {z.wqkv, z.wo, z.w13, z.w2, z.s_qkv, z.s_wo, z.s_w13, z.s_w2, z.gamma, z.gamma};
+    HCHK(hipSetDevice(m->opt.device));
+    HCHK(hipStreamSynchronize(m->stream));
+    for (int i = 0; i < 10; ++i) {
+        if (!bytes[i]) continue;
+        if (!dst[i]) return fail(m, HIPDEC_ERR_ARG, "null output pointer");
+        HCHK(hipMemcpy(dst[i], src[i], bytes[i], hipMemcpyDeviceToHost));
+    }
+    return HIPDEC_OK;
+}
+
+int hipdec_export_packed_head(hipdec_model *m, float *gamma_final, void *embed) {
+    if (!m) return HIPDEC_ERR_ARG;
+    if (!gamma_final || !embed) return fail(m, HIPDEC_ERR_ARG, "null output pointer");
+    hipdec_packed_sizes z;
+    int rc = hipdec_packed_sizes_of(&m->cfg, (uint32_t)m->wt, &z);
+    if (rc != HIPDEC_OK) return rc;
+    HCHK(hipSetDevice(m->opt.device));
+    HCHK(hipStreamSynchronize(m->stream));
+    HCHK(hipMemcpy(gamma_final, m->gfinal, z.gamma, hipMemcpyDeviceToHost));
+    HCHK(hipMemcpy(embed, m->embed, z.embed, hipMemcpyDeviceToHost));
+    return HIPDEC_OK;
+}
+
+static int create_front(const hipdec_config *cfg, const hipdec_layer_f32 *layers, const hipdec_head_f32 *head,
+                        const hipdec_packed_layer *packed, const hipdec_packed_head *phead, size_t n_layers,
+                        const hipdec_options *opts, hipdec_model **out) {
+    if (n_layers != cfg->nlayers) return fail(nullptr, HIPDEC_ERR_ARG, "layer count does not match cfg.nlayers");
+    const hipdec_config &c = *cfg;
+    hipdec_options o{};
+    if (opts) o = *opts;
+    if (o.kv_dtype > HIPDEC_KV_BF16 || o.ffn_activation > 1) return fail(nullptr, HIPDEC_ERR_ARG, "unknown option value");
+    {
+        const int crc = check_config(c, o.weight_dtype);
+        if (crc != HIPDEC_OK) return crc;
+    }
     hipdec_model *m = new hipdec_model();
     m->cfg = c;
     // HIPDEC_NO_GRAPH=1 in the environment forces eager launches (profilers that cannot follow
@@ -1368,7 +1476,7 @@ int hipdec_create(const hipdec_config *cfg, const hipdec_layer_f32 *layers, size
                 : (m->kvbf16 && quantised)                 ? PF_ACT_F16
                                                            : PF_ACT_PAIR;
     m->alpha = 1.0f / sqrtf(2.0f * (float)c.nlayers);   // lib.rs:201
-    int rc = create_impl(m, layers, head);
+    int rc = create_impl(m, layers, head, nullptr, packed, phead);
     if (rc != HIPDEC_OK) {
         g_create_error = m->err;
         hipdec_destroy(m);

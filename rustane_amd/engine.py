@@ -76,6 +76,7 @@ def lib():
         L.rs_http_prepare.argtypes = [C.c_char_p, C.c_int, C.c_char_p, C.c_uint64, C.c_uint32, C.POINTER(RsRequest),
                                       C.POINTER(C.c_int), u32p, C.c_size_t, u64p, C.c_char_p, C.c_size_t]
         L.rs_http_render_chat_prompt.argtypes = [C.c_char_p, C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t]
+        L.rs_packed_checkpoint_parse.argtypes = [C.c_char_p, C.c_size_t, C.POINTER(RsConfig), u32p, u32p, C.c_char_p, C.c_size_t]
         L.rs_weights_tensor.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.POINTER(fp), u64p]
         L.rs_session_new.restype = C.c_void_p
         L.rs_session_new.argtypes = [C.POINTER(RsConfig), C.c_void_p, u32p, C.c_size_t, C.c_float, C.c_uint32,
@@ -467,6 +468,16 @@ def write_checkpoint(path, cfg, weights, step=0, ffn_activation=0):
             raise CheckpointError(err.value.decode())
     finally:
         L.rs_weights_free(h)
+
+
+def parse_packed_checkpoint(data):
+    """Header and size check of a converted checkpoint (the weights as the decode library stores them for one
+    weight format) -> (RsConfig fields as a dict, step, weight format code)."""
+    L = lib()
+    rc, step, dtype, err = RsConfig(), C.c_uint32(), C.c_uint32(), C.create_string_buffer(512)
+    if L.rs_packed_checkpoint_parse(bytes(data), len(data), C.byref(rc), C.byref(step), C.byref(dtype), err, 512):
+        raise CheckpointError(err.value.decode())
+    return {k: int(getattr(rc, k)) for k, _ in RsConfig._fields_}, step.value, dtype.value
 
 
 # ---------------------------------------------------------------- JSONL session protocol (bin/generate.rs:39-144)

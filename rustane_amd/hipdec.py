@@ -20,7 +20,8 @@ HEAD_BLOCK = 256
 OK, ERR_ARG, ERR_FULL, ERR_HIP, ERR_UNSUPPORTED = 0, 1, 2, 3, 4
 
 EXPORTS = [
-    "hipdec_create", "hipdec_create_shared", "hipdec_destroy", "hipdec_last_error", "hipdec_len", "hipdec_set_len", "hipdec_set_prefill_activations",
+    "hipdec_create", "hipdec_create_shared", "hipdec_create_packed", "hipdec_packed_sizes_of", "hipdec_export_packed_layer",
+    "hipdec_export_packed_head", "hipdec_destroy", "hipdec_last_error", "hipdec_len", "hipdec_set_len", "hipdec_set_prefill_activations",
     "hipdec_seed_layer_cache_from_channel_first", "hipdec_decode_token", "hipdec_decode_token_from_id",
     "hipdec_decode_token_argmax", "hipdec_decode_token_argmax_from_id", "hipdec_decode_token_topk_from_id",
     "hipdec_decode_token_block_stats_from_id", "hipdec_materialize_current_logits_block",

@@ -140,3 +140,112 @@ def test_session_from_checkpoint_equals_session_from_arrays(tmp_path):
     a = engine.InferenceSession(cfg, w, prompt, weight_dtype=1, kv_dtype=0).generate(req)
     b = engine.InferenceSession(cfg2, w2, prompt, weight_dtype=1, kv_dtype=0, ffn_activation=act).generate(req)
     np.testing.assert_array_equal(a.results[0].sampled, b.results[0].sampled)
+
+
+# ---------------------------------------------------------------- converted checkpoints (this build's "RSTQ" file)
+def _packed_bytes(cfg, dtype, step=7, act=0, version=1, extra=0):
+    """A converted checkpoint of the right size for (cfg, weight format), built from the format description."""
+    import ctypes as C
+    from rustane_amd import hipdec
+
+    class Sizes(C.Structure):
+        _fields_ = [(n, C.c_uint64) for n in ("wqkv", "wo", "w13", "w2", "s_qkv", "s_wo", "s_w13", "s_w2", "gamma", "embed")]
+
+    lib = hipdec.load_library()
+    z = Sizes()
+    rc = lib.hipdec_packed_sizes_of(C.byref(cfg), dtype, C.byref(z))
+    if rc:
+        return None, rc
+    per_layer = z.wqkv + z.s_qkv + z.wo + z.s_wo + z.w13 + z.s_w13 + z.w2 + z.s_w2 + 2 * z.gamma
+    head = b"RSTQ" + np.array([version, step, dtype, act, cfg.dim, cfg.hidden, cfg.heads, cfg.kv_heads, cfg.hd, cfg.seq,
+                               cfg.nlayers, cfg.vocab], np.uint32).tobytes()
+    return head + bytes(z.gamma + z.embed + cfg.nlayers * per_layer + extra), 0
+
+
+def test_converted_checkpoint_header_and_sizes():
+    cfg = Config.make(dim=256, hidden=640, heads=2, hd=128, seq=64, nlayers=3, vocab=320)
+    sizes = {}
+    for dtype in (0, 1, 2, 3):
+        data, rc = _packed_bytes(cfg, dtype, step=41, act=1 if dtype == 2 else 0)
+        assert rc == 0
+        got, step, dt = engine.parse_packed_checkpoint(data)
+        assert (step, dt) == (41, dtype) and got["ffn_activation"] == (1 if dtype == 2 else 0)
+        assert [got[k] for k in ("dim", "hidden", "heads", "kv_heads", "hd", "seq", "nlayers", "vocab")] == \
+               [256, 640, 2, 2, 128, 64, 3, 320]
+        sizes[dtype] = len(data)
+    # fp32 : bf16 : e4m3 : 4-bit matrices are 4 : 2 : 1 : 0.5 bytes per weight (+ scales, norms and the bf16 embedding)
+    assert sizes[0] > sizes[1] > sizes[2] > sizes[3]
+    lin = 3 * (4 * 256 * 256 + 3 * 256 * 640)
+    assert sizes[1] - sizes[2] == lin - 3 * 4 * (768 + 256 + 1280 + 256)          # one byte less per weight, one fp32 scale per row more
+    assert sizes[2] - sizes[3] == lin // 2 + 3 * 4 * (768 + 256 + 1280 + 256) - 3 * 2 * (768 * 2 + 256 * 2 + 1280 * 2 + 256 * 5)
+
+
+def test_converted_checkpoint_rejections():
+    cfg = Config.make(dim=256, hidden=640, heads=2, hd=128, seq=64, nlayers=2, vocab=320)
+
+    def msg(data):
+        with pytest.raises(engine.CheckpointError) as e:
+            engine.parse_packed_checkpoint(data)
+        return str(e.value)
+
+    good, _ = _packed_bytes(cfg, 1)
+    assert msg(good[:40]) == "converted checkpoint too small for header"
+    assert msg(b"RSTK" + good[4:]) == "bad converted checkpoint magic"
+    assert msg(_packed_bytes(cfg, 1, version=2)[0]) == "unsupported converted checkpoint version 2"
+    bad = bytearray(good); bad[12:16] = np.uint32(9).tobytes()
+    assert msg(bytes(bad)) == "unknown weight format 9 in converted checkpoint"
+    bad = bytearray(good); bad[16:20] = np.uint32(5).tobytes()
+    assert msg(bytes(bad)) == "unknown ffn activation 5 in converted checkpoint"
+    bad = bytearray(good); bad[20:24] = np.uint32(0).tobytes()
+    assert msg(bytes(bad)) == "converted checkpoint header describes no model"
+    assert "does not match its header" in msg(good + b"\0")
+    assert "does not match its header" in msg(good[:-4])
+    # a shape the weight format cannot hold (4-bit groups of 128 along every reduction axis)
+    odd = bytearray(good); odd[12:16] = np.uint32(3).tobytes(); odd[24:28] = np.uint32(704).tobytes()
+    assert "multiples of the weight load width" in msg(bytes(odd))
+
+
+def _generate(*args):
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    return subprocess.run([os.path.join(root, "rustane_amd", "lib", "generate")] + [str(a) for a in args],
+                          capture_output=True, text=True, timeout=120)
+
+
+def _ids(stdout, key="generated_ids="):
+    return [ln[len(key):] for ln in stdout.splitlines() if ln.startswith(key)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("wdt,code", [("f32", 0), ("bf16", 1), ("fp8", 2), ("int4", 3)])
+def test_converted_checkpoint_generates_what_the_fp32_file_generates(tmp_path, wdt, code):
+    # offline conversion: generate --convert-to writes the weights as the device stores them for one format;
+    # a model created from that file (plain copies, no conversion) must give the very tokens of a model
+    # converted from the fp32 file at creation -- greedy and sampled
+    cfg = Config.make(dim=256, hidden=640, heads=2, hd=128, seq=96, nlayers=3, vocab=320)
+    w = synth.make_weights(cfg, seed=12, std=0.08, round_bf16=False)
+    src, dst = tmp_path / "ckpt_000009.bin", tmp_path / "ckpt_000009.rstq"
+    engine.write_checkpoint(src, cfg, w, step=9)
+    p = _generate("--checkpoint", src, "--weight-dtype", wdt, "--convert-to", dst)
+    assert p.returncode == 0, p.stderr
+    assert p.stdout.splitlines()[-1] == "converted_checkpoint=%s weight_dtype=%s step=9" % (dst, wdt)
+    data = dst.read_bytes()
+    got, step, dt = engine.parse_packed_checkpoint(data)
+    assert (step, dt, got["dim"], got["hidden"], got["nlayers"], got["vocab"]) == (9, code, 256, 640, 3, 320)
+    assert len(data) == len(_packed_bytes(cfg, code)[0])
+    common = ["--prompt-ids", "3,1,4,1,5,9,2,6,5,3,5", "--decode-backend", "hip", "--kv-dtype", "bf16"]
+    for extra in (["--steps", "12"], ["--steps", "10", "--temperature", "0.8", "--top-k", "6", "--samples", "3", "--seed", "5"]):
+        a = _generate("--checkpoint", src, "--weight-dtype", wdt, *common, *extra)
+        b = _generate("--checkpoint", dst, *common, *extra)                    # (the file names its weight format)
+        assert a.returncode == 0 and b.returncode == 0, a.stderr + b.stderr
+        key = "generated_ids=" if "--samples" not in extra else "sample"
+        ia = [ln for ln in a.stdout.splitlines() if ln.startswith(key) and "_ids=" in ln]
+        ib = [ln for ln in b.stdout.splitlines() if ln.startswith(key) and "_ids=" in ln]
+        assert ia and ia == ib
+        assert "loaded checkpoint: step=9 model=3L 256D 640H 320V seq=96" in b.stdout
+    # the format is the file's: naming another one is refused, and a converted file is not converted again
+    bad = _generate("--checkpoint", dst, "--weight-dtype", "bf16" if wdt != "bf16" else "int4", *common)
+    assert bad.returncode == 2 and "does not match the format this converted checkpoint holds" in bad.stderr
+    again = _generate("--checkpoint", dst, "--convert-to", tmp_path / "x.rstq")
+    assert again.returncode == 2 and "converted already" in again.stderr

@@ -352,3 +352,31 @@ def test_streams_and_chat(tmp_path):
     finally:
         srv.close()
         cache.close()
+
+
+@pytest.mark.gpu
+def test_server_over_a_converted_checkpoint(tmp_path):
+    # the server loads a checkpoint converted ahead of time (4-bit weights as the device stores them) with no flag
+    # naming the format; its answers are those of a cache built from the fp32 arrays in that format
+    cfg = Config.make(dim=256, hidden=640, heads=2, hd=128, seq=96, nlayers=2, vocab=320)
+    w = synth.make_weights(cfg, seed=14, std=0.08, round_bf16=False)
+    src, dst = tmp_path / "ckpt_000002.bin", tmp_path / "ckpt_000002.rstq"
+    engine.write_checkpoint(src, cfg, w, step=2)
+    gen = os.path.join(ROOT, "rustane_amd", "lib", "generate")
+    p = subprocess.run([gen, "--checkpoint", str(src), "--weight-dtype", "int4", "--convert-to", str(dst)],
+                       capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0, p.stderr
+    srv = Server(["--checkpoint", str(dst), "--decode-backend", "hip"])
+    cache = engine.SessionCache(cfg, w, max_entries=4, weight_dtype=3, kv_dtype=0)
+    try:
+        prompt = [7, 8, 9, 10, 11, 12]
+        for body, req in (({"prompt_ids": prompt, "max_tokens": 9}, engine.GenerationRequest(HIP, steps=9)),
+                          ({"prompt_ids": prompt + [1, 2], "max_tokens": 6, "temperature": 0.7, "top_k": 5, "seed": 3},
+                           engine.GenerationRequest(HIP, steps=6, temperature=0.7, top_k=5, seed=3))):
+            status, _, _, got = srv.request("POST", "/v1/completions", body)
+            assert status == 200, got
+            want = cache.generate(body["prompt_ids"], req).batch.results[0]
+            assert got["choices"][0]["generated_ids"] == list(map(int, want.sampled))
+    finally:
+        srv.close()
+        cache.close()
