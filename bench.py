@@ -98,7 +98,7 @@ def run_c3(args, workload, cfg, weights, n_prompt):
     }
 
 
-def cpu_baseline(cfg, weights, kv_bf16, prompt=None, gpu_stream=None, budget_s=20.0, max_steps=64):
+def cpu_baseline(cfg, weights, kv_bf16, prompt=None, gpu_stream=None, budget_s=20.0, max_steps=64, naive_steps=-1):
     """Times the oracle's KV-cached greedy loop (the CPU restatement of the reference's arithmetic) on
     this box's host cores.  With a prompt (the small workloads) the oracle replays the workload itself
     -- window forward over the prompt, then greedy steps -- and its tokens are compared with the
@@ -131,6 +131,22 @@ def cpu_baseline(cfg, weights, kv_bf16, prompt=None, gpu_stream=None, budget_s=2
     out = {"value": n / dt, "unit": "tok/s", "cores": cores, "kind": "port",
            "sample": "%d KV-cached greedy steps of the same model %s, fp32 CPU oracle" % (n, what)}
     out.update(extra)
+    steps = 0
+    if prompt is not None:
+        # the reference's other decode mode on the same cores: every token is a forward pass over the whole
+        # cfg.seq window from position 0 (crates/engine/src/inference.rs:650-700).  All 32 steps of the tiny
+        # workload, one of the 600M one (~3 TFLOP: 13 s on the 16 host cores of the GPU box) unless --cpu-naive-steps
+        # says otherwise.
+        steps = naive_steps if naive_steps >= 0 else (32 if cfg.nlayers * cfg.dim <= 8192 else 1)
+    if prompt is not None and steps > 0:
+        window = np.resize(np.asarray(prompt, np.uint32), cfg.seq)
+        naive = O.Oracle(cfg, weights, kv_round_bf16=kv_bf16)
+        t1 = time.perf_counter()
+        for _ in range(steps):
+            naive.forward_window(window)
+        dn = time.perf_counter() - t1
+        out["naive_full_context"] = {"value": steps / dn, "unit": "tok/s",
+                                     "sample": "%d whole-window (%d positions) forward passes of the same oracle" % (steps, cfg.seq)}
     return out
 
 
@@ -306,7 +322,7 @@ def measure(args, workload, with_cpu_baseline):
     if with_cpu_baseline:
         replay = workload in ("c1_tiny_fp32", "c2_600m_bf16_bs1")      # the oracle can afford the prompt here
         out["cpu_baseline"] = cpu_baseline(cfg, weights, kvdt == KvDtype.BF16, prompt if replay else None,
-                                           gpu_stream if replay else None)
+                                           gpu_stream if replay else None, naive_steps=args.cpu_naive_steps)
     return out
 
 
@@ -335,6 +351,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-all-configs", action="store_true",
                     help="only the selected workload (by default the line also carries a short run of every other one)")
+    ap.add_argument("--cpu-naive-steps", type=int, default=-1, metavar="N",
+                    help="whole-window forward passes of the CPU oracle to time beside its KV-cached loop "
+                         "(default: 32 for the tiny workload, 1 for the 600M one)")
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="also run 4 launches of a plain copy kernel of this size (for scaling traffic counters)")
