@@ -86,7 +86,7 @@ int main(int argc, char **argv) {
         else if (a == "--decode-backend") {
             std::string raw = val();
             if (!parse_decode_backend(raw, &req.decode_backend))
-                fail("--decode-backend must be one of: auto, naive, hip; got " + raw);
+                fail(decode_backend_error("--decode-backend", raw));
         } else if (a == "--help" || a == "-h") { usage(); return 0; }
         else if (a == "--prompt" || a == "--tokenizer" || a == "--add-special-tokens" || a == "--no-skip-special-tokens")
             // generate.rs:173-188: text goes through the tokenizers crate there; this engine works on ids

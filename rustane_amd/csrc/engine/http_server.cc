@@ -328,7 +328,7 @@ bool build_generation_request(const CompletionRequest &req, DecodeBackendRequest
     GenerationRequest g;
     g.decode_backend = default_backend;
     if (req.has_decode_backend && !parse_decode_backend(req.decode_backend, &g.decode_backend)) {      // serve.rs:574-583
-        *err = "decode_backend must be one of: auto, naive, hip; got " + req.decode_backend;
+        *err = decode_backend_error("decode_backend", req.decode_backend);
         return false;
     }
     g.steps = req.has_max_tokens ? req.max_tokens : 32;

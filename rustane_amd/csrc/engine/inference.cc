@@ -35,9 +35,14 @@ size_t argmax_last(const float *x, size_t n) {
 bool parse_decode_backend(const std::string &raw, DecodeBackendRequest *out) {
     if (raw == "auto") *out = DecodeBackendRequest::Auto;
     else if (raw == "naive") *out = DecodeBackendRequest::Naive;
-    else if (raw == "hip" || raw == "metal") *out = DecodeBackendRequest::Hip;
+    else if (raw == "hip") *out = DecodeBackendRequest::Hip;
     else return false;
     return true;
+}
+std::string decode_backend_error(const std::string &what, const std::string &raw) {
+    if (raw == "metal")
+        return what + " metal is the Apple-GPU backend, which this build does not have: use hip for the KV-cache path on the AMD GPU";
+    return what + " must be one of: auto, naive, hip; got " + raw;
 }
 const char *decode_backend_str(DecodeBackendRequest r) {
     switch (r) {

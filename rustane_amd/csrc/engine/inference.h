@@ -16,10 +16,13 @@ namespace rustane {
 
 constexpr size_t AUTO_KV_PARAM_THRESHOLD = 20000000;   // inference.rs:9 AUTO_METAL_PARAM_THRESHOLD
 
-// inference.rs:11-35 (Hip beside Auto / Naive; "metal" names the reference's own GPU backend and
-// is accepted by parse() as a request for the GPU KV-cache path of this build)
+// inference.rs:11-35, with Hip beside Auto / Naive.  "metal" stays the name of the reference's Apple-GPU
+// backend: this build has none, so parse() refuses it and decode_backend_error() says so by name
+// instead of treating it as another spelling of "hip".
 enum class DecodeBackendRequest { Auto, Naive, Hip };
 bool parse_decode_backend(const std::string &raw, DecodeBackendRequest *out);
+// The message for a value parse_decode_backend() refused; `what` names the flag or field.
+std::string decode_backend_error(const std::string &what, const std::string &raw);
 const char *decode_backend_str(DecodeBackendRequest r);
 
 // inference.rs:37-52

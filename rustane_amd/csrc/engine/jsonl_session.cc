@@ -94,7 +94,7 @@ bool jsonl_to_generation_request(const JsonlRequest &r, const GenerationRequest 
                                  std::string *err) {
     *out = defaults;
     if (r.has_decode_backend && !parse_decode_backend(r.decode_backend, &out->decode_backend)) {
-        *err = "decode_backend must be one of: auto, naive, hip; got " + r.decode_backend;
+        *err = decode_backend_error("decode_backend", r.decode_backend);
         return false;
     }
     if (r.has_samples) out->samples = r.samples;

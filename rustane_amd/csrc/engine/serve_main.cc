@@ -47,7 +47,7 @@ int main(int argc, char **argv) {
         else if (a == "--model-name") model_name = val();
         else if (a == "--decode-backend") {
             const std::string raw = val();
-            if (!parse_decode_backend(raw, &backend)) fail("--decode-backend must be one of: auto, naive, hip");
+            if (!parse_decode_backend(raw, &backend)) fail(decode_backend_error("--decode-backend", raw));
         } else if (a == "--softcap") softcap = strtof(val().c_str(), nullptr);
         else if (a == "--max-cache-sessions") max_cache_sessions = count("an integer");
         else if (a == "--weight-dtype") { wdt = val(); wdt_given = true; }

@@ -75,7 +75,7 @@ def test_parse_decode_backend():
     assert E.parse_decode_backend("auto") == E.DecodeBackendRequest.AUTO
     assert E.parse_decode_backend("naive") == E.DecodeBackendRequest.NAIVE
     assert E.parse_decode_backend("hip") == E.DecodeBackendRequest.HIP
-    assert E.parse_decode_backend("metal") == E.DecodeBackendRequest.HIP
+    assert E.parse_decode_backend("metal") is None          # the Apple-GPU backend is not an alias of hip
     assert E.parse_decode_backend("cuda") is None
 
 

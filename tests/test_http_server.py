@@ -104,6 +104,7 @@ def test_completion_rejections():
     assert msg('{"prompt_ids":[3,8192]}')[0] == "prompt token id 8192 at position 1 exceeds model vocab 8192"
     assert msg('{"prompt_ids":[1],"n":0}')[0] == "n must be >= 1"
     assert msg('{"prompt_ids":[1],"decode_backend":"cuda"}')[0] == "decode_backend must be one of: auto, naive, hip; got cuda"
+    assert msg('{"prompt_ids":[1],"decode_backend":"metal"}')[0].startswith("decode_backend metal is the Apple-GPU backend")
     # the model is checked before the prompt, the prompt before the generation fields (serve.rs:662-691)
     assert msg('{"model":"other","n":0}')[0].startswith("requested model")
     assert msg('{"n":0}')[0] == "one of prompt or prompt_ids is required"

@@ -44,6 +44,7 @@ def test_request_rejections():
     assert msg('{"append_prompt_ids":[1,4294967296]}').startswith("invalid json request: ")
     assert msg('{"steps":3} trailing').startswith("invalid json request: ")
     assert msg('{"decode_backend":"cuda"}') == "decode_backend must be one of: auto, naive, hip; got cuda"
+    assert msg('{"decode_backend":"metal"}').startswith("decode_backend metal is the Apple-GPU backend")
     assert msg('{"samples":0}') == "samples must be >= 1"
     assert msg('{"append_prompt_ids":[1],"append_prompt":"x"}') == "pass either append_prompt_ids or append_prompt, not both"
     assert msg('{"append_prompt":"hello"}') == "append_prompt requires the session to be started with --tokenizer"
