@@ -172,6 +172,10 @@ int hipdec_batch_begin(hipdec_model *m, size_t n_rows);
 int hipdec_batch_end(hipdec_model *m);
 /* steps taken since hipdec_batch_begin (each row is at position len + steps) */
 int hipdec_batch_steps(const hipdec_model *m, size_t *out_steps);
+/* Diagnostic, no counterpart in the reference: *out = 1 when the open batch runs the layers of a step as
+ * one persistent launch (bf16 weights, at most 8 rows, dimensions that are multiples of 256 within the
+ * kernel's register budget), 0 when it runs one kernel per product. */
+int hipdec_batch_layers_in_one_launch(const hipdec_model *m, int *out);
 /* tokens[n_rows]; out_logits[n_rows][vocab]  (hipdec_decode_logits_from_id per row) */
 int hipdec_decode_logits_from_ids_batch(hipdec_model *m, const uint32_t *tokens, float softcap, float *out_logits);
 /* tokens[n_rows] -> out_tokens[n_rows]  (Model::decode_token_argmax_from_id per row, lib.rs:340-375) */
@@ -264,6 +268,12 @@ int hipdec_export_weight(hipdec_model *m, size_t layer_idx, uint32_t which, floa
 /* Diagnostic: runs one greedy step with the persistent step kernel and returns the wall-clock stamps
  * (100 MHz ticks) workgroup 0 took at its phase boundaries: (nlayers + 1) * 32 slots, unused ones 0. */
 int hipdec_debug_step_profile(hipdec_model *m, uint32_t token, uint64_t *out, size_t cap, size_t *out_count);
+
+/* Diagnostic: one step of the open batch (tokens[n_rows], as hipdec_decode_token_argmax_from_ids_batch without
+ * the tokens) with the build of the one-launch layer kernel that takes time stamps: 16 slots per layer of
+ * workgroup 0's wall clock (100 MHz ticks) at its phase boundaries, (nlayers + 1) * 16 values, unused ones 0.
+ * HIPDEC_ERR_UNSUPPORTED when hipdec_batch_layers_in_one_launch says 0. */
+int hipdec_debug_batch_step_profile(hipdec_model *m, const uint32_t *tokens, uint64_t *out, size_t cap, size_t *out_count);
 
 /* Diagnostic: `reps` launches of a plain device-to-device copy kernel (k_calib_copy) of `bytes` bytes,
  * the known-size yardstick that hardware memory-traffic counters are scaled by. */

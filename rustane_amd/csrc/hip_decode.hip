@@ -4,6 +4,7 @@
 #include "hipdec_mega.h"
 #include "hipdec_prefill.h"
 #include "hipdec_batch.h"
+#include "hipdec_rows.h"
 #include "hipdec_sample.h"
 
 #include <math.h>
@@ -66,6 +67,18 @@ struct BatchState {
     uint32_t *d_ring = nullptr, *h_ring = nullptr;   // tokens of a sampled run, [steps][rows]; h_ring pinned
     size_t ring_elems = 0;
     int graph_rows = 0;
+    // the layers of a step as one persistent launch (hipdec_rows.h), where the model and the row count fit
+    bool rows_ready = false;             // buffers below exist and the kernel accepted its LDS size
+    bool rows_off = false;               // a wait timed out: the step keeps to one kernel per product from then on
+    bool rows_active = false;            // the open batch uses it
+    RowsArgs rows_args{};
+    void *rows_slab = nullptr;           // uncached exchange buffers (uncached_take), sized for ROWS_MAX_R rows
+    size_t rows_slab_cap = 0, rows_slab_bytes = 0;
+    unsigned *rows_epochs = nullptr;
+    float *rows_xb = nullptr;            // per-XCD copies of the exchanged vectors (ordinary memory)
+    size_t rows_xb_bytes = 0;
+    void **rows_suf = nullptr;           // device table [2][L] of the suffix caches
+    const void *rows_suf_seen = nullptr; // first suffix cache the table was written for
 };
 
 }  // namespace
@@ -783,6 +796,111 @@ int batch_alloc(hipdec_model *m, int rows) {
     return HIPDEC_OK;
 }
 
+// ---- the layers of a multi-row step as one persistent launch (hipdec_rows.h)
+bool rows_kernel_fits(const hipdec_model *m, int R) {
+    const hipdec_config &c = m->cfg;
+    if (!m->mega_ok || m->bt.rows_off || m->wt != WT_BF16 || R > ROWS_MAX_R) return false;
+    if (m->opt.flags & HIPDEC_FLAG_NO_MEGA) return false;
+    if (const char *v = getenv("HIPDEC_NO_ROWS_KERNEL")) if (v[0] == '1') return false;
+    const int G = m->mega_grid;
+    const long D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden, N = Q + 2 * KV;
+    if (D % 256 || Q % 256 || H % 256 || N % 2) return false;
+    if (D / 256 > ROWS_JA || Q / 256 > ROWS_JB || H / 256 > ROWS_JB || G % 4) return false;
+    auto band = [&](long rows) { return 2 * ((rows / 2 + G - 1) / G); };          // widest band of a product with `rows` rows
+    if (band(N) > 16 * ROWS_TA || band(2 * H) > 16 * ROWS_TA || band(D) > 16 * ROWS_TB) return false;
+    if (std::max(std::max(N * D, 2 * H * D), std::max(D * Q, D * H)) * 2 >= (1L << 31) - 65536) return false;   // descriptors and 32-bit offsets
+    if ((long)R * c.heads > G) return false;
+    if (c.hd != 64 && c.hd != 128) return false;
+    return rows_lds(ROWS_MAX_R, (int)D, (int)Q, (int)KV, (int)H, (int)c.nlayers, (int)c.hd, G).total <= 160 * 1024;
+}
+
+int rows_prepare(hipdec_model *m, int R) {
+    const hipdec_config &c = m->cfg;
+    BatchState &b = m->bt;
+    b.rows_active = false;
+    if (!rows_kernel_fits(m, R)) return HIPDEC_OK;
+    const int G = m->mega_grid;
+    const size_t D = c.dim, Q = c.q_dim, KV = c.kv_dim, H = c.hidden, REC = c.hd + MEGA_PREC;
+    if (!b.rows_ready) {
+        const int ns_cap = G;                                     // one row, one head: every workgroup a split
+        const size_t xb[6] = {ROWS_MAX_R * D * 4, ROWS_MAX_R * D * 4, ROWS_MAX_R * (Q + 2 * KV) * 4, ROWS_MAX_R * H * 4,
+                              (size_t)ns_cap * REC * 4, (size_t)G * 4};
+        size_t xoff[6], total = 0;
+        for (int i = 0; i < 6; ++i) { xoff[i] = total; total += (xb[i] + 255) & ~(size_t)255; }
+        b.rows_slab = uncached_take(m->opt.device, total, &b.rows_slab_cap);
+        if (!b.rows_slab) return HIPDEC_OK;                        // no uncached memory: the step stays as it is
+        b.rows_slab_bytes = total;
+        char *base = (char *)b.rows_slab;
+        RowsArgs &a = b.rows_args;
+        a.X = (float *)(base + xoff[0]); a.X2 = (float *)(base + xoff[1]); a.QKV = (float *)(base + xoff[2]);
+        a.GATE = (float *)(base + xoff[3]); a.PART = (float *)(base + xoff[4]); a.XT = (unsigned *)(base + xoff[5]);
+        int rc;
+        {
+            // the XCDs' own copies of X, X2, GATE and the folded attention output
+            const size_t cf[4] = {xb[0] / 4, xb[1] / 4, xb[3] / 4, ROWS_MAX_R * Q};
+            size_t off[4], stride = 0;
+            for (int i = 0; i < 4; ++i) { off[i] = stride; stride += (cf[i] + 63) & ~(size_t)63; }
+            b.rows_xb_bytes = (size_t)ROWS_XCD_COPIES * stride * 4;
+            if ((rc = dalloc(m, &b.rows_xb, b.rows_xb_bytes))) return rc;
+            a.XB = b.rows_xb; a.xb_stride = (int)stride; a.xb_copies = ROWS_XCD_COPIES;
+            a.xb_x = (int)off[0]; a.xb_x2 = (int)off[1]; a.xb_gate = (int)off[2]; a.xb_att = (int)off[3];
+        }
+        if ((rc = dalloc(m, &b.rows_epochs, 16))) return rc;
+        if ((rc = dalloc(m, &b.rows_suf, (size_t)2 * c.nlayers * sizeof(void *)))) return rc;
+        a.layers = m->mega.layers; a.gfinal = m->gfinal; a.rope_cos = m->rope_cos; a.rope_sin = m->rope_sin;
+        a.kc_suf = b.rows_suf; a.vc_suf = b.rows_suf + c.nlayers;
+        a.bp = b.d_bp; a.epochs = b.rows_epochs;
+        a.D = (int)D; a.Q = (int)Q; a.KV = (int)KV; a.H = (int)H; a.L = (int)c.nlayers; a.heads = (int)c.heads;
+        a.gqa = c.gqa_ratio ? (int)c.gqa_ratio : 1; a.act = (int)m->opt.ffn_activation; a.alpha = m->alpha;
+        const int lds_max = rows_lds(ROWS_MAX_R, a.D, a.Q, a.KV, a.H, a.L, (int)c.hd, G).total;
+        hipError_t e;
+#define ROWS_ATTR(KVB, HD)                                                                                          \
+    do {                                                                                                            \
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_rows<KVB, HD, MEGA_VAR_PLAIN>),                   \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_max);                               \
+        if (e == hipSuccess)                                                                                        \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_rows<KVB, HD, MEGA_VAR_STAMPS>),              \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds_max);                           \
+    } while (0)
+        if (m->kvbf16) { if (c.hd == 64) ROWS_ATTR(1, 64); else ROWS_ATTR(1, 128); }
+        else { if (c.hd == 64) ROWS_ATTR(0, 64); else ROWS_ATTR(0, 128); }
+#undef ROWS_ATTR
+        if (e != hipSuccess) { (void)hipGetLastError(); b.rows_off = true; return HIPDEC_OK; }
+        b.rows_ready = true;
+    }
+    RowsArgs &a = b.rows_args;
+    if (b.rows_suf_seen != b.kc_suf[0]) {                         // (the suffix caches are reallocated when the row capacity grows)
+        std::vector<void *> t(2 * c.nlayers);
+        for (uint32_t l = 0; l < c.nlayers; ++l) { t[l] = b.kc_suf[l]; t[c.nlayers + l] = b.vc_suf[l]; }
+        HCHK(hipStreamSynchronize(m->stream));
+        HCHK(hipMemcpy(b.rows_suf, t.data(), t.size() * sizeof(void *), hipMemcpyHostToDevice));
+        b.rows_suf_seen = b.kc_suf[0];
+    }
+    // A batch starts from exchange buffers without stamps and from epoch 0 (layer 0 then expects stamp 1):
+    // the row count may differ from the last batch's, and rows it did not have would carry stamps of unknown age.
+    HCHK(hipMemsetAsync(b.rows_slab, 0, b.rows_slab_bytes, m->stream));
+    HCHK(hipMemsetAsync(b.rows_xb, 0, b.rows_xb_bytes, m->stream));
+    HCHK(hipMemsetAsync(b.rows_epochs, 0, 16, m->stream));
+    a.R = R;
+    a.ns_max = std::max(1, std::min(G / (R * (int)c.heads), 64));
+    a.suf_rows = b.suf_rows;
+    b.rows_active = true;
+    return HIPDEC_OK;
+}
+
+// after a wait for the stream: a persistent multi-row launch that gave up leaves the abort flag set
+int rows_check(hipdec_model *m) {
+    BatchState &b = m->bt;
+    if (!b.rows_active) return HIPDEC_OK;
+    unsigned flag = 0;
+    HCHK(hipMemcpy(&flag, b.rows_epochs + 2, 4, hipMemcpyDeviceToHost));
+    if (!flag) return HIPDEC_OK;
+    b.rows_off = true;
+    b.rows_active = false;
+    for (auto &g : b.graphs) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
+    return fail(m, HIPDEC_ERR_HIP, "multi-row step kernel: a wait timed out (the batch has to be reopened; later steps use one kernel per product)");
+}
+
 void batch_enqueue(hipdec_model *m, int variant);
 
 // Everything that changes from step to step (tokens, position, sampler parameters) lives in device
@@ -850,7 +968,21 @@ void batch_enqueue(hipdec_model *m, int variant) {
     pf_launch_embed(m, R);
     const int nch = (D + PF_CHUNK - 1) / PF_CHUNK;
     const bool fp8 = m->wt == WT_FP8;
-    for (uint32_t l = 0; l < c.nlayers; ++l) {
+    if (b.rows_active) {
+        RowsArgs a = b.rows_args;
+        a.x_in = w.x; a.out_hi = w.xn_hi; a.out_lo = w.xn_lo; a.out_ssq = w.ssq;
+        const size_t lds = (size_t)rows_lds(R, D, Q, KV, H, (int)c.nlayers, (int)c.hd, m->mega_grid).total;
+        dim3 grid(m->mega_grid), block(ROWS_THREADS);
+#define ROWS_GO(KVB, HD)                                                                                            \
+    do {                                                                                                            \
+        if (a.prof) hipLaunchKernelGGL((k_rows<KVB, HD, MEGA_VAR_STAMPS>), grid, block, lds, m->stream, a);         \
+        else hipLaunchKernelGGL((k_rows<KVB, HD, MEGA_VAR_PLAIN>), grid, block, lds, m->stream, a);                 \
+    } while (0)
+        if (m->kvbf16) { if (c.hd == 64) ROWS_GO(1, 64); else ROWS_GO(1, 128); }
+        else { if (c.hd == 64) ROWS_GO(0, 64); else ROWS_GO(0, 128); }
+#undef ROWS_GO
+    }
+    for (uint32_t l = 0; l < (b.rows_active ? 0u : c.nlayers); ++l) {
         const DevLayer &L = m->layers[l];
         const int N = Q + 2 * KV;
         int sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.wqkv, L.s_qkv, R, N, D);
@@ -912,6 +1044,8 @@ int batch_fetch(hipdec_model *m, const void *dev, void *host, size_t floats) {
     if (floats > b.h_stage_floats) return fail(m, HIPDEC_ERR_ARG, "internal: staging buffer too small");
     HCHK(hipMemcpyAsync(b.h_stage, dev, floats * 4, hipMemcpyDeviceToHost, m->stream));
     HCHK(hipStreamSynchronize(m->stream));
+    int rc = rows_check(m);
+    if (rc) return rc;
     HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
     memcpy(host, b.h_stage, floats * 4);
     return HIPDEC_OK;
@@ -1029,6 +1163,7 @@ int batch_sampled_run(hipdec_model *m, int variant, const uint32_t *tokens, uint
     HCHK(hipMemcpyAsync(b.h_ring, b.d_ring, (size_t)R * n_steps * 4, hipMemcpyDeviceToHost, m->stream));
     HCHK(hipMemcpyAsync(m->h_samp->rng, m->d_rng, (size_t)R * sizeof(uint64_t), hipMemcpyDeviceToHost, m->stream));
     HCHK(hipStreamSynchronize(m->stream));
+    if ((rc = rows_check(m))) return rc;
     HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
     memcpy(out_tokens, b.h_ring, (size_t)R * n_steps * 4);
     memcpy(rng_states, m->h_samp->rng, (size_t)R * sizeof(uint64_t));
@@ -1077,6 +1212,7 @@ void hipdec_destroy(hipdec_model *m) {
     for (auto &g : m->bt.graphs) if (g) (void)hipGraphExecDestroy(g);
     for (void *p : m->allocs) (void)hipFree(p);
     if (m->xslab) uncached_give(m->opt.device, m->xslab_cap, m->xslab);
+    if (m->bt.rows_slab) uncached_give(m->opt.device, m->bt.rows_slab_cap, m->bt.rows_slab);
     if (m->h_sp) (void)hipHostFree(m->h_sp);
     if (m->h_out) (void)hipHostFree(m->h_out);
     if (m->pf.h_ids) (void)hipHostFree(m->pf.h_ids);
@@ -1731,6 +1867,10 @@ int hipdec_batch_begin(hipdec_model *m, size_t n_rows) {
     if (m->len >= m->cfg.seq) return fail(m, HIPDEC_ERR_FULL, "decode only supports lengths within cfg.seq");
     int rc = batch_alloc(m, (int)n_rows);
     if (rc) return rc;
+    const bool was_active = m->bt.rows_active;
+    if ((rc = rows_prepare(m, (int)n_rows))) return rc;
+    if (was_active != m->bt.rows_active)                              // the captured steps hold the other form
+        for (auto &g : m->bt.graphs) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
     m->bt.rows = (int)n_rows;
     m->bt.prefix = m->len;
     m->bt.slot = 0;
@@ -1742,6 +1882,12 @@ int hipdec_batch_end(hipdec_model *m) {
     if (!m) return HIPDEC_ERR_ARG;
     m->bt.rows = 0;
     m->bt.have_logits = false;
+    return HIPDEC_OK;
+}
+
+int hipdec_batch_layers_in_one_launch(const hipdec_model *m, int *out) {
+    if (!m || !out) return HIPDEC_ERR_ARG;
+    *out = (m->bt.rows && m->bt.rows_active) ? 1 : 0;
     return HIPDEC_OK;
 }
 
@@ -2100,6 +2246,33 @@ int hipdec_debug_step_profile(hipdec_model *m, uint32_t token, uint64_t *out, si
     if (rc) return rc;
     if (out_count) *out_count = n;
     m->len += 1;
+    return HIPDEC_OK;
+}
+
+int hipdec_debug_batch_step_profile(hipdec_model *m, const uint32_t *tokens, uint64_t *out, size_t cap, size_t *out_count) {
+    if (!m) return HIPDEC_ERR_ARG;
+    BatchState &b = m->bt;
+    if (b.rows <= 0 || !b.rows_active) return fail(m, HIPDEC_ERR_UNSUPPORTED, "the open batch does not run its layers as one launch");
+    const size_t n = (size_t)(m->cfg.nlayers + 1) * ROWS_PROF_SLOTS;
+    if (!out || cap < n) return fail(m, HIPDEC_ERR_ARG, "profile buffer too small");
+    unsigned long long *d = nullptr;
+    HCHK(hipMalloc((void **)&d, n * 8));
+    HCHK(hipMemset(d, 0, n * 8));
+    const uint32_t saved = m->opt.flags;
+    m->opt.flags |= HIPDEC_FLAG_NO_GRAPH;                    // (a captured step holds the plain build)
+    b.rows_args.prof = d;
+    int rc = batch_step(m, tokens, B_ARGMAX, 1, 1.0f, 0.0f);
+    b.rows_args.prof = nullptr;
+    m->opt.flags = saved;
+    if (rc == HIPDEC_OK) {
+        hipError_t e = hipStreamSynchronize(m->stream);
+        if (e == hipSuccess) e = hipMemcpy(out, d, n * 8, hipMemcpyDeviceToHost);
+        if (e != hipSuccess) { m->err = hipGetErrorString(e); rc = HIPDEC_ERR_HIP; }
+        if (rc == HIPDEC_OK) rc = rows_check(m);
+    }
+    (void)hipFree(d);
+    if (rc) return rc;
+    if (out_count) *out_count = n;
     return HIPDEC_OK;
 }
 

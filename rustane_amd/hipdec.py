@@ -26,8 +26,8 @@ EXPORTS = [
     "hipdec_decode_token_argmax", "hipdec_decode_token_argmax_from_id", "hipdec_decode_token_topk_from_id",
     "hipdec_decode_token_block_stats_from_id", "hipdec_materialize_current_logits_block",
     "hipdec_decode_logits_from_id", "hipdec_prefill", "hipdec_decode_greedy_run", "hipdec_last_device_ms",
-    "hipdec_bytes_per_token", "hipdec_export_weight", "hipdec_debug_step_profile", "hipdec_debug_calibration_copy",
-    "hipdec_batch_begin", "hipdec_batch_end", "hipdec_batch_steps", "hipdec_decode_logits_from_ids_batch",
+    "hipdec_bytes_per_token", "hipdec_export_weight", "hipdec_debug_step_profile", "hipdec_debug_batch_step_profile", "hipdec_debug_calibration_copy",
+    "hipdec_batch_begin", "hipdec_batch_end", "hipdec_batch_steps", "hipdec_batch_layers_in_one_launch", "hipdec_decode_logits_from_ids_batch",
     "hipdec_decode_token_argmax_from_ids_batch", "hipdec_decode_token_topk_from_ids_batch",
     "hipdec_decode_token_block_stats_from_ids_batch", "hipdec_materialize_current_logits_block_batch",
     "hipdec_decode_topk_sampled_run", "hipdec_decode_fullvocab_sampled_run", "hipdec_decode_topk_sampled_run_batch",
@@ -430,6 +430,21 @@ class HipDecodeModel:
     def batch_end(self):
         self._chk(self._lib.hipdec_batch_end(self._h))
         self._rows = 0
+
+    def batch_layers_in_one_launch(self):
+        v = C.c_int()
+        self._chk(self._lib.hipdec_batch_layers_in_one_launch(self._h, C.byref(v)))
+        return bool(v.value)
+
+    def debug_batch_step_profile(self, tokens):
+        """Time stamps of workgroup 0 for one step of the open batch: array [nlayers + 1][16] of 100 MHz ticks."""
+        t = self._toks(tokens)
+        n = (self.cfg.nlayers + 1) * 16
+        out = np.zeros(n, np.uint64)
+        cnt = C.c_size_t()
+        self._chk(self._lib.hipdec_debug_batch_step_profile(self._h, t.ctypes.data_as(C.POINTER(C.c_uint32)),
+                                                            out.ctypes.data_as(C.POINTER(C.c_uint64)), n, C.byref(cnt)))
+        return out.reshape(self.cfg.nlayers + 1, 16)
 
     def batch_steps(self):
         n = C.c_size_t()
