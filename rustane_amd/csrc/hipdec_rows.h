@@ -39,6 +39,8 @@
 #define ROWS_LPTR 10            // per-layer pointers kept in LDS: w[4], g1, g2, kc, vc, kc_suf, vc_suf
 #define ROWS_OOB 0x7ffffff0     // byte offset past every descriptor
 #define ROWS_PROF_SLOTS 16      // time stamps per layer in the profiling build
+#define ROWS_ATT_PRE 6          // attention: passes of cache rows a thread requests ahead (with R * heads items only a few
+                                // splits are to be had, so an item walks more rows than in the single-row kernel)
 
 enum { RK_QKV = 0, RK_WO = 1, RK_W13 = 2, RK_W2 = 3 };
 
@@ -236,7 +238,7 @@ __global__ __launch_bounds__(ROWS_THREADS, 1) void k_rows(RowsArgs a) {
     constexpr int KEPL = 16 / KESZ;
     constexpr int LPR = HD / KEPL;               // lanes per cache row
     constexpr int SLOTS = ROWS_THREADS / LPR;    // cache rows per pass
-    constexpr int PRE = MEGA_ATT_PRE;
+    constexpr int PRE = ROWS_ATT_PRE;
     constexpr int REC = HD + MEGA_PREC;
     extern __shared__ __align__(16) unsigned char rows_smem[];
     __shared__ RowsKind kinds[4];
@@ -349,11 +351,7 @@ __global__ __launch_bounds__(ROWS_THREADS, 1) void k_rows(RowsArgs a) {
 #pragma unroll
             for (int j = 0; j < JJ; ++j) {
                 if (t * JJ + j >= S0 && t * JJ + j < S1) {
-#ifdef ROWS_NO_WEIGHTS
-                    const bool valid = false;
-#else
                     const bool valid = (16 * t + r16 < nrows) && (j < spw);
-#endif
                     st[t * JJ + j] = rows_ldw(rs, valid ? lane_off + t * 16 * (K * 2) + j * 64 : ROWS_OOB);
                 }
             }
