@@ -133,3 +133,25 @@ def test_rows_kernel_not_taken_where_it_does_not_fit():
         dev.batch_begin(rows)
         assert dev.batch_layers_in_one_launch() == want
         dev.batch_end()
+
+
+@pytest.mark.parametrize("T,k,softcap", [(0.0, 0, 0.0), (0.8, 8, 0.0), (1.0, 0, 2.5), (0.9, 40, 3.0)])
+def test_session_samples_through_the_rows_kernel_equal_the_oracle_loop(T, k, softcap):
+    # The session layer steps the samples of a request together (the reference draws them one after the
+    # other, inference.rs:247-262); on a model the one-launch layers take, every sample's stream, greedy or
+    # drawn on the device, must equal the oracle's cached loop (inference.rs:542-648).
+    from rustane_amd import engine as E
+    cfg = Config.make(dim=256, hidden=512, heads=2, hd=128, seq=64, nlayers=3, vocab=1000)
+    prompt = [5, 6, 7, 8, 9, 10, 11, 12, 13]
+    w = synth.make_weights(cfg, seed=31, std=0.08, round_bf16=True)
+    req = E.GenerationRequest(E.DecodeBackendRequest.HIP, steps=10, temperature=T, top_k=k, samples=5, seed=21)
+    got = E.InferenceSession(cfg, w, prompt, softcap=softcap, weight_dtype=1).generate(req)
+    assert len(got.results) == 5
+    full = np.array(prompt, np.uint32)
+    for i, r in enumerate(got.results):
+        orc = O.Oracle(cfg, w)
+        lg, _, _ = orc.forward_window(full, softcap=softcap)
+        sampled, gen = orc.run_cached_sample(full, lg[0], req.steps, req.temperature, req.top_k, seed=req.seed + i,
+                                             softcap=softcap)
+        np.testing.assert_array_equal(r.sampled, sampled)
+        np.testing.assert_array_equal(r.generated, gen)
