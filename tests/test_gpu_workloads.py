@@ -196,6 +196,7 @@ def test_multi_sample_workload_against_the_recorded_oracle_run():
     rngs = [O.Rng(s0) for s0 in start]
     tf_tok = np.zeros((R, S - 1), np.uint32)
     dev.batch_begin(R)
+    assert dev.batch_layers_in_one_launch()              # this workload's step runs its layers as one persistent launch
     ordered = same_draw = 0
     worst = 0.0
     for i in range(1, S):
