@@ -10,8 +10,11 @@
 //    from LDS as (hi, lo) bf16 pairs (two instructions per weight load, nothing is rounded to 8
 //    bits).  The eight waves split the reduction axis; their 16 x 16 partial tiles meet in LDS;
 //  * a phase's weights are ONE round of loads per wave (at most 12 or 16 loads of 16 bytes per lane,
-//    which is what bounds the model sizes this kernel takes), requested a phase ahead into the
-//    register set the running phase does not use;
+//    which is what bounds the model sizes this kernel takes), requested in two halves, one and two
+//    phases ahead, into the register set the running phase does not use;
+//  * every exchanged vector crosses the fabric once per XCD: the workgroups that share an XCD each
+//    copy a share of it into the XCD's own copy, and everybody polls that copy (rows_relay);
+//  * a layer is two halves of the same shape that run through one copy of the code;
 //  * the staged activation rows are single-buffered (R rows of up to 4096 elements as pairs fill the
 //    LDS), so a phase has two workgroup barriers: inputs staged, partial tiles written;
 //  * attention items are (split, row, head); a row's keys and values are the shared prompt prefix,
@@ -129,7 +132,7 @@ __device__ __forceinline__ bool rows_relay(const float *src, float *dst, int n4,
 // the stamp `par`; stamp bit cleared.  A wave's 64 slots of one pass are one 256-element chunk of a row: with SSQ its sum of
 // squares goes to ssq[r][chunk].
 // Elements [r0, r0 + nres) of every row are also kept raw in res[r][.].  Returns a negative value when
-// the wait was aborted.  Out of line for the reason given at mega_poll_vec.
+// the wait was aborted.
 template <bool GAMMA, bool SSQ>
 __device__ __forceinline__ float rows_poll(const float *src, int R, int n, unsigned par, unsigned *abortf, uint16_t *xh,
                                         uint16_t *xl, int XS, const float *gamma, float *ssq, float *res, int r0, int nres,
