@@ -45,12 +45,13 @@ ALL_CONFIG_STEPS = {"c1_tiny_fp32": 31, "c2_600m_bf16_bs1": 255, "c3_600m_bf16_8
 
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, each
 # scaled by what the same counter reads for a plain copy of known size): measured separately with
-# rocprofv3 --pmc and recorded in profiles/k_mega_c2_600m_bf16_bs1.md and profiles/k_mega_hbm_traffic_c1_c4_c5.md
+# rocprofv3 --pmc and recorded in profiles/k_mega_c2_600m_bf16_bs1.md, profiles/k_mega_hbm_traffic_c1_c4_c5.md and
+# profiles/k_rows_c3_600m_bf16_8samples.md
 # (per step, i.e. the LM-head GEMV included where it is a launch of its own, at the KV length of the
 # profiled run); a benchmark run cannot collect it itself.
 TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries under profiles/, not measured in this run"
-MEASURED_TRAFFIC_BYTES = {"c1_tiny_fp32": 1.267e8, "c2_600m_bf16_bs1": 1.5083e9, "c4_5b_bf16_bs1": 1.3874e10,
-                          "c5_5b_fp8_bs1": 7.118e9, "c5_5b_int4_bs1": 4.008e9}
+MEASURED_TRAFFIC_BYTES = {"c1_tiny_fp32": 1.267e8, "c2_600m_bf16_bs1": 1.5083e9, "c3_600m_bf16_8samples": 1.811e9,
+                          "c4_5b_bf16_bs1": 1.3874e10, "c5_5b_fp8_bs1": 7.118e9, "c5_5b_int4_bs1": 4.008e9}
 
 
 def run_c3(args, workload, cfg, weights, n_prompt):
@@ -91,7 +92,8 @@ def run_c3(args, workload, cfg, weights, n_prompt):
         "prefill_ms": s.prefill_elapsed() * 1e3, "request_wall_ms": wall * 1e3,
         "device_ms_per_step": dev_ms / K,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "bytes_per_step": bytes_per_step},
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(workload),
+                     "traffic_source": TRAFFIC_SOURCE, "bytes_per_step": bytes_per_step},
         "mfma_roofline": {"bound": "mfma", "achieved": flops_per_step * K / (dev_ms * 1e-3) / 1e12, "peak": 2500.0,
                           "unit": "TFLOP/s", "frac": flops_per_step * K / (dev_ms * 1e-3) / 2.5e15},
         "sampled_head": [int(r.sampled[1]) for r in got.results],
