@@ -217,3 +217,27 @@ def test_rows_kernel_at_the_600m_shape_equals_one_kernel_per_product(kvdt, tol):
         toks = a.argmax(axis=1).astype(np.uint32)
         seen.update(int(t) for t in toks)
     assert len(seen) > 20
+
+
+def test_rows_kernel_step_profile_is_a_step_like_any_other():
+    # hipdec_debug_batch_step_profile runs the build with time stamps: the rows advance by one token exactly as
+    # with the plain build, and workgroup 0's stamps come back in order, 16 per layer
+    cfg = Config.make(dim=256, hidden=512, heads=2, hd=128, seq=96, nlayers=3, vocab=320)
+    rows = 4
+    w, dev, orcs, ids = setup(cfg, rows, 20)
+    dev.batch_begin(rows)
+    toks = np.array([3, 50, 101, 299], np.uint32)
+    pr = dev.debug_batch_step_profile(toks).astype(np.int64)
+    assert pr.shape == (cfg.nlayers + 1, 16) and dev.batch_steps() == 1
+    for l in range(cfg.nlayers):
+        assert np.all(pr[l] > 0) and np.all(np.diff(pr[l]) >= 0) and pr[l + 1][0] >= pr[l][15]
+    nxt = []
+    for r in range(rows):
+        nxt.append(O.argmax_lower(orcs[r].decode_logits_from_id(int(toks[r]))))
+    toks = np.array(nxt, np.uint32)
+    got = dev.decode_logits_from_ids_batch(toks)
+    for r in range(rows):
+        assert rel_err(got[r], orcs[r].decode_logits_from_id(int(toks[r]))) < 1e-4
+    dev.batch_end()
+    with pytest.raises(Exception):
+        dev.debug_batch_step_profile(toks)                    # no batch open
