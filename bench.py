@@ -200,6 +200,78 @@ def run_c4_sampled(args, workload, cfg, dev, kvdt, prompt_logits, n_prompt, gen_
     }
 
 
+def per_call_paths(dev, cfg, first, n_prompt, steps, chained_ms):
+    """The three per-token shapes the reference's own decode micro-benchmarks time
+    (crates/engine/tests/bench_decode_input_path.rs:132-235), each `steps` SYNCHRONOUS calls through the
+    C ABI from the end of the prompt: greedy argmax from the token id; per-block top-k candidates (k = 8, the
+    host merge and draw of the reference's loop included); block statistics, the host's block draw, the
+    block's logits and the host's token draw (temperature 0.8).  ms per token, wall clock, preallocated
+    buffers, the calls made straight through ctypes."""
+    import ctypes as C
+    from rustane_amd import engine as E
+    lib, eng, h = dev._lib, E.lib(), dev._h
+    fp, up = C.POINTER(C.c_float), C.POINTER(C.c_uint32)
+    B, K8, T = dev.blocks, 8, 0.8
+    out = {"steps": steps, "chained_device_ms_per_step": chained_ms}
+    tok = C.c_uint32()
+
+    def timed(body):
+        dev.set_len(n_prompt)
+        body(2)                                   # the variant's graph is captured on its first call
+        dev.set_len(n_prompt)
+        t0 = time.perf_counter()
+        body(steps)
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    def greedy(n):
+        cur = first
+        for _ in range(n):
+            rc = lib.hipdec_decode_token_argmax_from_id(h, cur, C.byref(tok))
+            assert rc == 0, rc
+            cur = tok.value
+    out["argmax_from_id_ms"] = timed(greedy)
+
+    vals, idxs = np.empty(B * K8, np.float32), np.empty(B * K8, np.uint32)
+    mv, mi = np.empty(K8, np.float32), np.empty(K8, np.uint32)
+    cnt, rng = C.c_size_t(), C.c_uint64(1)
+    vp, ip, mvp, mip = vals.ctypes.data_as(fp), idxs.ctypes.data_as(up), mv.ctypes.data_as(fp), mi.ctypes.data_as(up)
+    eng.rs_merge_topk_candidates.restype = C.c_uint64
+    eng.rs_merge_topk_candidates.argtypes = [fp, up, C.c_size_t, C.c_size_t, fp, up]
+    eng.rs_sample_topk_candidates.restype = C.c_uint32
+    eng.rs_sample_topk_candidates.argtypes = [up, fp, C.c_size_t, C.c_float, C.POINTER(C.c_uint64)]
+
+    def topk(n):
+        cur = first
+        for _ in range(n):
+            rc = lib.hipdec_decode_token_topk_from_id(h, cur, K8, vp, ip, B * K8, C.byref(cnt))
+            assert rc == 0, rc
+            m = eng.rs_merge_topk_candidates(vp, ip, cnt.value, K8, mvp, mip)
+            cur = eng.rs_sample_topk_candidates(mip, mvp, m, T, C.byref(rng))
+    out["topk8_candidates_from_id_ms"] = timed(topk)
+
+    mx, sm, blk = np.empty(B, np.float32), np.empty(B, np.float32), np.empty(256, np.float32)
+    mxp, smp, bp = mx.ctypes.data_as(fp), sm.ctypes.data_as(fp), blk.ctypes.data_as(fp)
+    valid = C.c_size_t()
+    eng.rs_sample_block_from_stats.restype = C.c_uint64
+    eng.rs_sample_block_from_stats.argtypes = [fp, fp, C.c_size_t, C.POINTER(C.c_uint64)]
+    eng.rs_sample_block_logits.restype = C.c_uint32
+    eng.rs_sample_block_logits.argtypes = [C.c_uint32, fp, C.c_size_t, C.c_float, C.POINTER(C.c_uint64)]
+    inv_t = float(np.float32(1.0) / np.float32(T))
+
+    def stats(n):
+        cur = first
+        for _ in range(n):
+            rc = lib.hipdec_decode_token_block_stats_from_id(h, cur, C.c_float(inv_t), C.c_float(0.0), mxp, smp, B, C.byref(cnt))
+            assert rc == 0, rc
+            b = eng.rs_sample_block_from_stats(mxp, smp, cnt.value, C.byref(rng))
+            rc = lib.hipdec_materialize_current_logits_block(h, b, C.c_float(0.0), bp, 256, C.byref(valid))
+            assert rc == 0, rc
+            cur = eng.rs_sample_block_logits(b * 256, bp, valid.value, T, C.byref(rng))
+    out["block_stats_then_block_from_id_ms"] = timed(stats)
+    dev.set_len(n_prompt)
+    return out
+
+
 _WEIGHTS = {}
 
 
@@ -321,6 +393,8 @@ def measure(args, workload, with_cpu_baseline):
     }
     if prefill_options:
         out["prefill_options"] = prefill_options
+    if workload == "c2_600m_bf16_bs1" and not args.no_per_call:
+        out["per_call"] = per_call_paths(dev, cfg, first, n_prompt, 48, dev_ms / K)
     if with_cpu_baseline:
         replay = workload in ("c1_tiny_fp32", "c2_600m_bf16_bs1")      # the oracle can afford the prompt here
         out["cpu_baseline"] = cpu_baseline(cfg, weights, kvdt == KvDtype.BF16, prompt if replay else None,
@@ -341,6 +415,10 @@ def summary(r):
         e["prefill_options"] = r["prefill_options"]
     if "mfma_roofline" in r:
         e["step_mfma_frac"] = r["mfma_roofline"]["frac"]
+    if "per_call" in r:
+        e["per_call"] = r["per_call"]
+    if "cpu_baseline" in r:
+        e["cpu_baseline"] = r["cpu_baseline"]
     return e
 
 
@@ -351,6 +429,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--workload", default="c2_600m_bf16_bs1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-per-call", action="store_true",
+                    help="skip the synchronous call-per-token figures of the 600M workload")
     ap.add_argument("--no-all-configs", action="store_true",
                     help="only the selected workload (by default the line also carries a short run of every other one)")
     ap.add_argument("--cpu-naive-steps", type=int, default=-1, metavar="N",

@@ -260,34 +260,6 @@ int hipdec_export_packed_head(hipdec_model *m, float *gamma_final, void *embed);
 int hipdec_create_packed(const hipdec_config *cfg, const hipdec_packed_layer *layers, size_t n_layers,
                          const hipdec_packed_head *head, const hipdec_options *opts, hipdec_model **out);
 
-/* Debug/verification: copy one stored weight matrix back as fp32 after de-quantisation, in
- * out-major [rows][k] order.  which: 0 wqkv (rows q_dim+2*kv_dim, k dim), 1 wo (dim, q_dim),
- * 2 w13 (2*hidden interleaved gate/up rows, dim), 3 w2 (dim, hidden), 4 embed (vocab, dim). */
-int hipdec_export_weight(hipdec_model *m, size_t layer_idx, uint32_t which, float *out, size_t cap);
-
-/* Diagnostic: runs one greedy step with the persistent step kernel and returns the wall-clock stamps
- * (100 MHz ticks) workgroup 0 took at its phase boundaries: (nlayers + 1) * 32 slots, unused ones 0. */
-int hipdec_debug_step_profile(hipdec_model *m, uint32_t token, uint64_t *out, size_t cap, size_t *out_count);
-
-/* Diagnostic: one step of the open batch (tokens[n_rows], as hipdec_decode_token_argmax_from_ids_batch without
- * the tokens) with the build of the one-launch layer kernel that takes time stamps: 16 slots per layer of
- * workgroup 0's wall clock (100 MHz ticks) at its phase boundaries, (nlayers + 1) * 16 values, unused ones 0.
- * HIPDEC_ERR_UNSUPPORTED when hipdec_batch_layers_in_one_launch says 0. */
-int hipdec_debug_batch_step_profile(hipdec_model *m, const uint32_t *tokens, uint64_t *out, size_t cap, size_t *out_count);
-
-/* Diagnostic: `reps` launches of a plain device-to-device copy kernel (k_calib_copy) of `bytes` bytes,
- * the known-size yardstick that hardware memory-traffic counters are scaled by. */
-int hipdec_debug_calibration_copy(size_t bytes, int reps);
-
-/* Verification: the draw kernels of the sampled runs on caller-supplied inputs (one row).  top-k: the
- * per-block candidate lists vals/idxs[blocks * top_k] as hipdec_decode_token_topk_from_id returns them
- * (engine/src/decode.rs:218-253 merge, engine/src/inference.rs:823-849 draw); full vocabulary: raw
- * logits[vocab] with their block statistics maxes/sums[ceil(vocab / 256)] (inference.rs:851-921).
- * *rng_state in and out, *out_token = the drawn token. */
-int hipdec_debug_sample_topk(const float *vals, const uint32_t *idxs, size_t blocks, uint32_t top_k, float temperature,
-                             float softcap, uint64_t *rng_state, uint32_t *out_token);
-int hipdec_debug_sample_fullvocab(const float *logits, size_t vocab, const float *maxes, const float *sums,
-                                  float temperature, float softcap, uint64_t *rng_state, uint32_t *out_token);
 /* The full-vocabulary draw for callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.
  * Same draw as hipdec_debug_sample_fullvocab (block from the statistics, then the token inside the
@@ -297,25 +269,12 @@ int hipdec_debug_sample_fullvocab(const float *logits, size_t vocab, const float
  * default stream) without waiting for them.  Calls no hipMalloc / hipFree: the kernels' run state lives
  * in a 256-byte array the library holds on every GPU it runs on, reset by the call itself.  Every call
  * on a GPU shares that array, so calls that overlap on one GPU (two streams, two threads) race.
+ * The library looks the array's address up once per GPU (not a capturable operation): in hipdec_create*,
+ * else in the first call of this entry point on that GPU -- which must then be made outside stream capture.
  * vocab <= 262144 (1024 blocks), else HIPDEC_ERR_ARG; errors are reported through hipdec_last_error(NULL). */
 int hipdec_sample_fullvocab_noalloc(const float *d_logits, size_t vocab, const float *d_maxes, const float *d_sums,
                                     float temperature, float softcap, uint64_t *d_rng_state, uint32_t *d_out_token,
                                     void *stream);
-/* 1 when this host's C library computes expf and tanhf as the on-device sampler reproduces them
- * (the probe the sampled runs consult), else 0. */
-int hipdec_debug_hostmath_probe(void);
-/* Verification of the two host C library functions the on-device sampler restates (fn 0: expf,
- * fn 1: tanhf): evaluate the restatement for n inputs on the host (on_device = 0) or on the GPU; */
-int hipdec_debug_hostmath_eval(int fn, const float *in, float *out, size_t n, int on_device);
-/* an order-independent checksum of its results over `count` consecutive float bit patterns starting
- * at first_bits, computed on the host (with host_threads threads) or on the GPU: equal checksums
- * mean equal results; */
-int hipdec_debug_hostmath_checksum(int fn, uint32_t first_bits, uint64_t count, int on_device, int host_threads,
-                                   uint64_t *out);
-/* and the number of those inputs for which the host evaluation differs from the C library's function. */
-int hipdec_debug_hostmath_count_mismatch(int fn, uint32_t first_bits, uint64_t count, int host_threads,
-                                         uint64_t *out_mismatches);
-
 #ifdef __cplusplus
 }
 #endif

@@ -100,10 +100,29 @@ bool parse_checkpoint(const uint8_t *bytes, size_t len, Checkpoint *out, std::st
     if ((len - cur) % 4 != 0) return bad(err, "checkpoint payload is not aligned to f32 values");
     const size_t payload_floats = (len - cur) / 4;
     if (shape) {
+        // The side file's numbers are not the header's: bound them as the device configuration does (32-bit
+        // fields, head size 64 or 128, whole groups of query heads per key/value head) and size the payload
+        // without wrap-around, so that a damaged side file cannot agree with the payload modulo 2^64.
+        const uint64_t lim = 0xffffffffull;
+        if (shape->heads == 0 || shape->kv_heads == 0 || shape->hidden == 0 || shape->heads > lim || shape->kv_heads > lim ||
+            shape->hidden > lim || (shape->hd != 64 && shape->hd != 128) || shape->heads % shape->kv_heads != 0 ||
+            shape->heads * shape->hd > lim)
+            return bad(err, "checkpoint shape file holds values no model has (heads, kv_heads, hidden within 32 bits; hd 64 or 128; heads a multiple of kv_heads)");
         out->cfg = ModelConfig::make(dim, shape->hidden, shape->heads, shape->kv_heads, shape->hd, seq, nlayers, vocab, act);
         const ModelConfig &sc = out->cfg;
-        const size_t per_layer = sc.dim * sc.q_dim + 2 * sc.dim * sc.kv_dim + sc.q_dim * sc.dim + 3 * sc.dim * sc.hidden + 2 * sc.dim;
-        if (payload_floats != sc.vocab * sc.dim + sc.dim + sc.nlayers * per_layer)
+        size_t per_layer = 0, t = 0, total = 0;
+        bool over = false;
+        auto add_prod = [&](size_t a, size_t b, size_t times) {
+            over |= __builtin_mul_overflow(a, b, &t) || __builtin_mul_overflow(t, times, &t) || __builtin_add_overflow(per_layer, t, &per_layer);
+        };
+        add_prod(sc.dim, sc.q_dim, 2);            // wq, wo
+        add_prod(sc.dim, sc.kv_dim, 2);           // wk, wv
+        add_prod(sc.dim, sc.hidden, 3);           // w1, w3, w2
+        add_prod(sc.dim, 2, 1);                   // the two norm gains
+        over |= __builtin_mul_overflow(per_layer, (size_t)sc.nlayers, &total);
+        over |= __builtin_mul_overflow((size_t)sc.vocab, (size_t)sc.dim, &t) || __builtin_add_overflow(total, t, &total) ||
+                __builtin_add_overflow(total, (size_t)sc.dim, &total);
+        if (over || payload_floats != total)
             return bad(err, "checkpoint payload does not match the shape file beside it");
     } else {
         const size_t heads = dim / 128;
@@ -153,8 +172,19 @@ bool load_checkpoint(const std::string &path, Checkpoint *out, std::string *err)
     close(fd);
     if (p == MAP_FAILED) return bad(err, "cannot map " + path + ": " + strerror(errno));
     const bool packed = len >= 4 && memcmp(p, "RSTQ", 4) == 0;
-    const bool ok = packed ? parse_packed_checkpoint((const uint8_t *)p, len, out, err)
-                           : parse_checkpoint((const uint8_t *)p, len, out, err, have_shape ? &shape : nullptr);
+    bool ok = packed ? parse_packed_checkpoint((const uint8_t *)p, len, out, err)
+                     : parse_checkpoint((const uint8_t *)p, len, out, err, have_shape ? &shape : nullptr);
+    if (!ok && !packed && have_shape) {
+        // A side file that does not fit the payload may be left over from an earlier file of the same name:
+        // a checkpoint the header alone describes (what the reference writes) is read as such.
+        std::string err2;
+        Checkpoint plain;
+        if (parse_checkpoint((const uint8_t *)p, len, &plain, &err2, nullptr)) {
+            *out = std::move(plain);
+            if (err) err->clear();
+            ok = true;
+        }
+    }
     munmap(p, len);
     return ok;
 }

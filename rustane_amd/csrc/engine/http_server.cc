@@ -539,6 +539,7 @@ bool HttpServer::listen_and_serve(const std::string &bind_addr, std::string *err
         if (fd < 0) {
             if (errno == EINTR) continue;
             fprintf(stderr, "accept failed: %s\n", strerror(errno));
+            usleep(100 * 1000);                       // (out of descriptors and the like: do not spin on it)
             continue;
         }
         timeval tv{30, 0};                            // a client that stops sending does not hold the one connection for ever

@@ -1,6 +1,7 @@
 // C ABI of the gfx950 decode backend (see include/hip_decode.h): model construction, weight
 // conversion, hipGraph-captured decode steps and the head variants.
 #include "../../include/hip_decode.h"
+#include "../../include/hip_decode_debug.h"
 #include "hipdec_mega.h"
 #include "hipdec_prefill.h"
 #include "hipdec_batch.h"
@@ -18,6 +19,9 @@
 #include <memory>
 #include <mutex>
 #include <thread>
+#include <unistd.h>
+
+extern char **environ;
 
 namespace {
 
@@ -122,6 +126,7 @@ struct hipdec_model {
     int mega_grid = 0;
     size_t mega_lds = 0;
     unsigned *d_epochs = nullptr;
+    unsigned *h_abort = nullptr, *d_abort = nullptr;  // abort flags of the persistent kernels: pinned host memory, mapped ([0] single-row, [16] multi-row)
     void *xslab = nullptr;                            // uncached slab holding the exchange buffers (uncached_take)
     size_t xslab_cap = 0;
     PrefillWork pf;
@@ -484,9 +489,10 @@ int sync_checked(hipdec_model *m) {
         HCHK(hipEventElapsedTime(&m->last_ms, m->ev_s0, m->ev_s1));
     }
     if (m->mega_ok) {
-        unsigned flag = 0;
-        HCHK(hipMemcpy(&flag, m->d_epochs + 2, 4, hipMemcpyDeviceToHost));
+        // (the kernels write the flag into mapped host memory; the wait above has made it visible)
+        const unsigned flag = __atomic_load_n(&m->h_abort[0], __ATOMIC_ACQUIRE);
         if (flag) {
+            __atomic_store_n(&m->h_abort[0], 0u, __ATOMIC_RELEASE);
             // The aborted step left a mix of old and new stamps in the exchange buffers and did not
             // advance the epochs, so a later step could accept its values: clear all of it and let
             // every later step take the one-kernel-per-product path (its captured graphs hold
@@ -811,7 +817,8 @@ bool rows_kernel_fits(const hipdec_model *m, int R) {
     if (std::max(std::max(N * D, 2 * H * D), std::max(D * Q, D * H)) * 2 >= (1L << 31) - 65536) return false;   // descriptors and 32-bit offsets
     if ((long)R * c.heads > G) return false;
     if (c.hd != 64 && c.hd != 128) return false;
-    return rows_lds(ROWS_MAX_R, (int)D, (int)Q, (int)KV, (int)H, (int)c.nlayers, (int)c.hd, G).total <= 160 * 1024;
+    // (the kernel's static LDS comes on top of this: the same margin as the single-row kernel keeps)
+    return rows_lds(ROWS_MAX_R, (int)D, (int)Q, (int)KV, (int)H, (int)c.nlayers, (int)c.hd, G).total <= 160 * 1024 - 2048;
 }
 
 int rows_prepare(hipdec_model *m, int R) {
@@ -827,7 +834,8 @@ int rows_prepare(hipdec_model *m, int R) {
                               (size_t)ns_cap * REC * 4, (size_t)G * 4};
         size_t xoff[6], total = 0;
         for (int i = 0; i < 6; ++i) { xoff[i] = total; total += (xb[i] + 255) & ~(size_t)255; }
-        b.rows_slab = uncached_take(m->opt.device, total, &b.rows_slab_cap);
+        // (a slab taken by an earlier attempt that failed further down is used again, not taken twice)
+        if (!b.rows_slab) b.rows_slab = uncached_take(m->opt.device, total, &b.rows_slab_cap);
         if (!b.rows_slab) return HIPDEC_OK;                        // no uncached memory: the step stays as it is
         b.rows_slab_bytes = total;
         char *base = (char *)b.rows_slab;
@@ -841,15 +849,15 @@ int rows_prepare(hipdec_model *m, int R) {
             size_t off[4], stride = 0;
             for (int i = 0; i < 4; ++i) { off[i] = stride; stride += (cf[i] + 63) & ~(size_t)63; }
             b.rows_xb_bytes = (size_t)ROWS_XCD_COPIES * stride * 4;
-            if ((rc = dalloc(m, &b.rows_xb, b.rows_xb_bytes))) return rc;
+            if (!b.rows_xb && (rc = dalloc(m, &b.rows_xb, b.rows_xb_bytes))) return rc;
             a.XB = b.rows_xb; a.xb_stride = (int)stride; a.xb_copies = ROWS_XCD_COPIES;
             a.xb_x = (int)off[0]; a.xb_x2 = (int)off[1]; a.xb_gate = (int)off[2]; a.xb_att = (int)off[3];
         }
-        if ((rc = dalloc(m, &b.rows_epochs, 16))) return rc;
-        if ((rc = dalloc(m, &b.rows_suf, (size_t)2 * c.nlayers * sizeof(void *)))) return rc;
+        if (!b.rows_epochs && (rc = dalloc(m, &b.rows_epochs, 16))) return rc;
+        if (!b.rows_suf && (rc = dalloc(m, &b.rows_suf, (size_t)2 * c.nlayers * sizeof(void *)))) return rc;
         a.layers = m->mega.layers; a.gfinal = m->gfinal; a.rope_cos = m->rope_cos; a.rope_sin = m->rope_sin;
         a.kc_suf = b.rows_suf; a.vc_suf = b.rows_suf + c.nlayers;
-        a.bp = b.d_bp; a.epochs = b.rows_epochs;
+        a.bp = b.d_bp; a.epochs = b.rows_epochs; a.abort = m->d_abort + 16;
         a.D = (int)D; a.Q = (int)Q; a.KV = (int)KV; a.H = (int)H; a.L = (int)c.nlayers; a.heads = (int)c.heads;
         a.gqa = c.gqa_ratio ? (int)c.gqa_ratio : 1; a.act = (int)m->opt.ffn_activation; a.alpha = m->alpha;
         const int lds_max = rows_lds(ROWS_MAX_R, a.D, a.Q, a.KV, a.H, a.L, (int)c.hd, G).total;
@@ -892,9 +900,9 @@ int rows_prepare(hipdec_model *m, int R) {
 int rows_check(hipdec_model *m) {
     BatchState &b = m->bt;
     if (!b.rows_active) return HIPDEC_OK;
-    unsigned flag = 0;
-    HCHK(hipMemcpy(&flag, b.rows_epochs + 2, 4, hipMemcpyDeviceToHost));
+    const unsigned flag = __atomic_load_n(&m->h_abort[16], __ATOMIC_ACQUIRE);
     if (!flag) return HIPDEC_OK;
+    __atomic_store_n(&m->h_abort[16], 0u, __ATOMIC_RELEASE);
     b.rows_off = true;
     b.rows_active = false;
     for (auto &g : b.graphs) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
@@ -903,12 +911,28 @@ int rows_check(hipdec_model *m) {
 
 void batch_enqueue(hipdec_model *m, int variant);
 
+bool profiler_attached() {
+    static const bool on = [] {
+        for (const char *name : {"ROCP_TOOL_LIBRARIES", "HSA_TOOLS_LIB", "ROCP_TOOL_LIB"}) {
+            const char *v = getenv(name);
+            if (v && v[0]) return true;
+        }
+        for (char **e = environ; e && *e; ++e)                      // rocprofv3 / rocprofiler-sdk configure their tool through these
+            if (!strncmp(*e, "ROCPROF_", 8) || !strncmp(*e, "ROCPROFILER_", 12)) return true;
+        return false;
+    }();
+    return on;
+}
+
 // Everything that changes from step to step (tokens, position, sampler parameters) lives in device
 // memory, so the ~210 launches of a step are captured once per (rows, head variant) and replayed.
 int batch_launch(hipdec_model *m, int variant) {
     BatchState &b = m->bt;
     const int R = b.rows;
-    if (m->opt.flags & HIPDEC_FLAG_NO_GRAPH) {
+    // Replaying the step's ~210-node graph under rocprofv3's kernel trace ended once in a segmentation
+    // fault inside the HIP runtime (cause not established): with a profiler tool library in the process
+    // the step is launched kernel by kernel instead.  The one-launch layer kernel's graphs are a few nodes.
+    if ((m->opt.flags & HIPDEC_FLAG_NO_GRAPH) || (profiler_attached() && !b.rows_active)) {
         batch_enqueue(m, variant);
         HCHK(hipGetLastError());
         return HIPDEC_OK;
@@ -1220,6 +1244,7 @@ void hipdec_destroy(hipdec_model *m) {
     if (m->bt.h_stage) (void)hipHostFree(m->bt.h_stage);
     if (m->bt.h_ring) (void)hipHostFree(m->bt.h_ring);
     if (m->h_samp) (void)hipHostFree(m->h_samp);
+    if (m->h_abort) (void)hipHostFree(m->h_abort);
     if (m->ev0) (void)hipEventDestroy(m->ev0);
     if (m->ev1) (void)hipEventDestroy(m->ev1);
     if (m->ev_s0) (void)hipEventDestroy(m->ev_s0);
@@ -1227,6 +1252,8 @@ void hipdec_destroy(hipdec_model *m) {
     if (m->stream) (void)hipStreamDestroy(m->stream);
     delete m;
 }
+
+static void *noalloc_scratch();
 
 // base != null: the new model takes base's weights (same configuration and weight format) instead of uploading any
 static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hipdec_head_f32 *head,
@@ -1364,6 +1391,12 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
     HCHK(hipMemset(m->d_ss, 0, sizeof(SampleParams)));
     TRY(dalloc(m, &m->d_rng, sizeof(uint64_t) * 32));
     HCHK(hipHostMalloc((void **)&m->h_samp, sizeof(SampleHost), hipHostMallocDefault));
+    // abort flags of the persistent kernels: host memory the device writes through a mapping, so that the
+    // host needs no copy of its own to look at them after a wait for the stream
+    HCHK(hipHostMalloc((void **)&m->h_abort, 128, hipHostMallocMapped));
+    memset(m->h_abort, 0, 128);
+    HCHK(hipHostGetDevicePointer((void **)&m->d_abort, m->h_abort, 0));
+    (void)noalloc_scratch();              // (resolves this device's scratch array of hipdec_sample_fullvocab_noalloc outside any capture)
     // ---- persistent per-token kernel: exchange buffers, layer table, eligibility
     {
         const int G = m->num_cu;
@@ -1393,6 +1426,13 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
         const size_t odd_tasks = std::max(tasks_of(D, Q), tasks_of(D, H));
         const size_t stage_floats = std::max((size_t)MEGA_WAVES * (c.hd + MEGA_PREC) + 3 * c.hd, 2 * odd_tasks);
         m->mega_lds = fixed_lds + stage_floats * 4;
+        // Models whose output / down projections are more than one register round per wave get a second round
+        // prefetched into LDS where it fits (hipdec_mega.h, issue_odd_lds): MEGA_LDS_TASKS tasks of 4 KB per wave.
+        const size_t odd_rounds_w = (odd_tasks + MEGA_WAVES - 1) / MEGA_WAVES;
+        const size_t lds_pf = 1024 + (size_t)MEGA_WAVES * MEGA_LDS_TASKS * 4096;
+        const char *env_pf = getenv("HIPDEC_NO_LDS_PREFETCH");
+        const bool lds_tasks_on = odd_rounds_w > MEGA_DEPTH_B && m->mega_lds + lds_pf <= lds_cap && !(env_pf && env_pf[0] == '1');
+        if (lds_tasks_on) m->mega_lds += lds_pf;
         const char *env = getenv("HIPDEC_NO_MEGA");
         bool want = !(m->opt.flags & HIPDEC_FLAG_NO_MEGA) && !(env && env[0] == '1');
         bool fits = ns_max >= 1 && m->mega_lds <= lds_cap && (V % 2 == 0) && (int)c.heads <= G &&
@@ -1439,11 +1479,12 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
             HCHK(hipMemset(a.CAND, 0, (size_t)G * 8));
             HCHK(hipMemset(m->d_epochs, 0, 16));
             HCHK(hipMemset(m->x_a, 0, D * 4));
-            a.epochs = m->d_epochs;
+            a.epochs = m->d_epochs; a.abort = m->d_abort;
             a.D = (int)D; a.Q = (int)Q; a.KV = (int)KV; a.H = (int)H; a.V = (int)V; a.L = (int)c.nlayers;
             a.hd = (int)c.hd; a.heads = (int)c.heads; a.gqa = c.gqa_ratio ? (int)c.gqa_ratio : 1;
             a.act = (int)m->opt.ffn_activation; a.ns_max = ns_max; a.seq = (int)S; a.alpha = m->alpha;
             a.stage_floats = (int)stage_floats;
+            a.lds_tasks = lds_tasks_on ? MEGA_LDS_TASKS : 0;
             m->mega_grid = G;
             hipError_t e;
             switch (wt) {
@@ -2002,6 +2043,14 @@ int hipdec_decode_fullvocab_sampled_run_batch(hipdec_model *m, const uint32_t *t
     return batch_sampled_run(m, B_STATS_S, tokens, 1, temperature, softcap, rng_states, n_steps, out_tokens);
 }
 
+int hipdec_debug_set_spin_limit(uint32_t check_mask, uint32_t limit) {
+    const unsigned v[2] = {check_mask, limit};
+    hipError_t e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = hipMemcpyToSymbol(HIP_SYMBOL(g_spin_ctl), v, sizeof v);
+    if (e != hipSuccess) { g_create_error = std::string("hipdec_debug_set_spin_limit: ") + hipGetErrorString(e); return HIPDEC_ERR_HIP; }
+    return HIPDEC_OK;
+}
+
 int hipdec_debug_hostmath_probe(void) { return hostmath_matches_libm() ? 1 : 0; }
 
 int hipdec_debug_sample_topk(const float *vals, const uint32_t *idxs, size_t blocks, uint32_t top_k, float temperature,
@@ -2071,6 +2120,21 @@ __global__ void k_noalloc_reset(SampleParams *ss, uint32_t *ring, float temperat
 static std::mutex g_scratch_mu;
 static void *g_scratch_ptr[64] = {};      // by device ordinal
 
+// This device's copy of the array, looked up once per device (hipGetSymbolAddress may load the code object,
+// which must not happen under stream capture: hipdec_create* call this, so a process that has created a
+// model on the device can record the entry point below into a graph from its first call on).
+static void *noalloc_scratch() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void)hipGetLastError(); return nullptr; }
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) == hipSuccess) g_scratch_ptr[dev] = p;
+        else (void)hipGetLastError();
+    }
+    return g_scratch_ptr[dev];
+}
+
 int hipdec_sample_fullvocab_noalloc(const float *d_logits, size_t vocab, const float *d_maxes, const float *d_sums,
                                     float temperature, float softcap, uint64_t *d_rng_state, uint32_t *d_out_token,
                                     void *stream) {
@@ -2082,21 +2146,11 @@ int hipdec_sample_fullvocab_noalloc(const float *d_logits, size_t vocab, const f
         g_create_error = "hipdec_sample_fullvocab_noalloc: vocab exceeds the 262144 rows (1024 blocks of 256) this entry point serves";
         return HIPDEC_ERR_ARG;
     }
-    int dev = -1;
-    hipError_t e = hipGetDevice(&dev);
-    void *base = nullptr;
-    if (e == hipSuccess && (dev < 0 || dev >= 64)) {
-        g_create_error = "hipdec_sample_fullvocab_noalloc: device ordinal out of range";
+    hipError_t e = hipSuccess;
+    void *base = noalloc_scratch();
+    if (!base) {
+        g_create_error = "hipdec_sample_fullvocab_noalloc: no scratch array for the current device";
         return HIPDEC_ERR_UNSUPPORTED;
-    }
-    if (e == hipSuccess) {
-        std::lock_guard<std::mutex> lock(g_scratch_mu);
-        if (!g_scratch_ptr[dev]) {
-            void *p = nullptr;
-            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));      // this device's copy of the array
-            if (e == hipSuccess) g_scratch_ptr[dev] = p;
-        }
-        base = g_scratch_ptr[dev];
     }
     if (e == hipSuccess) {
         SampleParams *ss = (SampleParams *)base;

@@ -44,6 +44,9 @@
                                 // every further split is two more polls per thread in the fold)
 #endif
 #define MEGA_LPTR 12            // pointers per layer in the LDS copy of the layer table
+#ifndef MEGA_LDS_TASKS
+#define MEGA_LDS_TASKS 2        // odd-phase tasks (4 KB each) per wave that are prefetched into LDS behind the register round
+#endif
 
 enum { MK_QKV = 0, MK_WO = 1, MK_W13 = 2, MK_W2 = 3, MK_HEAD = 4, MK_KINDS = 5 };
 
@@ -62,10 +65,12 @@ struct MegaArgs {
     unsigned long long *CAND;                        // [grid] argmax candidates
     StepParams *sp;
     uint32_t *ring;
-    unsigned *epochs;                                // [0] per-layer exchange counter, [1] head counter, [2] abort
+    unsigned *epochs;                                // [0] per-layer exchange counter, [1] head counter
+    unsigned *abort;                                 // abort flag (host memory mapped into the device)
     unsigned long long *prof;                        // nullable: workgroup 0 writes wall-clock stamps here
     int ring_cap;
     int D, Q, KV, H, V, L, hd, heads, gqa, act, do_head, advance, ns_max, seq, stage_floats;
+    int lds_tasks;                                   // 0, or MEGA_LDS_TASKS: the LDS has room for that many prefetched tasks per wave
     float alpha;
 };
 
@@ -90,6 +95,18 @@ __device__ __forceinline__ uint16_t ldg_u16(const void *p) {
 __device__ __forceinline__ unsigned ld_u32_coherent(const unsigned *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// The abort flag of a model lives in pinned host memory that the device maps: the host reads it after
+// its wait for the stream without a copy of its own, the kernels touch it only when a wait has lasted
+// for many polls.
+__device__ __forceinline__ unsigned ld_abort(const unsigned *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ void raise_abort(unsigned *p) {
+    __hip_atomic_store(p, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+// How a waiting thread bounds its wait: it looks at its poll count when (count & mask) == 0 and gives up
+// at `limit`.  Constants of the device so that a test can make the waits give up (hipdec_debug_set_spin_limit).
+__constant__ unsigned g_spin_ctl[2] = {127u, MEGA_SPIN_LIMIT};
 __device__ __forceinline__ void st_stamped(float *p, float v, unsigned par) {
     unsigned u = (__float_as_uint(v) & ~1u) | par;
     __hip_atomic_store((unsigned *)p, u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -108,10 +125,10 @@ __device__ __forceinline__ bool stamp_bad(const mega_u4 &v, unsigned pm) {
 __device__ __forceinline__ bool repoll16(mega_u4 &v, __amdgpu_buffer_rsrc_t r, int byte_off, unsigned pm, unsigned *abortf) {
     unsigned spins = 0;
     while (stamp_bad(v, pm)) {
-        if ((++spins & 127u) == 0) {
-            if (ld_u32_coherent(abortf)) return false;
-            if (spins > MEGA_SPIN_LIMIT) {
-                __hip_atomic_store(abortf, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((++spins & g_spin_ctl[0]) == 0) {
+            if (ld_abort(abortf)) return false;
+            if (spins > g_spin_ctl[1]) {
+                raise_abort(abortf);
                 return false;
             }
         }
@@ -196,6 +213,18 @@ __device__ __noinline__ float mega_poll_vec(const float *src, int n, unsigned pa
     return good ? ss : -1.0f;
 }
 
+// One load-to-LDS instruction of a wave: the 16 bytes at gptr of every active lane l land at LDS byte
+// address lds_base + 16 l (lds_base wave-uniform, through M0).  No destination registers, so a round of
+// weights requested this way costs no register set; it is counted by vmcnt like any other load and
+// completes in order with them.  Issued as assembly: the compiler then places no waits of its own for it
+// (the waits that cover it are stated by hand where the data is read).
+__device__ __forceinline__ void mega_dma16(const void *gptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(gptr), "s"(lds_base) : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t mega_lds_addr(const void *p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
+
 // Sum over the 64 lanes of a wave with data-parallel-primitive moves (no LDS round trips);
 // the total is valid in lane 63.  Fixed order: quads, halves of 8, rows of 16, then the rows.
 template <int CTRL, int ROW_MASK>
@@ -274,6 +303,8 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     // weight / scale pointers of every layer, copied once so that computing a load address never
     // waits on device memory: [L][MEGA_LPTR] = w[4], sc[4], g1, g2, kc, vc
     const void **lptr = (const void **)(ropes + 2 * (((Q + 2 * KV) / 2 + G - 1) / G) + 2);
+    // prefetch area of the odd phases: [wave][task][load] kilobytes, 1 KB aligned (present when a.lds_tasks != 0)
+    char *const wl = (char *)(((uintptr_t)(lptr + MEGA_LPTR * L) + 1023) & ~(uintptr_t)1023);
     for (int i = threadIdx.x; i < MEGA_LPTR * L; i += MEGA_THREADS) {
         const int l = i / MEGA_LPTR, j = i - l * MEGA_LPTR;
         const MegaLayer &ml = a.layers[l];
@@ -303,7 +334,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     }
     const int pos = a.sp->pos, tok = a.sp->tok, use_x_in = a.sp->use_x_in;
     const unsigned ep_layer = a.epochs[0], ep_head = a.epochs[1];
-    unsigned *abortf = a.epochs + 2;
+    unsigned *abortf = a.abort;
     __syncthreads();
 
     if (wave == 0) {
@@ -420,6 +451,49 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
     auto issue_odd = [&]() {
 #pragma unroll
         for (int s = 0; s < MEGA_DEPTH_B; ++s) issue_odd_one(ctxB, stB[s]);
+    };
+    // The tasks behind the register round of an odd phase, requested into LDS: up to MEGA_LDS_TASKS per wave,
+    // each wave into its own slots, which only it reads back (so its own vmcnt wait is all the
+    // synchronisation there is).  Requested in front of the phase's poll -- the wait for the attention
+    // partials or for the gate vector, during which the memory pipeline would otherwise idle.
+    int l_n = 0;                                             // tasks of the coming odd phase this wave has in LDS
+    uint32_t l_sc[MEGA_LDS_TASKS][2][2];                     // their 4-bit group scales
+    const uint32_t wl_wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)mega_lds_addr(wl)) + (uint32_t)wave * (MEGA_LDS_TASKS * 4096u);
+    auto issue_odd_lds = [&]() {
+        l_n = 0;
+        if (!a.lds_tasks) return;
+#pragma unroll
+        for (int q = 0; q < MEGA_LDS_TASKS; ++q) {
+            if (o_left > 0) {
+                const IssueCtx &c = ctxB;
+                const size_t row = (size_t)2 * (c.pair0 + o_pl);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int piece = o_sg * MEGA_SEG_PIECES + j * 64 + lane;
+                    if (piece < c.pieces) {
+#pragma unroll
+                        for (int r = 0; r < 2; ++r) {
+                            mega_dma16(c.W + (row + r) * c.rb + (size_t)piece * 16, wl_wave + (uint32_t)((q * 4 + j * 2 + r) * 1024));
+                            if (WT == WT_INT4) l_sc[q][r][j] = ldg_u16(c.SC + (row + r) * c.kg + (piece >> 2));
+                        }
+                    }
+                }
+                --o_left;
+                o_sg += MEGA_WAVES;
+                while (o_sg >= c.segs) { o_sg -= c.segs; ++o_pl; }
+                ++l_n;
+            }
+        }
+    };
+    auto read_lds_task = [&](const int q, MegaStage<WT> &t) {
+        const char *base = wl + ((size_t)wave * MEGA_LDS_TASKS + q) * 4096 + lane * 16;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                t.w[r][j] = *(const uint4 *)(base + (j * 2 + r) * 1024);
+                if (WT == WT_INT4) t.sc[r][j] = l_sc[q][r][j];
+            }
     };
     // one task: both rows of a pair times the staged vector over one segment
     auto mul_task = [&](const MegaStage<WT> &t, const float *xs, const int sg, const int pieces, float &o0, float &o1) {
@@ -833,6 +907,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         // 0.522 -> 0.504 ms per token; the 5B model, whose qkv phase is several rounds, loses 3 % without
         // the early request and keeps it.)
         const bool early = !(kind == MK_W2 && qkv_one_round);
+        issue_odd_lds();                                     // (needed sooner than the next even phase's tasks)
         if (early) {
             issue_even_one(ctxA, stA[0]);
             if (MEGA_DEPTH > 1) issue_even_one(ctxA, stA[1]);
@@ -903,7 +978,9 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             const int nm = k.ntasks > wave ? (k.ntasks - wave + MEGA_WAVES - 1) / MEGA_WAVES : 0;
             int f_t = wave, f_sg = wave;                     // next task and its segment
             while (f_sg >= k.segs) f_sg -= k.segs;
-            auto odd_round = [&](const int i) {
+            // src_lds: the round's tasks come from this wave's LDS slots (q = s) instead of set B; next: request the
+            // round that follows in set B
+            auto odd_round = [&](const int i, const int cnt, const bool src_lds, const bool next) {
                 float acc[MEGA_DEPTH_B][2];
                 int slot_t[MEGA_DEPTH_B];
 #pragma unroll
@@ -911,25 +988,35 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
 #pragma unroll
                 for (int s = 0; s < MEGA_DEPTH_B; ++s) {
                     slot_t[s] = f_t;
-                    if (i + s < nm) {
-                        mul_task(stB[s], xs, f_sg, k.pieces, acc[s][0], acc[s][1]);
+                    if (s < cnt) {
+                        if (src_lds) {
+                            MegaStage<WT> tl;
+                            read_lds_task(s, tl);
+                            mul_task(tl, xs, f_sg, k.pieces, acc[s][0], acc[s][1]);
+                        } else {
+                            mul_task(stB[s], xs, f_sg, k.pieces, acc[s][0], acc[s][1]);
+                        }
                         __builtin_amdgcn_sched_barrier(0);
                         f_t += MEGA_WAVES; f_sg += MEGA_WAVES;
                         while (f_sg >= k.segs) f_sg -= k.segs;
                     }
                 }
                 if (i == 0) mark();
-                if (i + MEGA_DEPTH_B < nm) issue_odd();
+                if (next) issue_odd();
 #pragma unroll
                 for (int s = 0; s < MEGA_DEPTH_B; ++s) {
-                    if (i + s < nm) {
+                    if (s < cnt) {
                         const float s0 = wave_sum_dpp(acc[s][0]), s1 = wave_sum_dpp(acc[s][1]);
                         if (lane == 63) { stage[2 * slot_t[s]] = s0; stage[2 * slot_t[s] + 1] = s1; }
                     }
                 }
             };
-            if (nm > 0) odd_round(0);                        // (first round outside the loop, as in the even phase)
-            for (int i = MEGA_DEPTH_B; i < nm; i += MEGA_DEPTH_B) odd_round(i);
+            static_assert(MEGA_LDS_TASKS <= MEGA_DEPTH_B, "an LDS round is at most one round of set B");
+            // round 0 from set B (first round outside the loop, as in the even phase); the tasks in LDS were
+            // requested behind it and are multiplied behind it; set B is refilled with what follows them
+            if (nm > 0) odd_round(0, min(nm, MEGA_DEPTH_B), false, MEGA_DEPTH_B + l_n < nm);
+            if (l_n > 0) odd_round(MEGA_DEPTH_B, l_n, true, false);
+            for (int i = MEGA_DEPTH_B + l_n; i < nm; i += MEGA_DEPTH_B) odd_round(i, min(nm - i, MEGA_DEPTH_B), false, i + MEGA_DEPTH_B < nm);
             lds_barrier();
             // thread r finishes local row r: the segments of its pair in order, scale, residual, publish
             if (tid < 2 * k.npl) {
@@ -971,9 +1058,9 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
             for (;;) {
                 c = __hip_atomic_load(a.CAND + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if ((((unsigned)(c >> 63)) ^ par_c) == 0) break;
-                if ((++spins & 127u) == 0) {
-                    if (ld_u32_coherent(abortf)) { ok = false; break; }
-                    if (spins > MEGA_SPIN_LIMIT) { __hip_atomic_store(abortf, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); ok = false; break; }
+                if ((++spins & g_spin_ctl[0]) == 0) {
+                    if (ld_abort(abortf)) { ok = false; break; }
+                    if (spins > g_spin_ctl[1]) { raise_abort(abortf); ok = false; break; }
                 }
             }
             if (ok) {

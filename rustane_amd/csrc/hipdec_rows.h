@@ -59,7 +59,8 @@ struct RowsArgs {
     uint16_t *out_hi, *out_lo;           // [R][D] last residual rows times the final gains, as pairs
     float *out_ssq;                      // [R][D / 256] their chunk sums of squares
     const BatchParams *bp;
-    unsigned *epochs;                    // [0] exchange counter (advances by L per launch), [1] launch counter, [2] abort flag
+    unsigned *epochs;                    // [0] exchange counter (advances by L per launch), [1] launch counter
+    unsigned *abort;                     // abort flag (host memory mapped into the device)
     unsigned long long *prof;            // nullable: workgroup 0 writes ROWS_PROF_SLOTS wall-clock stamps per layer here
     int R, D, Q, KV, H, L, heads, gqa, act, ns_max;
     size_t suf_rows;
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(ROWS_THREADS, 1) void k_rows(RowsArgs a) {
     }
     const int pos = a.bp->pos, slot = a.bp->slot, prefix = a.bp->prefix;
     const unsigned ep = a.epochs[0], ep_launch = a.epochs[1];
-    unsigned *abortf = a.epochs + 2;
+    unsigned *abortf = a.abort;
     // Which workgroups share this one's XCD (and its L2): every workgroup publishes its XCD number, wave 0
     // reads all of them and counts the members of its own XCD and those among them with a smaller index.
     const unsigned myx = rows_xcc_id();

@@ -33,7 +33,7 @@ EXPORTS = [
     "hipdec_decode_topk_sampled_run", "hipdec_decode_fullvocab_sampled_run", "hipdec_decode_topk_sampled_run_batch",
     "hipdec_decode_fullvocab_sampled_run_batch", "hipdec_debug_hostmath_eval", "hipdec_debug_hostmath_checksum",
     "hipdec_debug_hostmath_count_mismatch", "hipdec_debug_hostmath_probe", "hipdec_debug_sample_topk",
-    "hipdec_debug_sample_fullvocab", "hipdec_sample_fullvocab_noalloc",
+    "hipdec_debug_sample_fullvocab", "hipdec_sample_fullvocab_noalloc", "hipdec_debug_set_spin_limit",
 ]
 
 
@@ -229,6 +229,15 @@ def calibration_copy(nbytes, reps=1):
     rc = load_library().hipdec_debug_calibration_copy(nbytes, reps)
     if rc != OK:
         raise HipDecodeError(rc, "calibration copy failed")
+
+
+def set_spin_limit(check_mask=127, limit=1 << 22):
+    """Test hook: how the persistent kernels bound their waits (hipdec_debug_set_spin_limit); the defaults restore them."""
+    lib = load_library()
+    lib.hipdec_debug_set_spin_limit.argtypes = [C.c_uint32, C.c_uint32]
+    rc = lib.hipdec_debug_set_spin_limit(check_mask, limit)
+    if rc != OK:
+        raise HipDecodeError(rc, (lib.hipdec_last_error(None) or b"").decode())
 
 
 def _fptr(a):

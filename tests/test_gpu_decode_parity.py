@@ -381,3 +381,41 @@ def test_models_sharing_one_copy_of_the_weights():
     np.testing.assert_array_equal(twin16.prefill(ids_a), solo16.prefill(ids_a))
     twin.close()
     np.testing.assert_array_equal(twin16.decode_logits_from_id(ta), solo16.decode_logits_from_id(ta))
+
+
+def test_a_wait_that_gives_up_leaves_the_model_on_the_one_kernel_per_product_path():
+    """The persistent step kernel bounds every wait on another workgroup.  With the bound set to zero polls
+    (a test hook; every kernel still exits normally) the first stale poll gives up: the call reports
+    HIPDEC_ERR_HIP, the length is unchanged, and the model takes the one-kernel-per-product path from then
+    on -- the retried step and the steps after it against the oracle."""
+    from rustane_amd import hipdec
+    from rustane_amd.hipdec import ERR_HIP
+    cfg = tiny_cfg(320)
+    w, orc, dev = pair(cfg, std=0.08)
+    ids = np.array([4, 9, 2, 7, 1], np.uint32)
+    orc.forward_window(ids)
+    dev.prefill(ids, want_logits=False)
+    tok, failed = 3, False
+    hipdec.set_spin_limit(0, 0)
+    try:
+        for _ in range(8):                       # (a step whose polls all find fresh values would pass: try a few)
+            n0 = dev.len()
+            try:
+                got = dev.decode_logits_from_id(tok)
+            except HipDecodeError as e:
+                assert e.status == ERR_HIP and "timed out" in str(e)
+                assert dev.len() == n0
+                failed = True
+                break
+            want = orc.decode_logits_from_id(tok)
+            assert rel_err(got, want) < 1e-4
+            tok = int(O.argmax_lower(want))
+    finally:
+        hipdec.set_spin_limit()
+    assert failed, "no wait gave up with a zero poll limit"
+    for _ in range(5):
+        want = orc.decode_logits_from_id(tok)
+        got = dev.decode_logits_from_id(tok)
+        assert rel_err(got, want) < 1e-4
+        assert dev.decode_token_argmax_from_id(int(O.argmax_lower(want))) == int(O.argmax_lower(orc.decode_logits_from_id(int(O.argmax_lower(want)))))
+        tok = int(O.argmax_lower(want))

@@ -241,3 +241,44 @@ def test_rows_kernel_step_profile_is_a_step_like_any_other():
     dev.batch_end()
     with pytest.raises(Exception):
         dev.debug_batch_step_profile(toks)                    # no batch open
+
+
+def test_rows_kernel_wait_that_gives_up_reopens_on_the_kernel_per_product_step():
+    """The multi-row layer kernel bounds its waits like the single-row one: with the bound at zero polls (test
+    hook, every kernel exits normally) a step reports HIPDEC_ERR_HIP; the reopened batch runs one kernel per
+    product and its rows still equal their oracles."""
+    from rustane_amd import hipdec
+    from rustane_amd.hipdec import HipDecodeError, ERR_HIP
+    cfg = Config.make(dim=256, hidden=512, heads=2, hd=128, seq=96, nlayers=2, vocab=320)
+    rows = 3
+    w, dev, orcs, ids = setup(cfg, rows, 20)
+    dev.batch_begin(rows)
+    assert dev.batch_layers_in_one_launch()
+    toks = np.array([1, 8, 15], np.uint32)
+    failed = False
+    hipdec.set_spin_limit(0, 0)
+    try:
+        for _ in range(6):
+            try:
+                got = dev.decode_logits_from_ids_batch(toks)
+            except HipDecodeError as e:
+                assert e.status == ERR_HIP
+                failed = True
+                break
+            want = np.stack([orcs[r].decode_logits_from_id(int(toks[r])) for r in range(rows)])
+            for r in range(rows):
+                assert rel_err(got[r], want[r]) < 1e-4
+    finally:
+        hipdec.set_spin_limit()
+    assert failed, "no wait gave up with a zero poll limit"
+    dev.batch_end()
+    # the oracles of the rows restart from the prompt, like the reopened batch
+    orcs = []
+    for _ in range(rows):
+        o = O.Oracle(cfg, w)
+        o.forward_window(ids)
+        orcs.append(o)
+    dev.batch_begin(rows)
+    assert not dev.batch_layers_in_one_launch()
+    walk(dev, orcs, cfg, rows, 4, 1e-4)
+    dev.batch_end()

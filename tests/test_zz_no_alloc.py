@@ -25,6 +25,13 @@ class Hip:
         self.rt.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
         self.rt.hipStreamCreate.argtypes = [C.POINTER(C.c_void_p)]
         self.rt.hipStreamDestroy.argtypes = [C.c_void_p]
+        self.rt.hipStreamSynchronize.argtypes = [C.c_void_p]
+        self.rt.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+        self.rt.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        self.rt.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+        self.rt.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+        self.rt.hipGraphExecDestroy.argtypes = [C.c_void_p]
+        self.rt.hipGraphDestroy.argtypes = [C.c_void_p]
         self.bufs = []
 
     def ok(self, rc):
@@ -100,6 +107,46 @@ def test_noalloc_draw_equals_the_allocating_entry_point_on_consecutive_calls():
             got, want = _draw_pair(hip, lg, T, seed, softcap=cap, stream=side if rep == 2 else None)
             assert got == want, (V, T, cap, rep, got, want)
     hip.ok(hip.rt.hipStreamDestroy(side))
+
+
+@pytest.mark.gpu
+def test_noalloc_draw_recorded_into_a_graph_replays_like_the_eager_call():
+    """The use the entry point is for: recorded under stream capture (kernel nodes only -- it clears its
+    run state with a kernel, not a memset) and replayed, with the caller's own eager copies and waits
+    between the replays; every replay against the allocating entry point's draw."""
+    hip = Hip()
+    rng = np.random.default_rng(9)
+    V, T = 5000, 0.9
+    logits = (rng.standard_normal(V) * 3.0).astype(np.float32)
+    inv_t = float(np.float32(1.0) / np.float32(T))
+    mx, sm = O.block_stats(logits, inv_t, 0.0)
+    d_lg, d_mx, d_sm = hip.put(logits), hip.put(mx), hip.put(sm)
+    d_rng = hip.put(np.array([1], np.uint64))
+    d_tok = hip.put(np.array([0xFFFFFFFF], np.uint32))
+    s = hip.stream()
+    # the first call on a device looks the scratch array up, which is not a capturable operation (creating a
+    # model does the same): one eager call, then the capture
+    hipdec.sample_fullvocab_noalloc(d_lg, V, d_mx, d_sm, T, d_rng, d_tok, stream=s)
+    hip.ok(hip.rt.hipStreamSynchronize(s))
+    hip.ok(hip.rt.hipStreamBeginCapture(s, 1))                       # thread-local capture
+    hipdec.sample_fullvocab_noalloc(d_lg, V, d_mx, d_sm, T, d_rng, d_tok, stream=s)
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    hip.ok(hip.rt.hipStreamEndCapture(s, C.byref(graph)))
+    hip.ok(hip.rt.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0))
+    for seed in (41, 42, 43):
+        want = hipdec.debug_sample_fullvocab(logits, mx, sm, T, seed)
+        one = np.array([seed], np.uint64)
+        hip.ok(hip.rt.hipMemcpy(C.c_void_p(d_rng), one.ctypes.data_as(C.c_void_p), 8, 1))
+        none = np.array([0xFFFFFFFF], np.uint32)
+        hip.ok(hip.rt.hipMemcpy(C.c_void_p(d_tok), none.ctypes.data_as(C.c_void_p), 4, 1))
+        hip.ok(hip.rt.hipGraphLaunch(gexec, s))
+        hip.ok(hip.rt.hipStreamSynchronize(s))
+        got = (int(hip.get(d_tok, np.uint32, 1)[0]), int(hip.get(d_rng, np.uint64, 1)[0]))
+        assert got == want, (seed, got, want)
+    hip.ok(hip.rt.hipGraphExecDestroy(gexec))
+    hip.ok(hip.rt.hipGraphDestroy(graph))
+    hip.ok(hip.rt.hipStreamDestroy(s))
+    hip.free_all()
 
 
 @pytest.mark.gpu
