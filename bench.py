@@ -317,7 +317,8 @@ def measure(args, workload, with_cpu_baseline):
     if wdt != WeightDtype.F32 and n_prompt > 32:
         default_mode = 2 if (kvdt == KvDtype.BF16 and wdt in (WeightDtype.FP8_E4M3, WeightDtype.INT4_G128)) else 0
         prefill_options = {"default": ("bf16_pair", "bf16", "f16")[default_mode] + "_activations"}
-        for name, mode in (("bf16_pair_activations", 0), ("bf16_activations", 1), ("f16_activations", 2)):
+        # (mixed: the pair into the q/k/v and output projections, single bf16 numbers into the two feed-forward products)
+        for name, mode in (("bf16_pair_activations", 0), ("bf16_activations", 1), ("f16_activations", 2), ("mixed_pair_attention_bf16_ffn", 3)):
             if mode == default_mode:
                 continue
             dev.set_prefill_activations(mode)
@@ -456,7 +457,8 @@ def main():
             if name == args.workload:
                 continue
             short.steps, short.warmup = ALL_CONFIG_STEPS[name], 4
-            allc[name] = summary(measure(short, name, False))
+            # (the tiny workload is the one the CPU can replay whole: its entry carries the CPU figures of both decode modes)
+            allc[name] = summary(measure(short, name, name == "c1_tiny_fp32" and not args.no_cpu_baseline))
         out["all_configs"] = allc
     print(json.dumps(out))
 

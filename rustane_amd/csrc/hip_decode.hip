@@ -459,11 +459,11 @@ int run_step(hipdec_model *m, int variant) {
 int step_with(hipdec_model *m, int variant, size_t slot, const StepParams &p) {
     m->h_sp[slot] = p;
     HCHK(hipMemcpyAsync(m->d_sp, &m->h_sp[slot], sizeof(StepParams), hipMemcpyHostToDevice, m->stream));
-    HCHK(hipEventRecord(m->ev_s0, m->stream));
+    static const bool no_events = [] { const char *v = getenv("HIPDEC_NO_STEP_EVENTS"); return v && v[0] == '1'; }();
+    if (!no_events) HCHK(hipEventRecord(m->ev_s0, m->stream));
     int rc = run_step(m, variant);
     if (rc) return rc;
-    HCHK(hipEventRecord(m->ev_s1, m->stream));
-    m->step_timed = true;
+    if (!no_events) { HCHK(hipEventRecord(m->ev_s1, m->stream)); m->step_timed = true; }
     return HIPDEC_OK;
 }
 
@@ -484,10 +484,7 @@ StepParams base_params(hipdec_model *m, uint32_t token) {
 // stream sync after a step; a persistent-kernel wait that timed out shows up as an error here
 int sync_checked(hipdec_model *m) {
     HCHK(hipStreamSynchronize(m->stream));
-    if (m->step_timed) {           // device time of the single step that was just waited for
-        m->step_timed = false;
-        HCHK(hipEventElapsedTime(&m->last_ms, m->ev_s0, m->ev_s1));
-    }
+    // (the device time of the single step that was just waited for is worked out when hipdec_last_device_ms asks)
     if (m->mega_ok) {
         // (the kernels write the flag into mapped host memory; the wait above has made it visible)
         const unsigned flag = __atomic_load_n(&m->h_abort[0], __ATOMIC_ACQUIRE);
@@ -718,7 +715,9 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
         HCHK(hipMemcpyAsync(w.ids, w.h_ids, (size_t)T * 4, hipMemcpyHostToDevice, m->stream));
         // how this chunk's activations travel between its kernels (the few-row GEMM only takes pairs)
         const bool tiled = T > kSkinnyRows;
-        const int act = !tiled ? PF_ACT_PAIR : m->pf_act;
+        // (mode 3: the pair into the q/k/v and output projections, the hi parts alone into the two feed-forward products)
+        const int act = !tiled ? PF_ACT_PAIR : m->pf_act == 3 ? PF_ACT_PAIR : m->pf_act;
+        const int act_ffn = !tiled ? PF_ACT_PAIR : m->pf_act == 3 ? PF_ACT_BF16 : m->pf_act;
         const int f16 = act == PF_ACT_F16;
         pf_launch_embed(m, T, f16);
         const int nch = (D + PF_CHUNK - 1) / PF_CHUNK;
@@ -753,10 +752,10 @@ int prefill_batched(hipdec_model *m, const uint32_t *ids, size_t n, const float 
             sp = pf_gemm(m, m->wt, w.att_hi, w.att_lo, L.wo, L.s_wo, T, D, Q, act);
             pf_launch_resid(m, T, sp, L.s_wo, w.x, w.x2, L.g2, f16);
             // gate/up, activation
-            sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.w13, L.s_w13, T, 2 * H, D, act);
+            sp = pf_gemm(m, m->wt, w.xn_hi, w.xn_lo, L.w13, L.s_w13, T, 2 * H, D, act_ffn);
             pf_launch_gate(m, T, sp, L.s_w13, f16);
             // down projection, residual, next layer's first norm
-            sp = pf_gemm(m, m->wt, w.gate_hi, w.gate_lo, L.w2, L.s_w2, T, D, H, act);
+            sp = pf_gemm(m, m->wt, w.gate_hi, w.gate_lo, L.w2, L.s_w2, T, D, H, act_ffn);
             pf_launch_resid(m, T, sp, L.s_w2, w.x2, w.x, l + 1 < c.nlayers ? m->layers[l + 1].g1 : nullptr, f16);
         }
         HCHK(hipGetLastError());
@@ -1071,6 +1070,7 @@ int batch_fetch(hipdec_model *m, const void *dev, void *host, size_t floats) {
     int rc = rows_check(m);
     if (rc) return rc;
     HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+    m->step_timed = false;
     memcpy(host, b.h_stage, floats * 4);
     return HIPDEC_OK;
 }
@@ -1147,6 +1147,7 @@ int sampled_run(hipdec_model *m, int variant, uint32_t token, uint32_t top_k, fl
     HCHK(hipMemcpyAsync(m->h_samp->rng, m->d_rng, sizeof(uint64_t), hipMemcpyDeviceToHost, m->stream));
     SYNC_CHECKED(m);
     HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+    m->step_timed = false;
     memcpy(out_tokens, m->h_out, n_steps * 4);
     *rng_state = m->h_samp->rng[0];
     m->len += n_steps;
@@ -1189,6 +1190,7 @@ int batch_sampled_run(hipdec_model *m, int variant, const uint32_t *tokens, uint
     HCHK(hipStreamSynchronize(m->stream));
     if ((rc = rows_check(m))) return rc;
     HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+    m->step_timed = false;
     memcpy(out_tokens, b.h_ring, (size_t)R * n_steps * 4);
     memcpy(rng_states, m->h_samp->rng, (size_t)R * sizeof(uint64_t));
     b.slot += n_steps;
@@ -1705,7 +1707,7 @@ int hipdec_set_len(hipdec_model *m, size_t len) {
 
 int hipdec_set_prefill_activations(hipdec_model *m, int mode) {
     if (!m) return HIPDEC_ERR_ARG;
-    if (mode < 0 || mode > 2) return fail(m, HIPDEC_ERR_ARG, "prefill activation mode must be 0 (bf16 pair), 1 (bf16) or 2 (fp16)");
+    if (mode < 0 || mode > 3) return fail(m, HIPDEC_ERR_ARG, "prefill activation mode must be 0 (bf16 pair), 1 (bf16), 2 (fp16) or 3 (pair into the attention products, bf16 into the feed-forward ones)");
     m->pf_act = mode;
     return HIPDEC_OK;
 }
@@ -1896,6 +1898,7 @@ int hipdec_prefill(hipdec_model *m, const uint32_t *ids, size_t n, float softcap
         SYNC_CHECKED(m);
     }
     HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+    m->step_timed = false;
     m->len += n;
     return HIPDEC_OK;
 }
@@ -2018,6 +2021,7 @@ int hipdec_decode_greedy_run(hipdec_model *m, uint32_t token, size_t n_steps, ui
     HCHK(hipMemcpyAsync(m->h_out, m->d_ring, n_steps * 4, hipMemcpyDeviceToHost, m->stream));
     SYNC_CHECKED(m);
     HCHK(hipEventElapsedTime(&m->last_ms, m->ev0, m->ev1));
+    m->step_timed = false;
     memcpy(out_tokens, m->h_out, n_steps * 4);
     m->len += n_steps;
     return HIPDEC_OK;
@@ -2245,6 +2249,11 @@ int hipdec_debug_hostmath_count_mismatch(int fn, uint32_t first_bits, uint64_t c
 
 int hipdec_last_device_ms(const hipdec_model *m, float *out_ms) {
     if (!m || !out_ms) return HIPDEC_ERR_ARG;
+    if (m->step_timed) {
+        hipdec_model *mm = const_cast<hipdec_model *>(m);
+        mm->step_timed = false;
+        if (hipEventElapsedTime(&mm->last_ms, m->ev_s0, m->ev_s1) != hipSuccess) { (void)hipGetLastError(); mm->last_ms = 0.0f; }
+    }
     *out_ms = m->last_ms;
     return HIPDEC_OK;
 }

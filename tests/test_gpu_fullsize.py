@@ -8,7 +8,7 @@ import pytest
 
 import oracle_lib as O
 from rustane_amd import synth
-from rustane_amd.hipdec import HipDecodeModel, KvDtype, WeightDtype
+from rustane_amd.hipdec import Config, HipDecodeModel, KvDtype, WeightDtype
 
 pytestmark = pytest.mark.gpu
 FLAG_PREFILL_STEPS = 4
@@ -149,6 +149,33 @@ def test_5b_bf16_short_prompt_against_the_oracle(w5b, kvdt, tol):
         assert rel_err(b, a) < tol
         assert int(np.argmax(b)) == int(O.argmax_lower(a))
         tok = int(O.argmax_lower(a))
+
+
+@pytest.mark.parametrize("kvdt,tol", [(KvDtype.F32, 2e-4), (KvDtype.BF16, 2e-2)])
+def test_5b_shape_long_prompt_many_attention_splits_against_the_oracle(w5b, kvdt, tol):
+    """The 5B layer shape (dim 4096, 32 heads of 128, hidden 11008) on the first four layers of the 5B weights, so
+    that the CPU oracle can afford a prompt long enough for the token step to deal its attention over several
+    workgroups per head (a split covers 64 cache rows with an fp32 cache, 128 with a bf16 one): the chunked
+    matrix-core prefill of 260 rows, then token steps whose partial records are folded across 3 to 5 splits at
+    dim 4096 / 32 heads, each against the oracle."""
+    cfg5, w5 = w5b
+    cfg = Config.make(dim=cfg5.dim, hidden=cfg5.hidden, heads=cfg5.heads, hd=cfg5.hd, seq=512, nlayers=4, vocab=cfg5.vocab)
+    w = {"embed": w5["embed"], "gamma_final": w5["gamma_final"], "layers": w5["layers"][:4]}
+    dev = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=kvdt)
+    orc = O.Oracle(cfg, w, kv_round_bf16=(kvdt == KvDtype.BF16))
+    ids = synth.make_prompt(11, cfg.vocab, 260)
+    lg_o, _, _ = orc.forward_window(ids)
+    lg_d = dev.prefill(ids)
+    assert rel_err(lg_d, lg_o[0]) < tol
+    tok = int(O.argmax_lower(lg_o[0]))
+    assert int(np.argmax(lg_d)) == tok
+    for _ in range(4):
+        a = orc.decode_logits_from_id(tok)
+        b = dev.decode_logits_from_id(tok)
+        assert rel_err(b, a) < tol
+        assert int(np.argmax(b)) == int(O.argmax_lower(a))
+        tok = int(O.argmax_lower(a))
+    assert dev.len() == 264
 
 
 @pytest.mark.parametrize("wdt", [WeightDtype.FP8_E4M3, WeightDtype.INT4_G128])
