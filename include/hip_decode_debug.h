@@ -57,6 +57,11 @@ int hipdec_debug_hostmath_checksum(int fn, uint32_t first_bits, uint64_t count, 
 int hipdec_debug_hostmath_count_mismatch(int fn, uint32_t first_bits, uint64_t count, int host_threads,
                                          uint64_t *out_mismatches);
 
+/* Which form the single-row token step of this model takes: 0 one kernel per product, 1 the persistent
+ * kernel (hipdec_mega.h), 2 its short-phase form for bf16 models whose reduction lengths are multiples of
+ * 512 (hipdec_lean.h).  Environment HIPDEC_NO_LEAN=1 / HIPDEC_NO_MEGA=1 at creation select the earlier forms. */
+int hipdec_debug_step_kernel(const hipdec_model *m, int *out);
+
 /* Test hook for the bounded waits of the persistent kernels (every wait on another workgroup gives up
  * after a number of polls, raises the model's abort flag and every workgroup leaves; the host call then
  * returns HIPDEC_ERR_HIP and later steps take the one-kernel-per-product path).  check_mask: a waiting

@@ -3,6 +3,7 @@
 #include "../../include/hip_decode.h"
 #include "../../include/hip_decode_debug.h"
 #include "hipdec_mega.h"
+#include "hipdec_lean.h"
 #include "hipdec_prefill.h"
 #include "hipdec_batch.h"
 #include "hipdec_rows.h"
@@ -122,6 +123,7 @@ struct hipdec_model {
     float last_ms = 0.0f;
     // persistent one-launch-per-token step (hipdec_mega.h)
     bool mega_ok = false;
+    int lean_ce = 0;                                  // != 0: the step runs k_lean<lean_ce, ...> (hipdec_lean.h) instead of k_mega
     MegaArgs mega{};
     int mega_grid = 0;
     size_t mega_lds = 0;
@@ -310,10 +312,41 @@ template <int WT> void launch_mega_t(hipdec_model *m, const MegaArgs &a) {
 #undef MEGA
 #undef MEGA2
 }
+template <int CE> void launch_lean_t(hipdec_model *m, const MegaArgs &a) {
+    dim3 grid(m->mega_grid), block(MEGA_THREADS);
+#define LEAN2(KVB, HD, BP) hipLaunchKernelGGL((k_lean<CE, KVB, HD, BP>), grid, block, m->mega_lds, m->stream, a)
+#define LEAN(KVB, HD) do { if (a.prof) LEAN2(KVB, HD, MEGA_VAR_STAMPS); else LEAN2(KVB, HD, MEGA_VAR_PLAIN); } while (0)
+    if (m->kvbf16) { if (m->cfg.hd == 64) LEAN(1, 64); else LEAN(1, 128); }
+    else { if (m->cfg.hd == 64) LEAN(0, 64); else LEAN(0, 128); }
+#undef LEAN
+#undef LEAN2
+}
+template <int CE> hipError_t lean_set_lds_t(hipdec_model *m) {
+    hipError_t e = hipSuccess;
+#define LEAN_ATTR(KVB, HD)                                                                                       \
+    do {                                                                                                          \
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_lean<CE, KVB, HD, MEGA_VAR_PLAIN>),             \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)m->mega_lds);                    \
+        if (e == hipSuccess)                                                                                      \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_lean<CE, KVB, HD, MEGA_VAR_STAMPS>),        \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)m->mega_lds);                \
+    } while (0)
+    if (m->kvbf16) { if (m->cfg.hd == 64) LEAN_ATTR(1, 64); else LEAN_ATTR(1, 128); }
+    else { if (m->cfg.hd == 64) LEAN_ATTR(0, 64); else LEAN_ATTR(0, 128); }
+#undef LEAN_ATTR
+    return e;
+}
+// chunk counts (dim / 512) the short-phase kernel is built for
+constexpr bool lean_ce_built(int ce) { return ce == 1 || ce == 3; }
+
 void launch_mega(hipdec_model *m, int do_head, int advance) {
     MegaArgs a = m->mega;
     a.do_head = do_head;
     a.advance = advance;
+    if (m->lean_ce) {
+        if (m->lean_ce == 1) launch_lean_t<1>(m, a); else launch_lean_t<3>(m, a);
+        return;
+    }
     switch (m->wt) {
         case WT_F32: launch_mega_t<WT_F32>(m, a); break;
         case WT_BF16: launch_mega_t<WT_BF16>(m, a); break;
@@ -504,6 +537,7 @@ int sync_checked(hipdec_model *m) {
             HCHK(hipMemset(m->x_a, 0, (size_t)c.dim * 4));
             HCHK(hipMemset(m->d_epochs, 0, 16));
             m->mega_ok = false;
+            m->lean_ce = 0;
             for (auto &g : m->graphs) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
             m->err = "persistent decode kernel: a wait on another workgroup timed out (the grid needs the whole GPU to "
                      "itself); later steps use one kernel per product";
@@ -1422,11 +1456,22 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
         const size_t xs_floats = D + std::max(Q, H);
         const size_t xres_floats = 2 * ((D / 2 + G - 1) / G) + 2;
         const size_t rope_floats = 2 * (((Q + 2 * KV) / 2 + G - 1) / G) + 2;
-        const size_t fixed_lds = (xs_floats + 2 * xres_floats + rope_floats) * 4 + (size_t)MEGA_LPTR * c.nlayers * sizeof(void *);
+        // The short-phase kernel (hipdec_lean.h) takes bf16 models whose reduction lengths are all multiples of
+        // 512 and whose output / down projections are one round of four (pair, chunk) items per wave.
+        const size_t odd_pairs = (D / 2 + G - 1) / G;
+        const size_t lean_items = odd_pairs * (std::max(Q, H) / 512);
+        const char *env_lean = getenv("HIPDEC_NO_LEAN");
+        const bool lean_fits = wt == WT_BF16 && m->embed_wt == WT_BF16 && D % 512 == 0 && Q % 512 == 0 && H % 512 == 0 &&
+                               lean_ce_built((int)(D / 512)) && lean_items <= (size_t)MEGA_WAVES * LEAN_ITEMS_B &&
+                               !(env_lean && env_lean[0] == '1');
+        // (the short-phase kernel stages LEAN_PLANES bf16 numbers per element instead of one float: sized for it when it may run)
+        const size_t xs_lean_floats = lean_fits ? (xs_floats * LEAN_PLANES + 1) / 2 : 0;
+        const size_t fixed_lds = (std::max(xs_floats, xs_lean_floats) + 2 * xres_floats + rope_floats) * 4 + (size_t)MEGA_LPTR * c.nlayers * sizeof(void *);
         int ns_max = G / (int)c.heads;                 // one workgroup per (split, head)
         if (ns_max > 32) ns_max = 32;
         const size_t odd_tasks = std::max(tasks_of(D, Q), tasks_of(D, H));
-        const size_t stage_floats = std::max((size_t)MEGA_WAVES * (c.hd + MEGA_PREC) + 3 * c.hd, 2 * odd_tasks);
+        const size_t stage_floats = std::max(std::max((size_t)MEGA_WAVES * (c.hd + MEGA_PREC) + 3 * c.hd, 2 * odd_tasks),
+                                             lean_fits ? 2 * lean_items : (size_t)0);
         m->mega_lds = fixed_lds + stage_floats * 4;
         // Models whose output / down projections are more than one register round per wave get a second round
         // prefetched into LDS where it fits (hipdec_mega.h, issue_odd_lds): MEGA_LDS_TASKS tasks of 4 KB per wave.
@@ -1487,6 +1532,7 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
             a.act = (int)m->opt.ffn_activation; a.ns_max = ns_max; a.seq = (int)S; a.alpha = m->alpha;
             a.stage_floats = (int)stage_floats;
             a.lds_tasks = lds_tasks_on ? MEGA_LDS_TASKS : 0;
+            if (const char *pw = getenv("HIPDEC_PROF_WG")) a.prof_wg = std::max(0, std::min(G - 1, atoi(pw)));
             m->mega_grid = G;
             hipError_t e;
             switch (wt) {
@@ -1497,6 +1543,11 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
             }
             m->mega_ok = (e == hipSuccess);
             if (e != hipSuccess) (void)hipGetLastError();
+            if (m->mega_ok && lean_fits) {
+                const hipError_t el = D / 512 == 1 ? lean_set_lds_t<1>(m) : lean_set_lds_t<3>(m);
+                if (el == hipSuccess) m->lean_ce = (int)(D / 512);
+                else (void)hipGetLastError();
+            }
         }
         if (const char *v = getenv("HIPDEC_VERBOSE"))
             if (v[0] == '1')
@@ -2045,6 +2096,12 @@ int hipdec_decode_topk_sampled_run_batch(hipdec_model *m, const uint32_t *tokens
 int hipdec_decode_fullvocab_sampled_run_batch(hipdec_model *m, const uint32_t *tokens, float temperature, float softcap,
                                               uint64_t *rng_states, size_t n_steps, uint32_t *out_tokens) {
     return batch_sampled_run(m, B_STATS_S, tokens, 1, temperature, softcap, rng_states, n_steps, out_tokens);
+}
+
+int hipdec_debug_step_kernel(const hipdec_model *m, int *out) {
+    if (!m || !out) return HIPDEC_ERR_ARG;
+    *out = !m->mega_ok ? 0 : m->lean_ce ? 2 : 1;
+    return HIPDEC_OK;
 }
 
 int hipdec_debug_set_spin_limit(uint32_t check_mask, uint32_t limit) {

@@ -70,6 +70,7 @@ struct MegaArgs {
     unsigned long long *prof;                        // nullable: workgroup 0 writes wall-clock stamps here
     int ring_cap;
     int D, Q, KV, H, V, L, hd, heads, gqa, act, do_head, advance, ns_max, seq, stage_floats;
+    int prof_wg;                                     // workgroup whose time stamps the profiling build records
     int lds_tasks;                                   // 0, or MEGA_LDS_TASKS: the LDS has room for that many prefetched tasks per wave
     float alpha;
 };
@@ -348,7 +349,7 @@ __global__ __launch_bounds__(MEGA_THREADS, 1) void k_mega(MegaArgs a) {
         }
     }
 
-    unsigned long long *const prof = (VAR != MEGA_VAR_PLAIN && a.prof && b == 0 && tid == 0) ? a.prof : nullptr;
+    unsigned long long *const prof = (VAR != MEGA_VAR_PLAIN && a.prof && b == a.prof_wg && tid == 0) ? a.prof : nullptr;
     int prof_n = 0;
     auto mark = [&]() { if (prof) prof[prof_n++] = wall_clock64(); };
 

@@ -33,7 +33,7 @@ EXPORTS = [
     "hipdec_decode_topk_sampled_run", "hipdec_decode_fullvocab_sampled_run", "hipdec_decode_topk_sampled_run_batch",
     "hipdec_decode_fullvocab_sampled_run_batch", "hipdec_debug_hostmath_eval", "hipdec_debug_hostmath_checksum",
     "hipdec_debug_hostmath_count_mismatch", "hipdec_debug_hostmath_probe", "hipdec_debug_sample_topk",
-    "hipdec_debug_sample_fullvocab", "hipdec_sample_fullvocab_noalloc", "hipdec_debug_set_spin_limit",
+    "hipdec_debug_sample_fullvocab", "hipdec_sample_fullvocab_noalloc", "hipdec_debug_set_spin_limit", "hipdec_debug_step_kernel",
 ]
 
 
@@ -344,6 +344,13 @@ class HipDecodeModel:
         t = C.c_uint32()
         self._chk(self._lib.hipdec_decode_token_argmax(self._h, _fptr(x), C.byref(t)))
         return t.value
+
+    def step_kernel(self):
+        """0: one kernel per product, 1: the persistent step kernel, 2: its short-phase form (hipdec_debug_step_kernel)."""
+        v = C.c_int()
+        self._lib.hipdec_debug_step_kernel.argtypes = [C.c_void_p, C.POINTER(C.c_int)]
+        self._chk(self._lib.hipdec_debug_step_kernel(self._h, C.byref(v)))
+        return v.value
 
     def decode_token_argmax_from_id(self, token):
         t = C.c_uint32()

@@ -419,3 +419,69 @@ def test_a_wait_that_gives_up_leaves_the_model_on_the_one_kernel_per_product_pat
         assert rel_err(got, want) < 1e-4
         assert dev.decode_token_argmax_from_id(int(O.argmax_lower(want))) == int(O.argmax_lower(orc.decode_logits_from_id(int(O.argmax_lower(want)))))
         tok = int(O.argmax_lower(want))
+
+
+# ---- the short-phase form of the persistent step kernel (hipdec_lean.h): bf16 weights, reduction lengths multiples of 512
+LEAN_SHAPES = [
+    # dim 512: one chunk per row of the even phases; hd 128, fp32 cache
+    (dict(dim=512, hidden=1024, heads=4, hd=128, seq=96, nlayers=3, vocab=320), KvDtype.F32, 0, 1e-4),
+    # grouped key/value heads of 64, squared leaky ReLU, bf16 cache, an odd layer count
+    (dict(dim=512, hidden=512, heads=8, hd=64, seq=96, nlayers=3, vocab=600, kv_heads=4), KvDtype.BF16, 1, 2e-3),
+    # dim 1536 (three chunks per row, the 600M-class width), down projection of 2048
+    (dict(dim=1536, hidden=2048, heads=12, hd=128, seq=64, nlayers=2, vocab=512), KvDtype.F32, 0, 1e-4),
+]
+
+
+@pytest.mark.parametrize("shape,kvdt,act,tol", LEAN_SHAPES)
+def test_short_phase_kernel_matches_oracle(shape, kvdt, act, tol):
+    cfg = Config.make(**shape)
+    w, orc, dev = pair(cfg, std=0.06, wdt=WeightDtype.BF16, kvdt=kvdt, act=act)
+    assert dev.step_kernel() == 2
+    ids = synth.make_prompt(5, cfg.vocab, 21)
+    lg_o, _, _ = orc.forward_window(ids)
+    dev.prefill(ids, want_logits=False)
+    tok = int(O.argmax_lower(lg_o[0]))
+    for step in range(8):
+        a = orc.decode_logits_from_id(tok)
+        b = dev.decode_logits_from_id(tok)
+        assert rel_err(b, a) < tol, (step, rel_err(b, a))
+        tok = int(np.argsort(-a, kind="stable")[step % 3])
+    # greedy ids, chained on the device, against the oracle's own greedy loop from here
+    n0 = dev.len()
+    first = tok
+    want, t = [], first
+    for _ in range(6):
+        lg = orc.decode_logits_from_id(t)
+        t = int(O.argmax_lower(lg))
+        want.append(t)
+    got = dev.decode_greedy_run(first, 6)
+    assert dev.len() == n0 + 6
+    if kvdt == KvDtype.F32:
+        assert [int(x) for x in got] == want
+    # per-block top-k candidates and block statistics of the next step (head variants behind the same kernel)
+    a = orc.decode_logits_from_id(want[-1] if kvdt == KvDtype.F32 else int(got[-1]))
+    if kvdt == KvDtype.F32:
+        vals, idxs = dev.decode_token_topk_from_id(want[-1], 4)
+        mv, mi = O.merge_topk(vals, idxs, 4)
+        assert [int(i) for i in mi] == [int(i) for i in np.argsort(-a, kind="stable")[:4]]
+
+
+def test_short_phase_kernel_and_general_kernel_agree_and_repeat_bit_for_bit(monkeypatch):
+    cfg = Config.make(dim=512, hidden=1024, heads=4, hd=128, seq=96, nlayers=3, vocab=320)
+    w = synth.make_weights(cfg, seed=3, std=0.06, round_bf16=True)
+    ids = synth.make_prompt(9, cfg.vocab, 17)
+
+    def run():
+        dev = HipDecodeModel(cfg, w, weight_dtype=WeightDtype.BF16, kv_dtype=KvDtype.F32)
+        kind = dev.step_kernel()
+        lg = dev.prefill(ids)
+        out = [dev.decode_logits_from_id(int(t)) for t in (3, 7, 11, 200)]
+        return kind, out
+    k1, a = run()
+    k2, b = run()
+    monkeypatch.setenv("HIPDEC_NO_LEAN", "1")
+    k3, c = run()
+    assert (k1, k2, k3) == (2, 2, 1)
+    for x, y, z in zip(a, b, c):
+        assert np.array_equal(x, y)                     # a step is bit-reproducible, whatever ran before it
+        assert rel_err(x, z) < 2e-5                     # the two kernels differ in summation order only

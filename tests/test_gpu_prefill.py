@@ -176,5 +176,11 @@ def test_prefill_with_single_number_activations(wdt, n_prompt, flag, bound):
     ref.set_prefill_activations(0)
     ref.set_len(0)
     np.testing.assert_array_equal(ref.prefill(ids), lg_r)
+    # mode 3: the pair into the q/k/v and output projections, single bf16 numbers into the two feed-forward products
+    ref.set_prefill_activations(3)
+    ref.set_len(0)
+    lg_m = ref.prefill(ids)
+    assert rel_err(lg_m, lg_r) <= max(rel_err(lg_d, lg_r), 1e-6) * 1.5 + 1e-4 if flag == FLAG_PREFILL_BF16_ACT else True
+    ref.set_prefill_activations(0)
     with pytest.raises(Exception):
-        ref.set_prefill_activations(3)
+        ref.set_prefill_activations(4)
