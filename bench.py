@@ -45,12 +45,12 @@ ALL_CONFIG_STEPS = {"c1_tiny_fp32": 31, "c2_600m_bf16_bs1": 255, "c3_600m_bf16_8
 
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, each
 # scaled by what the same counter reads for a plain copy of known size): measured separately with
-# rocprofv3 --pmc and recorded in profiles/k_mega_c2_600m_bf16_bs1.md, profiles/k_mega_hbm_traffic_c1_c4_c5.md and
+# rocprofv3 --pmc and recorded in profiles/k_lean_c2_600m_bf16_bs1.md, profiles/k_mega_hbm_traffic_c1_c4_c5.md and
 # profiles/k_rows_c3_600m_bf16_8samples.md
 # (per step, i.e. the LM-head GEMV included where it is a launch of its own, at the KV length of the
 # profiled run); a benchmark run cannot collect it itself.
 TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries under profiles/, not measured in this run"
-MEASURED_TRAFFIC_BYTES = {"c1_tiny_fp32": 1.267e8, "c2_600m_bf16_bs1": 1.5083e9, "c3_600m_bf16_8samples": 1.811e9,
+MEASURED_TRAFFIC_BYTES = {"c1_tiny_fp32": 1.267e8, "c2_600m_bf16_bs1": 1.5092e9, "c3_600m_bf16_8samples": 1.811e9,
                           "c4_5b_bf16_bs1": 1.3874e10, "c5_5b_fp8_bs1": 7.118e9, "c5_5b_int4_bs1": 4.008e9}
 
 
