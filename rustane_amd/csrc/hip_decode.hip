@@ -578,6 +578,17 @@ constexpr int kSkinnyLdsBytes = 40 * 1024;   // dynamic LDS for the staged activ
 // the tiled GEMM whose operands go straight into LDS (k_pf_gemm_dl): bf16 weights, enough rows to fill its
 // 128 x 256 tiles, whole 64-element steps, activations as bf16 (pair or single)
 constexpr int kDlMinRows = 129;
+constexpr int kSkinnyI4Nt = 1;                    // 16-row weight tiles per wave of k_pf_gemm_skinny_i4 (2: 4 - 8 % slower on the 5B shapes)
+constexpr int kSkinnyI4Bn = 64 * kSkinnyI4Nt;     // weight rows per workgroup
+// the few-row GEMM of 4-bit models: the kernel of its own (HIPDEC_NO_SKINNY_I4=1: the general few-row kernel)
+bool pf_use_skinny_i4() {
+    static const bool off = [] { const char *v = getenv("HIPDEC_NO_SKINNY_I4"); return v && v[0] == '1'; }();
+    return !off;
+}
+int pf_skinny_i4_wgs_per_cu() {
+    static const int n = [] { const char *v = getenv("HIPDEC_SKINNY_I4_WGS"); const int x = v ? atoi(v) : 0; return x > 0 && x <= 16 ? x : 3; }();
+    return n;
+}
 bool pf_use_dl(int wt, int T, int K, int act) {
     static const bool off = getenv("HIPDEC_NO_DL_GEMM") != nullptr;
     return !off && wt == WT_BF16 && T >= kDlMinRows && K % PF_BKL == 0 && act != PF_ACT_F16;
@@ -603,6 +614,19 @@ PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K, bool dl =
         return PfSplit{(lsteps + sps - 1) / sps, sps};
     }
     const int nsteps = K / PF_BK;
+    if (T <= kSkinnyRows && wt == WT_INT4 && pf_use_skinny_i4()) {
+        // 4-bit weights: a workgroup owns kSkinnyI4Bn weight rows and every wave walks the whole K range of its
+        // split; a split is a whole number of 128-element scale groups (four steps each), a multiple of four
+        // of them where the staged activation slice (hi + lo) fits the LDS budget with that (the kernel then
+        // reads a round's four scales of a row as one aligned load).  Aim at a few workgroups per CU.
+        const int tiles = (N + kSkinnyI4Bn - 1) / kSkinnyI4Bn, groups = K / 128;
+        int s = std::max(1, (pf_skinny_i4_wgs_per_cu() * m->num_cu + tiles - 1) / tiles);
+        const int max_groups = std::max(1, ((kSkinnyLdsBytes / (4 * T)) - PF_SK_PAD) / 128);
+        int gps = std::min(max_groups, std::max(1, (groups + s - 1) / s));
+        if (gps >= 4) gps &= ~3;
+        else if (max_groups >= 4) gps = 4;
+        return PfSplit{(groups + gps - 1) / gps, 4 * gps};
+    }
     if (T <= kSkinnyRows) {
         // 4 waves per workgroup share a K range; aim at ~8 waves per CU over the whole grid
         const int tiles = (N + 31) / 32;
@@ -678,6 +702,15 @@ int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, c
     }
     const PfSplit sp = pf_split_k(m, wt, T, N, K);
     PfGemm g{Ahi, Alo, W, wt == WT_INT4 ? (const uint16_t *)scales : nullptr, m->pf.P, T, N, K, sp.steps_per_split};
+    if (T <= kSkinnyRows && wt == WT_INT4 && pf_use_skinny_i4()) {
+        const int rt = T <= 16 ? 1 : 2;
+        dim3 grid((N + kSkinnyI4Bn - 1) / kSkinnyI4Bn, sp.splits), block(256);
+        const size_t lds = (size_t)2 * T * (sp.steps_per_split * PF_BK + PF_SK_PAD) * 2 + (size_t)(sp.steps_per_split / 4) * 16 * rt * 4;
+        if (T <= 8) hipLaunchKernelGGL((k_pf_gemm_skinny_i4<1, true, kSkinnyI4Nt>), grid, block, lds, m->stream, g);
+        else if (rt == 1) hipLaunchKernelGGL((k_pf_gemm_skinny_i4<1, false, kSkinnyI4Nt>), grid, block, lds, m->stream, g);
+        else hipLaunchKernelGGL((k_pf_gemm_skinny_i4<2, false, kSkinnyI4Nt>), grid, block, lds, m->stream, g);
+        return sp.splits;
+    }
     if (T <= kSkinnyRows) {
         dim3 grid((N + 31) / 32, sp.splits), block(256);
         const size_t lds = (size_t)2 * T * (sp.steps_per_split * PF_BK + PF_SK_PAD) * 2;

@@ -85,6 +85,15 @@ def test_prefill_int4_weights(n_prompt):
     check_prefill_then_decode(cfg, n_prompt, 1e-4, wdt=WeightDtype.INT4_G128, kvdt=KvDtype.F32, std=0.05)
 
 
+@pytest.mark.parametrize("n_prompt", [5, 8, 13, 16, 27, 32])
+def test_few_row_products_of_4bit_weights(n_prompt):
+    # prompts of at most 32 rows go through the few-row GEMM of 4-bit weights: hi and lo parts in one operand tile
+    # up to 8 rows, one and two row tiles above; reductions of 3 groups (dim 384: the short scale path), 4 (q_dim 512)
+    # and 9 (hidden 1152: splits of 4 + 4 + 1 groups, a round that ends early)
+    cfg = Config.make(dim=384, hidden=1152, heads=4, hd=128, seq=64, nlayers=3, vocab=768, kv_heads=2)
+    check_prefill_then_decode(cfg, n_prompt, 1e-4, wdt=WeightDtype.INT4_G128, kvdt=KvDtype.F32, std=0.05)
+
+
 def test_prefill_int4_matches_token_step_prefill():
     cfg = Config.make(dim=384, hidden=1152, heads=3, hd=128, seq=200, nlayers=3, vocab=1024)
     w = synth.make_weights(cfg, seed=5, std=0.06, round_bf16=True)
