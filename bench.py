@@ -35,13 +35,16 @@ WORKLOADS = {
     "c5_5b_int4_bs1": ("config_5b", "INT4_G128", "BF16", 512, 256),
     # 8 samples over one shared 512-token prompt, temperature 0.8, top-k 8, stepped together
     "c3_600m_bf16_8samples": ("config_600m", "BF16", "BF16", 512, 256),
+    # the same request on the 5B model with 4-bit weights (the multi-sample step as one kernel per product)
+    "c5_5b_int4_8samples": ("config_5b", "INT4_G128", "BF16", 512, 128),
 }
+MULTI_SAMPLE_WORKLOADS = ("c3_600m_bf16_8samples", "c5_5b_int4_8samples")
 C3_SAMPLES, C3_TEMPERATURE, C3_TOP_K = 8, 0.8, 8
 ALL_CONFIG_ORDER = ["c1_tiny_fp32", "c2_600m_bf16_bs1", "c3_600m_bf16_8samples", "c4_5b_bf16_bs1", "c5_5b_fp8_bs1",
-                    "c5_5b_int4_bs1"]
+                    "c5_5b_int4_bs1", "c5_5b_int4_8samples"]
 # timed steps of the short runs behind the all_configs entries (generated steps - 1 of the workload, capped)
 ALL_CONFIG_STEPS = {"c1_tiny_fp32": 31, "c2_600m_bf16_bs1": 255, "c3_600m_bf16_8samples": 64, "c4_5b_bf16_bs1": 32,
-                    "c5_5b_fp8_bs1": 64, "c5_5b_int4_bs1": 64}
+                    "c5_5b_fp8_bs1": 64, "c5_5b_int4_bs1": 64, "c5_5b_int4_8samples": 32}
 
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, each
 # scaled by what the same counter reads for a plain copy of known size): measured separately with
@@ -54,7 +57,7 @@ MEASURED_TRAFFIC_BYTES = {"c1_tiny_fp32": 1.267e8, "c2_600m_bf16_bs1": 1.5092e9,
                           "c4_5b_bf16_bs1": 1.3874e10, "c5_5b_fp8_bs1": 7.118e9, "c5_5b_int4_bs1": 4.008e9}
 
 
-def run_c3(args, workload, cfg, weights, n_prompt):
+def run_c3(args, workload, cfg, weights, n_prompt, wdt, kvdt):
     """Multi-sample workload through the session layer: a step is one pass of the weights that
     advances all 8 samples by one token (per-block top-k candidates, their merge and the reference's
     draw, all on the device: the whole request is one enqueued run); value = sampled tokens per
@@ -62,7 +65,7 @@ def run_c3(args, workload, cfg, weights, n_prompt):
     from rustane_amd import engine as E
     from rustane_amd import synth
     prompt = synth.make_prompt(7, cfg.vocab, n_prompt)
-    s = E.InferenceSession(cfg, weights, prompt, weight_dtype=1, kv_dtype=1)
+    s = E.InferenceSession(cfg, weights, prompt, weight_dtype=int(wdt), kv_dtype=int(kvdt))
     K, W = args.steps, args.warmup
     room = cfg.seq - n_prompt - 1
     K = min(K, room)
@@ -86,8 +89,8 @@ def run_c3(args, workload, cfg, weights, n_prompt):
         "metric": "decode tok/s @600M bf16 bs1; % of HBM peak GB/s; prefill ms",
         "value": C3_SAMPLES * K / decode_s, "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": decode_s * 1e3 / K, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": workload, "prompt_tokens": n_prompt, "batch": C3_SAMPLES, "kv_dtype": "bf16",
+        "dtype": {"F32": "f32", "BF16": "bf16", "FP8_E4M3": "fp8_e4m3", "INT4_G128": "int4"}[wdt.name], "data": "synthetic",
+        "config": {"workload": workload, "prompt_tokens": n_prompt, "batch": C3_SAMPLES, "kv_dtype": kvdt.name.lower(),
                    "temperature": C3_TEMPERATURE, "top_k": C3_TOP_K, "params": cfg.param_count(), "mean_kv_len": mean_kv},
         "prefill_ms": s.prefill_elapsed() * 1e3, "request_wall_ms": wall * 1e3,
         "device_ms_per_step": dev_ms / K,
@@ -296,8 +299,8 @@ def measure(args, workload, with_cpu_baseline):
     cfg = getattr(synth, cfg_name)()
     wdt, kvdt = WeightDtype[wdt], KvDtype[kvdt]
     weights = cached_weights(cfg_name, cfg, args.seed, wdt != WeightDtype.F32)
-    if workload == "c3_600m_bf16_8samples":
-        return run_c3(args, workload, cfg, weights, n_prompt)
+    if workload in MULTI_SAMPLE_WORKLOADS:
+        return run_c3(args, workload, cfg, weights, n_prompt, wdt, kvdt)
     dev = HipDecodeModel(cfg, weights, weight_dtype=wdt, kv_dtype=kvdt)
     prompt = synth.make_prompt(7, cfg.vocab, n_prompt)
 
