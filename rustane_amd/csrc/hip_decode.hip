@@ -585,10 +585,7 @@ bool pf_use_skinny_i4() {
     static const bool off = [] { const char *v = getenv("HIPDEC_NO_SKINNY_I4"); return v && v[0] == '1'; }();
     return !off;
 }
-int pf_skinny_i4_wgs_per_cu() {
-    static const int n = [] { const char *v = getenv("HIPDEC_SKINNY_I4_WGS"); const int x = v ? atoi(v) : 0; return x > 0 && x <= 16 ? x : 3; }();
-    return n;
-}
+constexpr int kSkinnyI4WgsPerCu = 3;              // workgroups per CU its K splits aim at
 bool pf_use_dl(int wt, int T, int K, int act) {
     static const bool off = getenv("HIPDEC_NO_DL_GEMM") != nullptr;
     return !off && wt == WT_BF16 && T >= kDlMinRows && K % PF_BKL == 0 && act != PF_ACT_F16;
@@ -620,7 +617,7 @@ PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K, bool dl =
         // of them where the staged activation slice (hi + lo) fits the LDS budget with that (the kernel then
         // reads a round's four scales of a row as one aligned load).  Aim at a few workgroups per CU.
         const int tiles = (N + kSkinnyI4Bn - 1) / kSkinnyI4Bn, groups = K / 128;
-        int s = std::max(1, (pf_skinny_i4_wgs_per_cu() * m->num_cu + tiles - 1) / tiles);
+        int s = std::max(1, (kSkinnyI4WgsPerCu * m->num_cu + tiles - 1) / tiles);
         const int max_groups = std::max(1, ((kSkinnyLdsBytes / (4 * T)) - PF_SK_PAD) / 128);
         int gps = std::min(max_groups, std::max(1, (groups + s - 1) / s));
         if (gps >= 4) gps &= ~3;

@@ -7,8 +7,10 @@
 //    w13) or 16 (wo, w2) weight rows; a tile is 16 weight rows, v_mfma_f32_16x16x32_bf16 takes a
 //    lane's 16-byte weight load as its A operand as loaded (lane l: row l % 16, reduction elements
 //    8 * (l / 16) .. + 8 of a 32-element step), and the R activation rows are the B operand, read
-//    from LDS as (hi, lo) bf16 pairs (two instructions per weight load, nothing is rounded to 8
-//    bits).  The eight waves split the reduction axis; their 16 x 16 partial tiles meet in LDS;
+//    from LDS as (hi, lo) bf16 pairs: columns 0..7 of the operand tile are the rows' hi parts,
+//    columns 8..15 their lo parts, so ONE instruction per weight load multiplies both (nothing is
+//    rounded to 8 bits).  The eight waves split the reduction axis; their 16 x 16 partial tiles meet
+//    in LDS, where the two halves of every result row are added;
 //  * a phase's weights are ONE round of loads per wave (at most 12 or 16 loads of 16 bytes per lane,
 //    which is what bounds the model sizes this kernel takes), requested in two halves, one and two
 //    phases ahead, into the register set the running phase does not use;
@@ -368,8 +370,11 @@ __global__ __launch_bounds__(ROWS_THREADS, 1) void k_rows(RowsArgs a) {
     auto multiply = [&](const auto &st, auto tt_c, auto jj_c, const int kind) {
         constexpr int TT = decltype(tt_c)::value, JJ = decltype(jj_c)::value;
         const int spw = __builtin_amdgcn_readfirstlane(kinds[kind].spw), ntiles = __builtin_amdgcn_readfirstlane(kinds[kind].ntiles);
-        const int nsrc = r16 < R ? r16 : 0;                  // activation rows past R repeat row 0 (their results are not read)
-        const uint16_t *ph = xh + nsrc * XS + wave * spw * 32 + c4 * 8, *pl = xl + nsrc * XS + wave * spw * 32 + c4 * 8;
+        // The 16 columns of the operand tile are the hi parts of the (at most 8) activation rows and, beside them,
+        // their lo parts: one instruction per weight load multiplies both, and the two halves of a result row are
+        // added where the tiles are summed.  (Rows past R repeat row 0; their results are not read.)
+        const int nsrc = (r16 & 7) < R ? (r16 & 7) : 0;
+        const uint16_t *pp = (r16 < 8 ? xh : xl) + nsrc * XS + wave * spw * 32 + c4 * 8;
 #pragma unroll
         for (int t = 0; t < TT; ++t) {
             if (t < ntiles) {
@@ -378,9 +383,8 @@ __global__ __launch_bounds__(ROWS_THREADS, 1) void k_rows(RowsArgs a) {
                 for (int j = 0; j < JJ; ++j) {
                     if (j < spw) {
                         const rows_bf16x8 w = __builtin_bit_cast(rows_bf16x8, st[t * JJ + j]);
-                        const rows_bf16x8 bh = *(const rows_bf16x8 *)(ph + j * 32), bl = *(const rows_bf16x8 *)(pl + j * 32);
-                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, bh, acc, 0, 0, 0);
-                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, bl, acc, 0, 0, 0);
+                        const rows_bf16x8 bx = *(const rows_bf16x8 *)(pp + j * 32);
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, bx, acc, 0, 0, 0);
                     }
                 }
                 float *rp = red + (wave * ROWS_TA + t) * 256 + (4 * c4) * 16 + r16;
@@ -395,7 +399,7 @@ __global__ __launch_bounds__(ROWS_THREADS, 1) void k_rows(RowsArgs a) {
 #pragma unroll
         for (int w = 0; w < ROWS_WAVES; ++w) {
             const float *rp = red + (w * ROWS_TA + t) * 256 + m * 16 + n;
-            s0 += rp[0]; s1 += rp[16];
+            s0 += rp[0] + rp[8]; s1 += rp[16] + rp[24];        // (columns n and n + 8: hi and lo parts' products)
         }
     };
     auto row_inv = [&](const int n) {
