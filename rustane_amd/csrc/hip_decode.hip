@@ -112,6 +112,7 @@ struct hipdec_model {
     float *d_topk_vals = nullptr, *d_bmax = nullptr, *d_bsum = nullptr, *d_out = nullptr;
     uint32_t *d_topk_idxs = nullptr, *d_ring = nullptr;
     float *h_out = nullptr;                           // pinned staging, max(vocab, 2*blocks*32) floats
+    float *d_hout = nullptr;                          // the same memory as the device sees it (nullptr: not mapped)
     size_t h_out_elems = 0;
     size_t len = 0;
     int NS = 1, blocks = 0;
@@ -129,6 +130,10 @@ struct hipdec_model {
     size_t mega_lds = 0;
     unsigned *d_epochs = nullptr;
     unsigned *h_abort = nullptr, *d_abort = nullptr;  // abort flags of the persistent kernels: pinned host memory, mapped ([0] single-row, [16] multi-row)
+    // The same mapped block, further on: the step parameters ([32]..) and the one-slot token ring ([48]) of a
+    // single step that the host waits for.  The kernel reads its parameters from there and leaves the token there,
+    // so such a step is one launch and one wait: no parameter upload in front of it, no copy behind it.
+    bool direct_step = false;                         // the step just enqueued used them
     void *xslab = nullptr;                            // uncached slab holding the exchange buffers (uncached_take)
     size_t xslab_cap = 0;
     PrefillWork pf;
@@ -339,10 +344,15 @@ template <int CE> hipError_t lean_set_lds_t(hipdec_model *m) {
 // chunk counts (dim / 512) the short-phase kernel is built for
 constexpr bool lean_ce_built(int ce) { return ce == 1 || ce == 3; }
 
-void launch_mega(hipdec_model *m, int do_head, int advance) {
+void launch_mega(hipdec_model *m, int do_head, int advance, bool direct = false) {
     MegaArgs a = m->mega;
     a.do_head = do_head;
     a.advance = advance;
+    if (direct) {      // parameters and token slot in mapped host memory (see hipdec_model::direct_step)
+        a.sp = (StepParams *)(m->d_abort + 32);
+        a.ring = m->d_abort + 48;
+        a.ring_cap = 1;
+    }
     if (m->lean_ce) {
         if (m->lean_ce == 1) launch_lean_t<1>(m, a); else launch_lean_t<3>(m, a);
         return;
@@ -488,11 +498,41 @@ int run_step(hipdec_model *m, int variant) {
     return HIPDEC_OK;
 }
 
+// A single step the caller waits for, on a model whose whole step (head included) is one persistent launch: the
+// kernel takes its parameters from mapped host memory and writes the token there (HIPDEC_NO_DIRECT_STEP=1: the
+// general way, for comparisons).
+static bool direct_step_ok(const hipdec_model *m, int variant) {
+    static const bool off = [] { const char *v = getenv("HIPDEC_NO_DIRECT_STEP"); return v && v[0] == '1'; }();
+    if (off || !m->mega_ok || m->wt != m->embed_wt) return false;
+    return variant == V_X || variant == V_ARGMAX || ((variant == V_TOPK || variant == V_STATS) && m->d_hout);
+}
+
 // upload the step parameters from pinned slot `slot`, then run one step
-int step_with(hipdec_model *m, int variant, size_t slot, const StepParams &p) {
+int step_with(hipdec_model *m, int variant, size_t slot, const StepParams &p, bool caller_waits = false) {
+    static const bool no_events = [] { const char *v = getenv("HIPDEC_NO_STEP_EVENTS"); return v && v[0] == '1'; }();
+    m->direct_step = false;
+    if (caller_waits && direct_step_ok(m, variant)) {     // (one mapped block: only for a step that is waited for before the next)
+        StepParams *hp = (StepParams *)(m->h_abort + 32);
+        *hp = p;
+        hp->step = 0;
+        __atomic_thread_fence(__ATOMIC_RELEASE);
+        if (!no_events) HCHK(hipEventRecord(m->ev_s0, m->stream));
+        launch_mega(m, variant == V_X ? 0 : 1, 1, true);
+        // per-block candidates / statistics straight into the pinned buffer the caller's arrays are filled from
+        const StepParams *dp = (const StepParams *)(m->d_abort + 32);
+        if (variant == V_TOPK)
+            hipLaunchKernelGGL(k_head_topk, dim3(m->blocks), dim3(256), 0, m->stream, m->logits, (int)m->cfg.vocab, dp, m->d_hout,
+                               (uint32_t *)(m->d_hout + (size_t)m->blocks * p.top_k));
+        else if (variant == V_STATS)
+            hipLaunchKernelGGL(k_head_block_stats, dim3(m->blocks), dim3(256), 0, m->stream, m->logits, (int)m->cfg.vocab, dp, m->d_hout,
+                               m->d_hout + m->blocks);
+        HCHK(hipGetLastError());
+        if (!no_events) { HCHK(hipEventRecord(m->ev_s1, m->stream)); m->step_timed = true; }
+        m->direct_step = true;
+        return HIPDEC_OK;
+    }
     m->h_sp[slot] = p;
     HCHK(hipMemcpyAsync(m->d_sp, &m->h_sp[slot], sizeof(StepParams), hipMemcpyHostToDevice, m->stream));
-    static const bool no_events = [] { const char *v = getenv("HIPDEC_NO_STEP_EVENTS"); return v && v[0] == '1'; }();
     if (!no_events) HCHK(hipEventRecord(m->ev_s0, m->stream));
     int rc = run_step(m, variant);
     if (rc) return rc;
@@ -549,9 +589,16 @@ int sync_checked(hipdec_model *m) {
 #define SYNC_CHECKED(m) do { int rc_ = sync_checked(m); if (rc_ != HIPDEC_OK) return rc_; } while (0)
 
 int softcap_out(hipdec_model *m, int start, int n, float cap, float *host_out) {
-    hipLaunchKernelGGL(k_softcap_copy, dim3((n + 255) / 256), dim3(256), 0, m->stream, m->logits, m->d_out, start, n, cap);
-    HCHK(hipGetLastError());
-    HCHK(hipMemcpyAsync(m->h_out, m->d_out, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, m->stream));
+    static const bool no_direct = [] { const char *v = getenv("HIPDEC_NO_DIRECT_STEP"); return v && v[0] == '1'; }();
+    if (m->d_hout && !no_direct) {
+        // the kernel writes the pinned buffer itself: one launch and one wait, no copy behind it
+        hipLaunchKernelGGL(k_softcap_copy, dim3((n + 255) / 256), dim3(256), 0, m->stream, m->logits, m->d_hout, start, n, cap);
+        HCHK(hipGetLastError());
+    } else {
+        hipLaunchKernelGGL(k_softcap_copy, dim3((n + 255) / 256), dim3(256), 0, m->stream, m->logits, m->d_out, start, n, cap);
+        HCHK(hipGetLastError());
+        HCHK(hipMemcpyAsync(m->h_out, m->d_out, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, m->stream));
+    }
     SYNC_CHECKED(m);
     memcpy(host_out, m->h_out, (size_t)n * sizeof(float));
     return HIPDEC_OK;
@@ -1459,8 +1506,8 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
     HCHK(hipHostMalloc((void **)&m->h_samp, sizeof(SampleHost), hipHostMallocDefault));
     // abort flags of the persistent kernels: host memory the device writes through a mapping, so that the
     // host needs no copy of its own to look at them after a wait for the stream
-    HCHK(hipHostMalloc((void **)&m->h_abort, 128, hipHostMallocMapped));
-    memset(m->h_abort, 0, 128);
+    HCHK(hipHostMalloc((void **)&m->h_abort, 256, hipHostMallocMapped));
+    memset(m->h_abort, 0, 256);
     HCHK(hipHostGetDevicePointer((void **)&m->d_abort, m->h_abort, 0));
     (void)noalloc_scratch();              // (resolves this device's scratch array of hipdec_sample_fullvocab_noalloc outside any capture)
     // ---- persistent per-token kernel: exchange buffers, layer table, eligibility
@@ -1606,7 +1653,8 @@ static int create_impl(hipdec_model *m, const hipdec_layer_f32 *layers, const hi
     m->h_out_elems = V > 2 * (size_t)m->blocks * HIPDEC_MAX_GPU_TOPK ? V : 2 * (size_t)m->blocks * HIPDEC_MAX_GPU_TOPK;
     if (m->h_out_elems < S) m->h_out_elems = S;
     if (m->h_out_elems < D) m->h_out_elems = D;
-    HCHK(hipHostMalloc((void **)&m->h_out, m->h_out_elems * 4, hipHostMallocDefault));
+    HCHK(hipHostMalloc((void **)&m->h_out, m->h_out_elems * 4, hipHostMallocMapped));
+    if (hipHostGetDevicePointer((void **)&m->d_hout, m->h_out, 0) != hipSuccess) { m->d_hout = nullptr; (void)hipGetLastError(); }
     SYNC_CHECKED(m);
     return done(HIPDEC_OK);
 }
@@ -1835,7 +1883,7 @@ int hipdec_decode_token(hipdec_model *m, const float *x_in, float *x_out) {
     if ((rc = upload_x(m, x_in))) return rc;
     StepParams p = base_params(m, 0);
     p.use_x_in = 1;
-    if ((rc = step_with(m, V_X, 0, p))) return rc;
+    if ((rc = step_with(m, V_X, 0, p, true))) return rc;
     if ((rc = read_x(m, x_out))) return rc;
     m->len += 1;
     return HIPDEC_OK;
@@ -1845,13 +1893,19 @@ int hipdec_decode_token_from_id(hipdec_model *m, uint32_t token, float *x_out) {
     int rc = check_step(m, token, true);
     if (rc) return rc;
     if (!x_out) return fail(m, HIPDEC_ERR_ARG, "null buffer");
-    if ((rc = step_with(m, V_X, 0, base_params(m, token)))) return rc;
+    if ((rc = step_with(m, V_X, 0, base_params(m, token), true))) return rc;
     if ((rc = read_x(m, x_out))) return rc;
     m->len += 1;
     return HIPDEC_OK;
 }
 
 static int finish_argmax(hipdec_model *m, uint32_t *out_token) {
+    if (m->direct_step) {
+        SYNC_CHECKED(m);
+        *out_token = __atomic_load_n(m->h_abort + 48, __ATOMIC_ACQUIRE);
+        m->len += 1;
+        return HIPDEC_OK;
+    }
     HCHK(hipMemcpyAsync(m->h_out, m->d_ring, 4, hipMemcpyDeviceToHost, m->stream));
     SYNC_CHECKED(m);
     memcpy(out_token, m->h_out, 4);
@@ -1866,7 +1920,7 @@ int hipdec_decode_token_argmax(hipdec_model *m, const float *x_in, uint32_t *out
     if ((rc = upload_x(m, x_in))) return rc;
     StepParams p = base_params(m, 0);
     p.use_x_in = 1;
-    if ((rc = step_with(m, V_ARGMAX, 0, p))) return rc;
+    if ((rc = step_with(m, V_ARGMAX, 0, p, true))) return rc;
     return finish_argmax(m, out_token);
 }
 
@@ -1874,7 +1928,7 @@ int hipdec_decode_token_argmax_from_id(hipdec_model *m, uint32_t token, uint32_t
     int rc = check_step(m, token, true);
     if (rc) return rc;
     if (!out_token) return fail(m, HIPDEC_ERR_ARG, "null buffer");
-    if ((rc = step_with(m, V_ARGMAX, 0, base_params(m, token)))) return rc;
+    if ((rc = step_with(m, V_ARGMAX, 0, base_params(m, token), true))) return rc;
     return finish_argmax(m, out_token);
 }
 
@@ -1888,9 +1942,11 @@ int hipdec_decode_token_topk_from_id(hipdec_model *m, uint32_t token, uint32_t t
     if (!out_vals || !out_idxs || cap < count) return fail(m, HIPDEC_ERR_ARG, "output buffers too small for top-k candidates");
     StepParams p = base_params(m, token);
     p.top_k = (int)top_k;
-    if ((rc = step_with(m, V_TOPK, 0, p))) return rc;
-    HCHK(hipMemcpyAsync(m->h_out, m->d_topk_vals, count * 4, hipMemcpyDeviceToHost, m->stream));
-    HCHK(hipMemcpyAsync(m->h_out + count, m->d_topk_idxs, count * 4, hipMemcpyDeviceToHost, m->stream));
+    if ((rc = step_with(m, V_TOPK, 0, p, true))) return rc;
+    if (!m->direct_step) {
+        HCHK(hipMemcpyAsync(m->h_out, m->d_topk_vals, count * 4, hipMemcpyDeviceToHost, m->stream));
+        HCHK(hipMemcpyAsync(m->h_out + count, m->d_topk_idxs, count * 4, hipMemcpyDeviceToHost, m->stream));
+    }
     SYNC_CHECKED(m);
     memcpy(out_vals, m->h_out, count * 4);
     memcpy(out_idxs, m->h_out + count, count * 4);
@@ -1908,9 +1964,11 @@ int hipdec_decode_token_block_stats_from_id(hipdec_model *m, uint32_t token, flo
     StepParams p = base_params(m, token);
     p.inv_t = inv_temperature;
     p.softcap = softcap;
-    if ((rc = step_with(m, V_STATS, 0, p))) return rc;
-    HCHK(hipMemcpyAsync(m->h_out, m->d_bmax, B * 4, hipMemcpyDeviceToHost, m->stream));
-    HCHK(hipMemcpyAsync(m->h_out + B, m->d_bsum, B * 4, hipMemcpyDeviceToHost, m->stream));
+    if ((rc = step_with(m, V_STATS, 0, p, true))) return rc;
+    if (!m->direct_step) {
+        HCHK(hipMemcpyAsync(m->h_out, m->d_bmax, B * 4, hipMemcpyDeviceToHost, m->stream));
+        HCHK(hipMemcpyAsync(m->h_out + B, m->d_bsum, B * 4, hipMemcpyDeviceToHost, m->stream));
+    }
     SYNC_CHECKED(m);
     memcpy(out_maxes, m->h_out, B * 4);
     memcpy(out_sums, m->h_out + B, B * 4);
