@@ -9,8 +9,8 @@
 //    8 * (l / 16) .. + 8 of a 32-element step), and the R activation rows are the B operand, read
 //    from LDS as (hi, lo) bf16 pairs: columns 0..7 of the operand tile are the rows' hi parts,
 //    columns 8..15 their lo parts, so ONE instruction per weight load multiplies both (nothing is
-//    rounded to 8 bits).  The eight waves split the reduction axis; their 16 x 16 partial tiles meet
-//    in LDS, where the two halves of every result row are added;
+//    rounded to 8 bits; the two halves of a result row are added in registers).  The eight waves
+//    split the reduction axis; their 16 x 16 partial tiles meet in LDS;
 //  * a phase's weights are ONE round of loads per wave (at most 12 or 16 loads of 16 bytes per lane,
 //    which is what bounds the model sizes this kernel takes), requested in two halves, one and two
 //    phases ahead, into the register set the running phase does not use;
@@ -372,7 +372,7 @@ __global__ __launch_bounds__(ROWS_THREADS, 1) void k_rows(RowsArgs a) {
         const int spw = __builtin_amdgcn_readfirstlane(kinds[kind].spw), ntiles = __builtin_amdgcn_readfirstlane(kinds[kind].ntiles);
         // The 16 columns of the operand tile are the hi parts of the (at most 8) activation rows and, beside them,
         // their lo parts: one instruction per weight load multiplies both, and the two halves of a result row are
-        // added where the tiles are summed.  (Rows past R repeat row 0; their results are not read.)
+        // added before the tile goes to LDS.  (Rows past R repeat row 0; their results are not read.)
         const int nsrc = (r16 & 7) < R ? (r16 & 7) : 0;
         const uint16_t *pp = (r16 < 8 ? xh : xl) + nsrc * XS + wave * spw * 32 + c4 * 8;
 #pragma unroll
@@ -387,6 +387,10 @@ __global__ __launch_bounds__(ROWS_THREADS, 1) void k_rows(RowsArgs a) {
                         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, bx, acc, 0, 0, 0);
                     }
                 }
+                // columns n and n + 8 of a result row (the hi and lo parts' products) are 8 lanes apart: one rotation
+                // within the row of 16 lanes adds them
+                acc[0] += dpp_get<0x128, 0xf>(acc[0]); acc[1] += dpp_get<0x128, 0xf>(acc[1]);
+                acc[2] += dpp_get<0x128, 0xf>(acc[2]); acc[3] += dpp_get<0x128, 0xf>(acc[3]);
                 float *rp = red + (wave * ROWS_TA + t) * 256 + (4 * c4) * 16 + r16;
                 rp[0] = acc[0]; rp[16] = acc[1]; rp[32] = acc[2]; rp[48] = acc[3];
             }
@@ -399,7 +403,7 @@ __global__ __launch_bounds__(ROWS_THREADS, 1) void k_rows(RowsArgs a) {
 #pragma unroll
         for (int w = 0; w < ROWS_WAVES; ++w) {
             const float *rp = red + (w * ROWS_TA + t) * 256 + m * 16 + n;
-            s0 += rp[0] + rp[8]; s1 += rp[16] + rp[24];        // (columns n and n + 8: hi and lo parts' products)
+            s0 += rp[0]; s1 += rp[16];
         }
     };
     auto row_inv = [&](const int n) {
