@@ -35,16 +35,17 @@ WORKLOADS = {
     "c5_5b_int4_bs1": ("config_5b", "INT4_G128", "BF16", 512, 256),
     # 8 samples over one shared 512-token prompt, temperature 0.8, top-k 8, stepped together
     "c3_600m_bf16_8samples": ("config_600m", "BF16", "BF16", 512, 256),
-    # the same request on the 5B model with 4-bit weights (the multi-sample step as one kernel per product)
+    # the same request on the 5B model with 4-bit / 8-bit weights (the multi-sample step as one kernel per product)
     "c5_5b_int4_8samples": ("config_5b", "INT4_G128", "BF16", 512, 128),
+    "c5_5b_fp8_8samples": ("config_5b", "FP8_E4M3", "BF16", 512, 128),
 }
-MULTI_SAMPLE_WORKLOADS = ("c3_600m_bf16_8samples", "c5_5b_int4_8samples")
+MULTI_SAMPLE_WORKLOADS = ("c3_600m_bf16_8samples", "c5_5b_int4_8samples", "c5_5b_fp8_8samples")
 C3_SAMPLES, C3_TEMPERATURE, C3_TOP_K = 8, 0.8, 8
 ALL_CONFIG_ORDER = ["c1_tiny_fp32", "c2_600m_bf16_bs1", "c3_600m_bf16_8samples", "c4_5b_bf16_bs1", "c5_5b_fp8_bs1",
-                    "c5_5b_int4_bs1", "c5_5b_int4_8samples"]
+                    "c5_5b_int4_bs1", "c5_5b_int4_8samples", "c5_5b_fp8_8samples"]
 # timed steps of the short runs behind the all_configs entries (generated steps - 1 of the workload, capped)
 ALL_CONFIG_STEPS = {"c1_tiny_fp32": 31, "c2_600m_bf16_bs1": 255, "c3_600m_bf16_8samples": 64, "c4_5b_bf16_bs1": 32,
-                    "c5_5b_fp8_bs1": 64, "c5_5b_int4_bs1": 64, "c5_5b_int4_8samples": 32}
+                    "c5_5b_fp8_bs1": 64, "c5_5b_int4_bs1": 64, "c5_5b_int4_8samples": 32, "c5_5b_fp8_8samples": 32}
 
 # HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE + WRITE_SIZE, each
 # scaled by what the same counter reads for a plain copy of known size): measured separately with

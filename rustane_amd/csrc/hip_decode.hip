@@ -633,6 +633,11 @@ bool pf_use_skinny_i4() {
     return !off;
 }
 constexpr int kSkinnyI4WgsPerCu = 3;              // workgroups per CU its K splits aim at
+// the few-row GEMM of e4m3 models likewise (HIPDEC_NO_SKINNY_F8=1: the general few-row kernel)
+bool pf_use_skinny_f8(int K) {
+    static const bool off = [] { const char *v = getenv("HIPDEC_NO_SKINNY_F8"); return v && v[0] == '1'; }();
+    return !off && K % 64 == 0;
+}
 bool pf_use_dl(int wt, int T, int K, int act) {
     static const bool off = getenv("HIPDEC_NO_DL_GEMM") != nullptr;
     return !off && wt == WT_BF16 && T >= kDlMinRows && K % PF_BKL == 0 && act != PF_ACT_F16;
@@ -670,6 +675,17 @@ PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K, bool dl =
         if (gps >= 4) gps &= ~3;
         else if (max_groups >= 4) gps = 4;
         return PfSplit{(groups + gps - 1) / gps, 4 * gps};
+    }
+    if (T <= kSkinnyRows && wt == WT_FP8 && pf_use_skinny_f8(K)) {
+        // e4m3 weights: 64 weight rows per workgroup, every wave walks the whole K range of its split, a split is a
+        // whole number of 64-element blocks, a multiple of eight of them (one round of loads) where that fits
+        const int tiles = (N + 63) / 64, blocks = K / 64;
+        const int s = std::max(1, (kSkinnyI4WgsPerCu * m->num_cu + tiles - 1) / tiles);
+        const int max_blocks = std::max(1, ((kSkinnyLdsBytes / (4 * T)) - PF_SK_PAD) / 64);
+        int bps = std::min(max_blocks, std::max(1, (blocks + s - 1) / s));
+        if (bps >= 8) bps &= ~7;
+        else if (max_blocks >= 8) bps = 8;
+        return PfSplit{(blocks + bps - 1) / bps, 2 * bps};
     }
     if (T <= kSkinnyRows) {
         // 4 waves per workgroup share a K range; aim at ~8 waves per CU over the whole grid
@@ -753,6 +769,14 @@ int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, c
         if (T <= 8) hipLaunchKernelGGL((k_pf_gemm_skinny_i4<1, true, kSkinnyI4Nt>), grid, block, lds, m->stream, g);
         else if (rt == 1) hipLaunchKernelGGL((k_pf_gemm_skinny_i4<1, false, kSkinnyI4Nt>), grid, block, lds, m->stream, g);
         else hipLaunchKernelGGL((k_pf_gemm_skinny_i4<2, false, kSkinnyI4Nt>), grid, block, lds, m->stream, g);
+        return sp.splits;
+    }
+    if (T <= kSkinnyRows && wt == WT_FP8 && pf_use_skinny_f8(K)) {
+        dim3 grid((N + 63) / 64, sp.splits), block(256);
+        const size_t lds = (size_t)2 * T * (sp.steps_per_split * PF_BK + PF_SK_PAD) * 2;
+        if (T <= 8) hipLaunchKernelGGL((k_pf_gemm_skinny_f8<1, true>), grid, block, lds, m->stream, g);
+        else if (T <= 16) hipLaunchKernelGGL((k_pf_gemm_skinny_f8<1, false>), grid, block, lds, m->stream, g);
+        else hipLaunchKernelGGL((k_pf_gemm_skinny_f8<2, false>), grid, block, lds, m->stream, g);
         return sp.splits;
     }
     if (T <= kSkinnyRows) {

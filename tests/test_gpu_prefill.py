@@ -94,6 +94,14 @@ def test_few_row_products_of_4bit_weights(n_prompt):
     check_prefill_then_decode(cfg, n_prompt, 1e-4, wdt=WeightDtype.INT4_G128, kvdt=KvDtype.F32, std=0.05)
 
 
+@pytest.mark.parametrize("n_prompt", [6, 8, 14, 31])
+def test_few_row_products_of_e4m3_weights(n_prompt):
+    # prompts of at most 32 rows of an e4m3 model go through the few-row GEMM written for that format (reductions
+    # that are multiples of 64: dim 384, q_dim 512, hidden 1152 = 18 blocks, i.e. rounds and splits that end early)
+    cfg = Config.make(dim=384, hidden=1152, heads=4, hd=128, seq=64, nlayers=3, vocab=768, kv_heads=2)
+    check_prefill_then_decode(cfg, n_prompt, 1e-4, wdt=WeightDtype.FP8_E4M3, kvdt=KvDtype.F32, std=0.05)
+
+
 def test_prefill_int4_matches_token_step_prefill():
     cfg = Config.make(dim=384, hidden=1152, heads=3, hd=128, seq=200, nlayers=3, vocab=1024)
     w = synth.make_weights(cfg, seed=5, std=0.06, round_bf16=True)
