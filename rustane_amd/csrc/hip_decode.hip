@@ -626,7 +626,8 @@ constexpr int kSkinnyLdsBytes = 40 * 1024;   // dynamic LDS for the staged activ
 // 128 x 256 tiles, whole 64-element steps, activations as bf16 (pair or single)
 constexpr int kDlMinRows = 129;
 constexpr int kSkinnyI4Nt = 1;                    // 16-row weight tiles per wave of k_pf_gemm_skinny_i4 (2: 4 - 8 % slower on the 5B shapes)
-constexpr int kSkinnyI4Bn = 64 * kSkinnyI4Nt;     // weight rows per workgroup
+constexpr int kSkinnyI4Waves = 8;                 // waves per workgroup (4: as fast at 9+ rows, 5 - 15 % slower at 8)
+constexpr int kSkinnyI4Bn = 16 * kSkinnyI4Nt * kSkinnyI4Waves;   // weight rows per workgroup
 // the few-row GEMM of 4-bit models: the kernel of its own (HIPDEC_NO_SKINNY_I4=1: the general few-row kernel)
 bool pf_use_skinny_i4() {
     static const bool off = [] { const char *v = getenv("HIPDEC_NO_SKINNY_I4"); return v && v[0] == '1'; }();
@@ -670,7 +671,7 @@ PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K, bool dl =
         // reads a round's four scales of a row as one aligned load).  Aim at a few workgroups per CU.
         const int tiles = (N + kSkinnyI4Bn - 1) / kSkinnyI4Bn, groups = K / 128;
         int s = std::max(1, (kSkinnyI4WgsPerCu * m->num_cu + tiles - 1) / tiles);
-        const int max_groups = std::max(1, ((kSkinnyLdsBytes / (4 * T)) - PF_SK_PAD) / 128);
+        const int max_groups = std::min(PF_SQ_GU, std::max(1, ((kSkinnyLdsBytes / (4 * T)) - PF_SK_PAD) / 128));
         int gps = std::min(max_groups, std::max(1, (groups + s - 1) / s));
         if (gps >= 4) gps &= ~3;
         else if (max_groups >= 4) gps = 4;
@@ -764,11 +765,11 @@ int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, c
     PfGemm g{Ahi, Alo, W, wt == WT_INT4 ? (const uint16_t *)scales : nullptr, m->pf.P, T, N, K, sp.steps_per_split};
     if (T <= kSkinnyRows && wt == WT_INT4 && pf_use_skinny_i4()) {
         const int rt = T <= 16 ? 1 : 2;
-        dim3 grid((N + kSkinnyI4Bn - 1) / kSkinnyI4Bn, sp.splits), block(256);
-        const size_t lds = (size_t)2 * T * (sp.steps_per_split * PF_BK + PF_SK_PAD) * 2 + (size_t)(sp.steps_per_split / 4) * 16 * rt * 4;
-        if (T <= 8) hipLaunchKernelGGL((k_pf_gemm_skinny_i4<1, true, kSkinnyI4Nt>), grid, block, lds, m->stream, g);
-        else if (rt == 1) hipLaunchKernelGGL((k_pf_gemm_skinny_i4<1, false, kSkinnyI4Nt>), grid, block, lds, m->stream, g);
-        else hipLaunchKernelGGL((k_pf_gemm_skinny_i4<2, false, kSkinnyI4Nt>), grid, block, lds, m->stream, g);
+        dim3 grid((N + kSkinnyI4Bn - 1) / kSkinnyI4Bn, sp.splits), block(64 * kSkinnyI4Waves);
+        const size_t lds = (size_t)2 * T * (sp.steps_per_split * PF_BK + PF_SK_PAD) * 2;
+        if (T <= 8) hipLaunchKernelGGL((k_pf_gemm_skinny_i4<1, true, kSkinnyI4Nt, kSkinnyI4Waves>), grid, block, lds, m->stream, g);
+        else if (rt == 1) hipLaunchKernelGGL((k_pf_gemm_skinny_i4<1, false, kSkinnyI4Nt, kSkinnyI4Waves>), grid, block, lds, m->stream, g);
+        else hipLaunchKernelGGL((k_pf_gemm_skinny_i4<2, false, kSkinnyI4Nt, kSkinnyI4Waves>), grid, block, lds, m->stream, g);
         return sp.splits;
     }
     if (T <= kSkinnyRows && wt == WT_FP8 && pf_use_skinny_f8(K)) {

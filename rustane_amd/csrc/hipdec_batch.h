@@ -32,11 +32,9 @@ __global__ __launch_bounds__(256) void k_bd_qkv_epi(const float *__restrict__ P,
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= (size_t)R * npairs) return;
     const int t = (int)(gid / npairs), p = (int)(gid - (size_t)t * npairs), row0 = 2 * p;
-    float s0 = 0.0f, s1 = 0.0f;
-    for (int z = 0; z < splits; ++z) {
-        const float2 v = *(const float2 *)(P + z * plane + (size_t)t * N + row0);
-        s0 += v.x; s1 += v.y;
-    }
+    float sv[2] = {0.0f, 0.0f};
+    pf_sum_planes<2>(P, splits, plane, (size_t)t * N + row0, sv);
+    float s0 = sv[0], s1 = sv[1];
     if (wscale) { s0 *= wscale[row0]; s1 *= wscale[row0 + 1]; }
     const float inv = pf_row_inv(ssq, t, nch, D);
     s0 *= inv; s1 *= inv;
@@ -165,7 +163,7 @@ __global__ __launch_bounds__(256) void k_bd_sum_planes(const float *__restrict__
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     float s = 0.0f;
-    for (int z = 0; z < splits; ++z) s += P[z * plane + i];
+    pf_sum_planes<1>(P, splits, plane, i, &s);
     out[i] = s * pf_row_inv(ssq, (int)(i / V), nch, D);
 }
 

@@ -38,6 +38,31 @@ __device__ __forceinline__ float wave_sum(float v) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
     return v;
 }
+
+// Sum over the 64 lanes of a wave with data-parallel-primitive moves (no LDS round trips);
+// the total is valid in lane 63.  Fixed order: quads, halves of 8, rows of 16, then the rows.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_get(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v += dpp_get<0xB1, 0xf>(v);      // quad_perm [1,0,3,2]
+    v += dpp_get<0x4E, 0xf>(v);      // quad_perm [2,3,0,1]
+    v += dpp_get<0x141, 0xf>(v);     // row_half_mirror
+    v += dpp_get<0x140, 0xf>(v);     // row_mirror: every lane of a row now holds the row's sum
+    v += dpp_get<0x142, 0xa>(v);     // row_bcast:15 into rows 1 and 3
+    v += dpp_get<0x143, 0xc>(v);     // row_bcast:31 into rows 2 and 3
+    return v;
+}
+// sum over aligned groups of N lanes (8, 16 or 32); every lane of the group receives it
+template <int N> __device__ __forceinline__ float group_sum_dpp(float v) {
+    v += dpp_get<0xB1, 0xf>(v);
+    v += dpp_get<0x4E, 0xf>(v);
+    v += dpp_get<0x141, 0xf>(v);
+    if (N >= 16) v += dpp_get<0x140, 0xf>(v);
+    if (N >= 32) v += __shfl_xor(v, 16, WAVE);
+    return v;
+}
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));

@@ -75,7 +75,14 @@ __device__ __forceinline__ float pf_block_sum(float v, float *red) {
 #define PF_CHUNK 256
 __device__ __forceinline__ float pf_row_inv(const float *__restrict__ ssq, int t, int nch, int D) {
     float s = 0.0f;
-    for (int c = 0; c < nch; ++c) s += ssq[t * nch + c];
+    for (int c = 0; c < nch; c += 8) {                   // eight loads in flight, added in chunk order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = ssq[t * nch + min(c + u, nch - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (c + u < nch) s += v[u];
+    }
     return 1.0f / sqrtf(s * (1.0f / (float)D) + 1e-5f);
 }
 
@@ -89,6 +96,32 @@ __device__ __forceinline__ float pf_row_part(const float *__restrict__ ssq, int 
 }
 __device__ __forceinline__ float pf_row_finish(float part, int D) {
     return 1.0f / sqrtf(wave_sum(part) * (1.0f / (float)D) + 1e-5f);
+}
+
+// s[0..W) += sum over the split planes of the W floats at offset o, in plane order.  U planes are
+// requested at a time (past the last plane the last one is requested again and not added): a loop
+// of one load and one add per plane is a chain of `splits` round trips to the L2, which is what
+// these small kernels' run time consists of.
+template <int W, int U>
+__device__ __forceinline__ void pf_sum_planes_u(const float *__restrict__ P, int splits, size_t plane, size_t o, float *s) {
+    typedef float vt __attribute__((ext_vector_type(W)));
+    for (int z = 0; z < splits; z += U) {
+        vt p[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) p[u] = *(const vt *)(P + (size_t)min(z + u, splits - 1) * plane + o);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (z + u < splits) {
+#pragma unroll
+                for (int e = 0; e < W; ++e) s[e] += p[u][e];
+            }
+        }
+    }
+}
+template <int W>
+__device__ __forceinline__ void pf_sum_planes(const float *__restrict__ P, int splits, size_t plane, size_t o, float *s) {
+    if (splits > 4) pf_sum_planes_u<W, 8>(P, splits, plane, o, s);
+    else pf_sum_planes_u<W, 4>(P, splits, plane, o, s);
 }
 
 // x[t] = embed[ids[t]] (cpu/embedding.rs:8-16); hi/lo = x * gamma1 of the first layer; chunk sums of squares.
@@ -124,11 +157,9 @@ __global__ __launch_bounds__(256) void k_pf_resid(const float *__restrict__ P, i
     float ss = 0.0f;
     if (d < D) {
         const size_t o = (size_t)t * D + d;
-        float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        for (int z = 0; z < splits; ++z) {
-            const float4 p = *(const float4 *)(P + z * plane + o);
-            s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
-        }
+        float sv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        pf_sum_planes<4>(P, splits, plane, o, sv);
+        float4 s = make_float4(sv[0], sv[1], sv[2], sv[3]);
         if (wscale) {
             const float4 ws = *(const float4 *)(wscale + d);
             s.x *= ws.x; s.y *= ws.y; s.z *= ws.z; s.w *= ws.w;
@@ -166,10 +197,7 @@ __global__ __launch_bounds__(256) void k_pf_qkv_epi(const float *__restrict__ P,
     const float part = pf_row_part(ssq, t, nch);
     float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (row0 < N) {
-        for (int z = 0; z < splits; ++z) {
-            const float4 v = *(const float4 *)(P + z * plane + (size_t)t * N + row0);
-            s[0] += v.x; s[1] += v.y; s[2] += v.z; s[3] += v.w;
-        }
+        pf_sum_planes<4>(P, splits, plane, (size_t)t * N + row0, s);
     }
     const float inv = pf_row_finish(part, D);
     if (row0 >= N) return;
@@ -218,11 +246,9 @@ __global__ __launch_bounds__(256) void k_pf_gate_epi(const float *__restrict__ P
     const float part = pf_row_part(ssq, t, nch);
     float h[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     if (j < H) {
-        for (int z = 0; z < splits; ++z) {
-            const float4 a = *(const float4 *)(P + z * plane + (size_t)t * 2 * H + 2 * j);
-            const float4 b = *(const float4 *)(P + z * plane + (size_t)t * 2 * H + 2 * j + 4);
-            h[0] += a.x; h[1] += a.y; h[2] += a.z; h[3] += a.w; h[4] += b.x; h[5] += b.y; h[6] += b.z; h[7] += b.w;
-        }
+        // (two requests of 16 bytes per plane, four planes at a time)
+        pf_sum_planes_u<4, 4>(P, splits, plane, (size_t)t * 2 * H + 2 * j, h);
+        pf_sum_planes_u<4, 4>(P, splits, plane, (size_t)t * 2 * H + 2 * j + 4, h + 4);
     }
     const float inv = pf_row_finish(part, D);
     if (j >= H) return;
@@ -860,36 +886,40 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
 // row, so one load instruction touches 32 rows for 16 bytes each, a workgroup streams 16 KB of weights against
 // 32 KB of staged activations, and every nibble costs five to six vector instructions on its way to bf16: the
 // 5B model's products of 8 rows ran at 0.7 - 1.6 TB/s (28 / 17 / 17 / 8 us for the gate-up, down, q/k/v and output
-// projections; this kernel: 18.5 / 12.4 / 7.7 / 6.1 us stand-alone).  Here
+// projections).  Here
 //  * the products are v_mfma_f32_16x16x32_bf16: lane (n = l % 16, kg = l / 16) holds weight row n and the 32
 //    elements kg of a 128-element scale group -- ONE 16-byte load, and the four lanes of a row read 64
 //    contiguous bytes; dword j of the load is the lane's 8 elements of matrix instruction j of the group;
-//  * a wave owns NT tiles of 16 weight rows and walks the workgroup's whole K range, the four waves share the
+//  * a wave owns NT tiles of 16 weight rows and walks the workgroup's whole K range, the WAVES waves share the
 //    staged activations and nothing is reduced across waves;
 //  * a nibble n' (offset binary) becomes the bf16 number 16 + n' with two instructions per PAIR: the nibbles
-//    j and j + 4 of a dword are shifted into mantissa bits 3..6 of the two halves of 0x41804180.  The
-//    activations are staged in the matching order (elements 0 4 1 5 2 6 3 7 of every eight), and since
-//    16 + n' = 24 + (n' - 8) the group's sum of activations, worked out while staging, leaves the result as
-//    24 times that sum before the group's scale is applied (all in fp32);
+//    j and j + 4 of a dword are shifted into mantissa bits 3..6 of the two halves of 0x41804180 (one shift, one
+//    and-or).  The activations are staged in the matching order (elements 0 4 1 5 2 6 3 7 of every eight), and
+//    since 16 + n' = 24 + (n' - 8) every group's activations are also multiplied by a tile of -24s on the
+//    matrix cores, which are idle otherwise: the two result tiles add up to the product with n' - 8 before the
+//    group's scale is applied (all in fp32);
 //  * PACK (at most 8 activation rows): the hi parts are rows 0..7 and the lo parts rows 8..15 of ONE operand
 //    tile, so a weight fragment is multiplied once, not twice; the two halves of the result tile (lanes 32
-//    apart) are added at the end, which is exact in the same sense as summing the two products' tiles.
-#define PF_SQ_GU 4                       // scale groups per wave and tile whose loads are issued together
+//    apart) are added at the end, which is exact in the same sense as summing the two products' tiles;
+//  * a workgroup lives for a few microseconds, all of them at the same time, so what it does before its first
+//    matrix instruction is on the critical path of the launch: the staging loop has no integer division, no
+//    sums and no cross-lane traffic, and the weights of the split's whole K range are requested before it (the
+//    host keeps a split within PF_SQ_GU groups).
+#define PF_SQ_GU 8                       // scale groups of a split: what a wave requests per tile, all at once
 typedef float pf_f32x4 __attribute__((ext_vector_type(4)));
-template <int RT, bool PACK, int NT>     // RT tiles of 16 activation rows (T <= 16 RT; PACK: T <= 8, RT = 1); NT weight tiles per wave
-__global__ __launch_bounds__(256) void k_pf_gemm_skinny_i4(PfGemm g) {
+template <int RT, bool PACK, int NT, int WAVES>   // RT tiles of 16 activation rows (T <= 16 RT; PACK: T <= 8, RT = 1); NT weight tiles per wave
+__global__ __launch_bounds__(64 * WAVES) void k_pf_gemm_skinny_i4(PfGemm g) {
     static_assert(!PACK || RT == 1, "packed planes are one row tile");
-    constexpr int XS = PACK ? 16 : 16 * RT;                // sums per group: [hi rows | lo rows] (PACK) or rows
-    extern __shared__ __align__(16) uint16_t s_act[];      // [2][T][astride] bf16, then [groups][XS] sums
+    constexpr int NTHR = 64 * WAVES;
+    extern __shared__ __align__(16) uint16_t s_act[];      // [2][T][astride] bf16
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kg = lane >> 4;
-    const int n0 = blockIdx.x * (64 * NT) + wave * (16 * NT), z = blockIdx.y;
+    const int n0 = blockIdx.x * (16 * NT * WAVES) + wave * (16 * NT), z = blockIdx.y;
     const int nsteps = g.K / PF_BK;
     const int zb = z * g.steps_per_split, ze = min(nsteps, zb + g.steps_per_split);
     const int g_begin = zb / 4, g_end = ze / 4;            // (the host makes every split a whole number of groups)
     const int krange = (ze - zb) * PF_BK, astride = g.steps_per_split * PF_BK + PF_SK_PAD;
     const int kgrp = g.K / 128;
-    float *s_xsum = (float *)(s_act + 2 * g.T * astride);
 
     const char *wrow[NT];
     const uint16_t *srow[NT];
@@ -899,79 +929,69 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny_i4(PfGemm g) {
         wrow[nt] = (const char *)g.W + row * (size_t)(g.K / 2) + 16 * kg;
         srow[nt] = g.S + row * (size_t)kgrp;
     }
-    // a round of PF_SQ_GU groups per tile in flight; sc: the round's four scales of a row
+    // slot u holds the split's group u; sc0[q]: the four scales of slots 4q .. 4q+3
     uint4 w0[PF_SQ_GU][NT];
-    uint2 sc0[NT];
-    auto wload = [&](uint4 (&w)[PF_SQ_GU][NT], uint2 (&sc)[NT], int gi) {
+    uint2 sc0[PF_SQ_GU / 4][NT];
+    auto wload = [&](const int u, const int gg) {
 #pragma unroll
-        for (int u = 0; u < PF_SQ_GU; ++u) {
-            const int gg = min(gi + u, g_end - 1);            // a padded group re-reads the last one (and is skipped below)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) w[u][nt] = *(const uint4 *)(wrow[nt] + (size_t)gg * 64);
-        }
-        // scales: a row's four of the round as one load (rounds start at multiples of four groups); where fewer
-        // than four are left in the row the load starts earlier and is shifted
-        if (kgrp >= PF_SQ_GU) {
-            const int gq = min(gi, kgrp - 1), gs = min(gq, kgrp - PF_SQ_GU), sh = 16 * (gq - gs);
+        for (int nt = 0; nt < NT; ++nt) w0[u][nt] = *(const uint4 *)(wrow[nt] + (size_t)gg * 64);
+    };
+    // scales: a row's four from group gi on as one load (gi is a multiple of four groups from the split's first,
+    // which is one from the row's first); where fewer than four are left in the row the load starts earlier and
+    // is shifted
+    auto sload = [&](const int q, const int gi) {
+        if (kgrp >= 4) {
+            const int gs = min(gi, kgrp - 4), sh = 16 * (gi - gs);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const uint2 v = *(const uint2 *)(srow[nt] + gs);
                 const unsigned long long x = (((unsigned long long)v.y << 32) | v.x) >> sh;
-                sc[nt] = make_uint2((uint32_t)x, (uint32_t)(x >> 32));
+                sc0[q][nt] = make_uint2((uint32_t)x, (uint32_t)(x >> 32));
             }
         } else {                                              // a reduction of fewer than four groups
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const uint32_t s0 = srow[nt][min(gi, kgrp - 1)], s1 = srow[nt][min(gi + 1, kgrp - 1)], s2 = srow[nt][min(gi + 2, kgrp - 1)];
-                sc[nt] = make_uint2(s0 | (s1 << 16), s2);
+                sc0[q][nt] = make_uint2(s0 | (s1 << 16), s2);
             }
         }
     };
-    // The activation rows [0, T) x this workgroup's K range are requested first and the first round of weights
-    // behind them, so that staging waits for its own loads only.  Staged: every eight elements as 0 4 1 5 2 6 3 7,
-    // and the sums of every (row, group): a group is 16 chunks, held by 16 neighbouring threads.
+    // The activation rows [0, T) x this workgroup's K range are requested first and the weights behind them, so
+    // that staging waits for its own loads only.  Staged: every eight elements as 0 4 1 5 2 6 3 7.
     {
-        constexpr int MAXIT = 5;                               // 40 KB of staged rows: at most 1280 chunks of hi and lo
-        const int cpr = krange / 8, items = g.T * cpr;         // (cpr is a multiple of 16)
+        constexpr int MAXIT = (1280 + NTHR - 1) / NTHR;        // 40 KB of staged rows: at most 1280 chunks of hi and lo
+        const int cpr = krange / 8, items = g.T * cpr;         // (cpr is a multiple of 16, items at most 1280)
+        const float rcp = 1.0f / (float)cpr;
         uint4 hh[MAXIT], ll[MAXIT];
+        int dst[MAXIT];
 #pragma unroll
         for (int it = 0; it < MAXIT; ++it) {
-            const int cc = min(it * 256 + tid, items - 1);
-            const int t = cc / cpr, kc = cc - t * cpr;
-            const size_t src = (size_t)t * g.K + (size_t)zb * PF_BK + kc * 8;
-            hh[it] = *(const uint4 *)(g.Ahi + src); ll[it] = *(const uint4 *)(g.Alo + src);
+            if (it * NTHR < items) {
+                const int cc = min(it * NTHR + tid, items - 1);
+                // cc / cpr without the division: the quotient's fraction is a multiple of 1 / cpr >= 1 / 1280, the
+                // half chunk added keeps it that far from the next integer, the rounding errors are below 1e-5
+                const int t = (int)(((float)cc + 0.5f) * rcp), kc = cc - t * cpr;
+                const size_t src = (size_t)t * g.K + (size_t)zb * PF_BK + kc * 8;
+                hh[it] = *(const uint4 *)(g.Ahi + src); ll[it] = *(const uint4 *)(g.Alo + src);
+                dst[it] = t * astride + kc * 8;
+            }
         }
-        wload(w0, sc0, g_begin);
+#pragma unroll
+        for (int u = 0; u < PF_SQ_GU; ++u)
+            if (g_begin + u < g_end) wload(u, g_begin + u);
+#pragma unroll
+        for (int q = 0; q < PF_SQ_GU / 4; ++q)
+            if (g_begin + 4 * q < g_end) sload(q, g_begin + 4 * q);
 #pragma unroll
         for (int it = 0; it < MAXIT; ++it) {
-            const int c = it * 256 + tid;
-            const bool in = c < items;
-            const int cc = min(c, items - 1);
-            const int t = cc / cpr, kc = cc - t * cpr;
-            const uint4 h = hh[it], l = ll[it];
-            if (in) {
-                *(uint4 *)(s_act + t * astride + kc * 8) =
-                    make_uint4((h.x & 0xffffu) | (h.z << 16), (h.x >> 16) | (h.z & 0xffff0000u), (h.y & 0xffffu) | (h.w << 16), (h.y >> 16) | (h.w & 0xffff0000u));
-                *(uint4 *)(s_act + (g.T + t) * astride + kc * 8) =
-                    make_uint4((l.x & 0xffffu) | (l.z << 16), (l.x >> 16) | (l.z & 0xffff0000u), (l.y & 0xffffu) | (l.w << 16), (l.y >> 16) | (l.w & 0xffff0000u));
-            }
-            const uint32_t hv[4] = {h.x, h.y, h.z, h.w}, lv[4] = {l.x, l.y, l.z, l.w};
-            float sh = 0.0f, sl = 0.0f;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                sh += __uint_as_float(hv[i] << 16) + __uint_as_float(hv[i] & 0xffff0000u);
-                sl += __uint_as_float(lv[i] << 16) + __uint_as_float(lv[i] & 0xffff0000u);
-            }
-            if (!PACK) { sh += sl; sl = 0.0f; }
-#pragma unroll
-            for (int o = 1; o < 16; o <<= 1) {
-                sh += __shfl_xor(sh, o, 64);
-                if (PACK) sl += __shfl_xor(sl, o, 64);
-            }
-            if (in && (tid & 15) == 0) {
-                const int gl = kc >> 4;
-                s_xsum[gl * XS + t] = sh;
-                if (PACK) s_xsum[gl * XS + 8 + t] = sl;
+            if (it * NTHR < items && it * NTHR + tid < items) {
+                const uint4 h = hh[it], l = ll[it];
+                *(uint4 *)(s_act + dst[it]) =
+                    make_uint4(__builtin_amdgcn_perm(h.z, h.x, 0x05040100u), __builtin_amdgcn_perm(h.z, h.x, 0x07060302u),
+                               __builtin_amdgcn_perm(h.w, h.y, 0x05040100u), __builtin_amdgcn_perm(h.w, h.y, 0x07060302u));
+                *(uint4 *)(s_act + g.T * astride + dst[it]) =
+                    make_uint4(__builtin_amdgcn_perm(l.z, l.x, 0x05040100u), __builtin_amdgcn_perm(l.z, l.x, 0x07060302u),
+                               __builtin_amdgcn_perm(l.w, l.y, 0x05040100u), __builtin_amdgcn_perm(l.w, l.y, 0x07060302u));
             }
         }
     }
@@ -988,70 +1008,65 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny_i4(PfGemm g) {
             al[rt] = ah[rt] + g.T * astride;
         }
     }
+    // the unpacking constants live in registers: as literals each pair would cost an "and" and an "or"
+    uint32_t nib_mask, nib_bias, m24;
+    asm volatile("s_mov_b32 %0, 0x00780078" : "=s"(nib_mask));
+    asm volatile("v_mov_b32 %0, 0x41804180" : "=v"(nib_bias));
+    asm volatile("v_mov_b32 %0, 0xc1c0c1c0" : "=v"(m24));              // two bf16 numbers -24
+    const pf_bf16x8 BC = __builtin_bit_cast(pf_bf16x8, make_uint4(m24, m24, m24, m24));
     pf_f32x4 acc[RT][NT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = pf_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    auto round = [&](const uint4 (&wc)[PF_SQ_GU][NT], const uint2 (&scc)[NT], const int gi) {
+    // group gl (counted from the split's first) out of slot u
+    auto group = [&](const int u, const int gl) {
+        pf_f32x4 ag[RT][NT], cg[RT];
 #pragma unroll
-        for (int u = 0; u < PF_SQ_GU; ++u) {
-            if (gi + u < g_end) {
-                const int gl = gi + u - g_begin;
-                pf_f32x4 ag[RT][NT];
+        for (int rt = 0; rt < RT; ++rt) {
+            cg[rt] = pf_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt)
+            for (int nt = 0; nt < NT; ++nt) ag[rt][nt] = pf_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) ag[rt][nt] = pf_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int j = 0; j < 4; ++j) {
+            uint4 xh[RT], xl[RT];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    uint4 xh[RT], xl[RT];
+            for (int rt = 0; rt < RT; ++rt) {
+                xh[rt] = *(const uint4 *)(ah[rt] + gl * 128 + 8 * j);
+                if (!PACK) xl[rt] = *(const uint4 *)(al[rt] + gl * 128 + 8 * j);
+            }
 #pragma unroll
-                    for (int rt = 0; rt < RT; ++rt) {
-                        xh[rt] = *(const uint4 *)(ah[rt] + gl * 128 + 8 * j);
-                        if (!PACK) xl[rt] = *(const uint4 *)(al[rt] + gl * 128 + 8 * j);
-                    }
+            for (int rt = 0; rt < RT; ++rt) {
+                cg[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, xh[rt]), BC, cg[rt], 0, 0, 0);
+                if (!PACK) cg[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, xl[rt]), BC, cg[rt], 0, 0, 0);
+            }
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-                        const uint32_t q = j == 0 ? wc[u][nt].x : j == 1 ? wc[u][nt].y : j == 2 ? wc[u][nt].z : wc[u][nt].w;
-                        const uint4 b = make_uint4(((q << 3) & 0x00780078u) | 0x41804180u, ((q >> 1) & 0x00780078u) | 0x41804180u,
-                                                   ((q >> 5) & 0x00780078u) | 0x41804180u, ((q >> 9) & 0x00780078u) | 0x41804180u);
-                        const pf_bf16x8 B = __builtin_bit_cast(pf_bf16x8, b);
-#pragma unroll
-                        for (int rt = 0; rt < RT; ++rt) {
-                            ag[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, xh[rt]), B, ag[rt][nt], 0, 0, 0);
-                            if (!PACK) ag[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, xl[rt]), B, ag[rt][nt], 0, 0, 0);
-                        }
-                    }
-                }
+            for (int nt = 0; nt < NT; ++nt) {
+                const uint32_t q = j == 0 ? w0[u][nt].x : j == 1 ? w0[u][nt].y : j == 2 ? w0[u][nt].z : w0[u][nt].w;
+                const uint4 b = make_uint4(((q << 3) & nib_mask) | nib_bias, ((q >> 1) & nib_mask) | nib_bias,
+                                           ((q >> 5) & nib_mask) | nib_bias, ((q >> 9) & nib_mask) | nib_bias);
+                const pf_bf16x8 B = __builtin_bit_cast(pf_bf16x8, b);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
-                    const float4 xs = *(const float4 *)(s_xsum + gl * XS + 16 * rt + 4 * kg);
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-                        const uint32_t sw = u < 2 ? scc[nt].x : scc[nt].y;
-                        const float scale = __uint_as_float((u & 1) ? (sw & 0xffff0000u) : (sw << 16));
-                        acc[rt][nt][0] = fmaf(fmaf(-24.0f, xs.x, ag[rt][nt][0]), scale, acc[rt][nt][0]);
-                        acc[rt][nt][1] = fmaf(fmaf(-24.0f, xs.y, ag[rt][nt][1]), scale, acc[rt][nt][1]);
-                        acc[rt][nt][2] = fmaf(fmaf(-24.0f, xs.z, ag[rt][nt][2]), scale, acc[rt][nt][2]);
-                        acc[rt][nt][3] = fmaf(fmaf(-24.0f, xs.w, ag[rt][nt][3]), scale, acc[rt][nt][3]);
-                    }
+                    ag[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, xh[rt]), B, ag[rt][nt], 0, 0, 0);
+                    if (!PACK) ag[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, xl[rt]), B, ag[rt][nt], 0, 0, 0);
                 }
             }
         }
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const uint32_t sw = (u & 2) ? sc0[u >> 2][nt].y : sc0[u >> 2][nt].x;
+                const float scale = __uint_as_float((u & 1) ? (sw & 0xffff0000u) : (sw << 16));
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[rt][nt][i] = fmaf(ag[rt][nt][i] + cg[rt][i], scale, acc[rt][nt][i]);
+            }
     };
-    for (int gi = g_begin; gi < g_end; gi += PF_SQ_GU) {
-        uint4 wc[PF_SQ_GU][NT];
-        uint2 scc[NT];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            scc[nt] = sc0[nt];
-#pragma unroll
-            for (int u = 0; u < PF_SQ_GU; ++u) wc[u][nt] = w0[u][nt];
-        }
-        if (gi + PF_SQ_GU < g_end) wload(w0, sc0, gi + PF_SQ_GU);      // the next round in flight while this one multiplies
-        round(wc, scc, gi);
-    }
+    for (int u = 0; u < PF_SQ_GU; ++u)
+        if (g_begin + u < g_end) group(u, u);
     // lane (n, kg) holds rows 16 rt + 4 kg + i of column n of each tile (PACK: kg 0, 1 the hi parts' products of
     // rows 4 kg + i, kg 2, 3 the lo parts' of rows 4 (kg - 2) + i)
     float *Pz = g.P + (size_t)z * g.T * g.N;
