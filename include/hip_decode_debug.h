@@ -62,6 +62,17 @@ int hipdec_debug_hostmath_count_mismatch(int fn, uint32_t first_bits, uint64_t c
  * 512 (hipdec_lean.h).  Environment HIPDEC_NO_LEAN=1 / HIPDEC_NO_MEGA=1 at creation select the earlier forms. */
 int hipdec_debug_step_kernel(const hipdec_model *m, int *out);
 
+/* The launch of one product P[splits][rows][n] = A[rows][k] x W[n][k]^T of the prompt prefill and the
+ * multi-row step on a device of num_cu compute units, worked out on the host (no GPU needed): out[0] the
+ * kernel (0 tiled, 1 tiled with its operands loaded straight into LDS, 2 few-row, 3 few-row for 4-bit
+ * weights, 4 few-row for e4m3 weights), out[1] the K splits (planes written), out[2] the reduction steps per
+ * split (32 elements each in the few-row kernels, 64 in the tiled ones), out[3..5] the grid, out[6] the
+ * threads per workgroup, out[7] the dynamic LDS bytes.  It is the plan the library's own launches follow;
+ * tests check it against what the kernels assume (whole scale groups per split, the staged rows within the
+ * LDS budget, no empty split).  HIPDEC_ERR_ARG for shapes the library never launches (k not a multiple of
+ * 32, of 128 for 4-bit weights; fp32 weights with more than 32 rows). */
+int hipdec_debug_gemm_plan(uint32_t weight_dtype, int rows, int n, int k, int num_cu, uint64_t out[8]);
+
 /* Test hook for the bounded waits of the persistent kernels (every wait on another workgroup gives up
  * after a number of polls, raises the model's abort flag and every workgroup leaves; the host call then
  * returns HIPDEC_ERR_HIP and later steps take the one-kernel-per-product path).  check_mask: a waiting

@@ -643,7 +643,7 @@ bool pf_use_dl(int wt, int T, int K, int act) {
     static const bool off = getenv("HIPDEC_NO_DL_GEMM") != nullptr;
     return !off && wt == WT_BF16 && T >= kDlMinRows && K % PF_BKL == 0 && act != PF_ACT_F16;
 }
-PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K, bool dl = false) {
+PfSplit pf_split_k(int num_cu, int wt, int T, int N, int K, bool dl = false) {
     if (dl) {
         // One workgroup per CU, so the grid runs in rounds of num_cu workgroups and a partly filled last
         // round costs a whole one.  K splits change the round count: with s splits the work takes
@@ -656,7 +656,7 @@ PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K, bool dl =
         double best_cost = 1e30;
         for (int s = 1; s <= 8 && lsteps / s >= 4; ++s) {
             const int sps = (lsteps + s - 1) / s, ns = (lsteps + sps - 1) / sps;
-            const double rounds = (double)(((size_t)tiles * ns + m->num_cu - 1) / m->num_cu);
+            const double rounds = (double)(((size_t)tiles * ns + num_cu - 1) / num_cu);
             const double cost = rounds * t_full * sps / lsteps + (ns - 1) * t_plane;
             if (cost < best_cost * 0.97) { best_cost = cost; best = ns; }
         }
@@ -670,7 +670,7 @@ PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K, bool dl =
         // of them where the staged activation slice (hi + lo) fits the LDS budget with that (the kernel then
         // reads a round's four scales of a row as one aligned load).  Aim at a few workgroups per CU.
         const int tiles = (N + kSkinnyI4Bn - 1) / kSkinnyI4Bn, groups = K / 128;
-        int s = std::max(1, (kSkinnyI4WgsPerCu * m->num_cu + tiles - 1) / tiles);
+        int s = std::max(1, (kSkinnyI4WgsPerCu * num_cu + tiles - 1) / tiles);
         const int max_groups = std::min(PF_SQ_GU, std::max(1, ((kSkinnyLdsBytes / (4 * T)) - PF_SK_PAD) / 128));
         int gps = std::min(max_groups, std::max(1, (groups + s - 1) / s));
         if (gps >= 4) gps &= ~3;
@@ -681,7 +681,7 @@ PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K, bool dl =
         // e4m3 weights: 64 weight rows per workgroup, every wave walks the whole K range of its split, a split is a
         // whole number of 64-element blocks, a multiple of eight of them (one round of loads) where that fits
         const int tiles = (N + 63) / 64, blocks = K / 64;
-        const int s = std::max(1, (kSkinnyI4WgsPerCu * m->num_cu + tiles - 1) / tiles);
+        const int s = std::max(1, (kSkinnyI4WgsPerCu * num_cu + tiles - 1) / tiles);
         const int max_blocks = std::max(1, ((kSkinnyLdsBytes / (4 * T)) - PF_SK_PAD) / 64);
         int bps = std::min(max_blocks, std::max(1, (blocks + s - 1) / s));
         if (bps >= 8) bps &= ~7;
@@ -691,7 +691,7 @@ PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K, bool dl =
     if (T <= kSkinnyRows) {
         // 4 waves per workgroup share a K range; aim at ~8 waves per CU over the whole grid
         const int tiles = (N + 31) / 32;
-        int s = std::max(1, (2 * m->num_cu) / tiles);
+        int s = std::max(1, (2 * num_cu) / tiles);
         s = std::min(s, std::max(1, nsteps / 8));
         // the workgroup's slice of the activation rows (hi + lo) has to fit its LDS budget
         int max_steps = std::max(1, ((kSkinnyLdsBytes / (4 * T)) - PF_SK_PAD) / PF_BK);
@@ -704,13 +704,40 @@ PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K, bool dl =
     const int bn = PF_BN_OF(wt);
     const int tiles = ((N + bn - 1) / bn) * ((T + PF_BM - 1) / PF_BM);
     const int lsteps = (K + PF_BKL - 1) / PF_BKL;
-    int s = (2 * m->num_cu + tiles - 1) / tiles;
+    int s = (2 * num_cu + tiles - 1) / tiles;
     s = std::min(s, 8);
     s = std::min(s, std::max(1, lsteps / 4));
     s = std::max(s, 1);
     int sps = (lsteps + s - 1) / s;
     if (wt == WT_INT4) sps = (sps + 1) & ~1;       // a split covers whole scale groups (two steps each)
     return PfSplit{(lsteps + sps - 1) / sps, sps};
+}
+PfSplit pf_split_k(const hipdec_model *m, int wt, int T, int N, int K, bool dl = false) { return pf_split_k(m->num_cu, wt, T, N, K, dl); }
+
+// What one product launches: which kernel, its grid, workgroup size and dynamic LDS, and the K splits (= planes
+// written).  pf_gemm launches exactly this; hipdec_debug_gemm_plan hands it to tests, which check it against
+// what the kernels assume without a GPU.
+enum { PF_K_TILED = 0, PF_K_DL = 1, PF_K_FEW = 2, PF_K_FEW_I4 = 3, PF_K_FEW_F8 = 4 };
+struct PfPlan { int kernel, splits, steps_per_split; unsigned gx, gy, gz, threads; size_t lds; };
+PfPlan pf_plan(int num_cu, int wt, int T, int N, int K, int act) {
+    if (pf_use_dl(wt, T, K, act)) {
+        const PfSplit sp = pf_split_k(num_cu, wt, T, N, K, true);
+        return PfPlan{PF_K_DL, sp.splits, sp.steps_per_split, (unsigned)((N + PF_DL_BN - 1) / PF_DL_BN),
+                      (unsigned)((T + PF_DL_BM - 1) / PF_DL_BM), (unsigned)sp.splits, 64 * PF_DL_WAVES, 0};
+    }
+    const PfSplit sp = pf_split_k(num_cu, wt, T, N, K);
+    // the few-row kernels stage [hi | lo][T][steps_per_split * PF_BK + PF_SK_PAD] bf16 values
+    const size_t staged = (size_t)2 * T * (sp.steps_per_split * PF_BK + PF_SK_PAD) * 2;
+    if (T <= kSkinnyRows && wt == WT_INT4 && pf_use_skinny_i4())
+        return PfPlan{PF_K_FEW_I4, sp.splits, sp.steps_per_split, (unsigned)((N + kSkinnyI4Bn - 1) / kSkinnyI4Bn),
+                      (unsigned)sp.splits, 1, 64 * kSkinnyI4Waves, staged};
+    if (T <= kSkinnyRows && wt == WT_FP8 && pf_use_skinny_f8(K))
+        return PfPlan{PF_K_FEW_F8, sp.splits, sp.steps_per_split, (unsigned)((N + 63) / 64), (unsigned)sp.splits, 1, 256, staged};
+    if (T <= kSkinnyRows)
+        return PfPlan{PF_K_FEW, sp.splits, sp.steps_per_split, (unsigned)((N + 31) / 32), (unsigned)sp.splits, 1, 256, staged};
+    const int bn = PF_BN_OF(wt);
+    return PfPlan{PF_K_TILED, sp.splits, sp.steps_per_split, (unsigned)((N + bn - 1) / bn), (unsigned)((T + PF_BM - 1) / PF_BM),
+                  (unsigned)sp.splits, 256, 0};
 }
 
 int pf_ensure(hipdec_model *m, int T, bool with_head = false) {
@@ -753,52 +780,42 @@ int pf_ensure(hipdec_model *m, int T, bool with_head = false) {
 // act: PF_ACT_* of the activation arrays (the few-row kernel only takes pairs)
 int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, const void *W, const void *scales,
             int T, int N, int K, int act = PF_ACT_PAIR) {
-    if (pf_use_dl(wt, T, K, act)) {
-        const PfSplit sp = pf_split_k(m, wt, T, N, K, true);
-        PfGemm g{Ahi, Alo, W, nullptr, m->pf.P, T, N, K, sp.steps_per_split};
-        dim3 grid((N + PF_DL_BN - 1) / PF_DL_BN, (T + PF_DL_BM - 1) / PF_DL_BM, sp.splits), block(64 * PF_DL_WAVES);
+    const PfPlan p = pf_plan(m->num_cu, wt, T, N, K, act);
+    const dim3 grid(p.gx, p.gy, p.gz), block(p.threads);
+    const size_t lds = p.lds;
+    PfGemm g{Ahi, Alo, W, wt == WT_INT4 && p.kernel != PF_K_DL ? (const uint16_t *)scales : nullptr, m->pf.P, T, N, K, p.steps_per_split};
+    switch (p.kernel) {
+    case PF_K_DL:
         if (act == PF_ACT_PAIR) hipLaunchKernelGGL((k_pf_gemm_dl<true, PF_BKL, 2, PF_DL_WAVES, 1>), grid, block, 0, m->stream, g);
         else hipLaunchKernelGGL((k_pf_gemm_dl<false, PF_BKL, 3, PF_DL_WAVES, 1>), grid, block, 0, m->stream, g);
-        return sp.splits;
-    }
-    const PfSplit sp = pf_split_k(m, wt, T, N, K);
-    PfGemm g{Ahi, Alo, W, wt == WT_INT4 ? (const uint16_t *)scales : nullptr, m->pf.P, T, N, K, sp.steps_per_split};
-    if (T <= kSkinnyRows && wt == WT_INT4 && pf_use_skinny_i4()) {
-        const int rt = T <= 16 ? 1 : 2;
-        dim3 grid((N + kSkinnyI4Bn - 1) / kSkinnyI4Bn, sp.splits), block(64 * kSkinnyI4Waves);
-        const size_t lds = (size_t)2 * T * (sp.steps_per_split * PF_BK + PF_SK_PAD) * 2;
+        break;
+    case PF_K_FEW_I4:
         if (T <= 8) hipLaunchKernelGGL((k_pf_gemm_skinny_i4<1, true, kSkinnyI4Nt, kSkinnyI4Waves>), grid, block, lds, m->stream, g);
-        else if (rt == 1) hipLaunchKernelGGL((k_pf_gemm_skinny_i4<1, false, kSkinnyI4Nt, kSkinnyI4Waves>), grid, block, lds, m->stream, g);
+        else if (T <= 16) hipLaunchKernelGGL((k_pf_gemm_skinny_i4<1, false, kSkinnyI4Nt, kSkinnyI4Waves>), grid, block, lds, m->stream, g);
         else hipLaunchKernelGGL((k_pf_gemm_skinny_i4<2, false, kSkinnyI4Nt, kSkinnyI4Waves>), grid, block, lds, m->stream, g);
-        return sp.splits;
-    }
-    if (T <= kSkinnyRows && wt == WT_FP8 && pf_use_skinny_f8(K)) {
-        dim3 grid((N + 63) / 64, sp.splits), block(256);
-        const size_t lds = (size_t)2 * T * (sp.steps_per_split * PF_BK + PF_SK_PAD) * 2;
+        break;
+    case PF_K_FEW_F8:
         if (T <= 8) hipLaunchKernelGGL((k_pf_gemm_skinny_f8<1, true>), grid, block, lds, m->stream, g);
         else if (T <= 16) hipLaunchKernelGGL((k_pf_gemm_skinny_f8<1, false>), grid, block, lds, m->stream, g);
         else hipLaunchKernelGGL((k_pf_gemm_skinny_f8<2, false>), grid, block, lds, m->stream, g);
-        return sp.splits;
-    }
-    if (T <= kSkinnyRows) {
-        dim3 grid((N + 31) / 32, sp.splits), block(256);
-        const size_t lds = (size_t)2 * T * (sp.steps_per_split * PF_BK + PF_SK_PAD) * 2;
+        break;
+    case PF_K_FEW:
         if (wt == WT_F32) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_F32>, grid, block, lds, m->stream, g);
         else if (wt == WT_BF16) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_BF16>, grid, block, lds, m->stream, g);
         else if (wt == WT_FP8) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_FP8>, grid, block, lds, m->stream, g);
         else hipLaunchKernelGGL(k_pf_gemm_skinny<WT_INT4>, grid, block, lds, m->stream, g);
-        return sp.splits;
-    }
-    const int bn = PF_BN_OF(wt);
-    dim3 grid((N + bn - 1) / bn, (T + PF_BM - 1) / PF_BM, sp.splits), block(256);
+        break;
+    default:
 #define PFG(WTX) do { if (act == PF_ACT_F16) hipLaunchKernelGGL((k_pf_gemm<WTX, PF_ACT_F16>), grid, block, 0, m->stream, g); \
                       else if (act == PF_ACT_BF16) hipLaunchKernelGGL((k_pf_gemm<WTX, PF_ACT_BF16>), grid, block, 0, m->stream, g); \
                       else hipLaunchKernelGGL((k_pf_gemm<WTX, PF_ACT_PAIR>), grid, block, 0, m->stream, g); } while (0)
-    if (wt == WT_BF16) PFG(WT_BF16);
-    else if (wt == WT_FP8) PFG(WT_FP8);
-    else PFG(WT_INT4);
+        if (wt == WT_BF16) PFG(WT_BF16);
+        else if (wt == WT_FP8) PFG(WT_FP8);
+        else PFG(WT_INT4);
 #undef PFG
-    return sp.splits;
+        break;
+    }
+    return p.splits;
 }
 
 // launches shared by the prompt prefill and the multi-sample step
@@ -2214,6 +2231,16 @@ int hipdec_decode_fullvocab_sampled_run_batch(hipdec_model *m, const uint32_t *t
 int hipdec_debug_step_kernel(const hipdec_model *m, int *out) {
     if (!m || !out) return HIPDEC_ERR_ARG;
     *out = !m->mega_ok ? 0 : m->lean_ce ? 2 : 1;
+    return HIPDEC_OK;
+}
+
+int hipdec_debug_gemm_plan(uint32_t weight_dtype, int rows, int n, int k, int num_cu, uint64_t out[8]) {
+    if (!out || weight_dtype > HIPDEC_W_INT4_G128 || rows < 1 || n < 1 || k < PF_BK || k % PF_BK || num_cu < 1) return HIPDEC_ERR_ARG;
+    if (weight_dtype == HIPDEC_W_INT4_G128 && k % 128) return HIPDEC_ERR_ARG;
+    if (weight_dtype == HIPDEC_W_F32 && rows > kSkinnyRows) return HIPDEC_ERR_ARG;     // fp32 weights go 32 rows at a time
+    const PfPlan p = pf_plan(num_cu, (int)weight_dtype, rows, n, k, PF_ACT_PAIR);
+    out[0] = (uint64_t)p.kernel; out[1] = (uint64_t)p.splits; out[2] = (uint64_t)p.steps_per_split;
+    out[3] = p.gx; out[4] = p.gy; out[5] = p.gz; out[6] = p.threads; out[7] = p.lds;
     return HIPDEC_OK;
 }
 

@@ -34,6 +34,7 @@ EXPORTS = [
     "hipdec_decode_fullvocab_sampled_run_batch", "hipdec_debug_hostmath_eval", "hipdec_debug_hostmath_checksum",
     "hipdec_debug_hostmath_count_mismatch", "hipdec_debug_hostmath_probe", "hipdec_debug_sample_topk",
     "hipdec_debug_sample_fullvocab", "hipdec_sample_fullvocab_noalloc", "hipdec_debug_set_spin_limit", "hipdec_debug_step_kernel",
+    "hipdec_debug_gemm_plan",
 ]
 
 
@@ -238,6 +239,22 @@ def set_spin_limit(check_mask=127, limit=1 << 22):
     rc = lib.hipdec_debug_set_spin_limit(check_mask, limit)
     if rc != OK:
         raise HipDecodeError(rc, (lib.hipdec_last_error(None) or b"").decode())
+
+
+GEMM_KERNELS = ("tiled", "tiled_direct_lds", "few_row", "few_row_int4", "few_row_e4m3")
+
+
+def gemm_plan(weight_dtype, rows, n, k, num_cu=256):
+    """The launch the library uses for the product of `rows` activation rows with an [n][k] weight matrix
+    (hipdec_debug_gemm_plan; host arithmetic only, no GPU needed)."""
+    lib = load_library()
+    out = (C.c_uint64 * 8)()
+    lib.hipdec_debug_gemm_plan.argtypes = [C.c_uint32, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_uint64)]
+    rc = lib.hipdec_debug_gemm_plan(int(weight_dtype), rows, n, k, num_cu, out)
+    if rc != OK:
+        raise HipDecodeError(rc, "the library launches no such product")
+    return {"kernel": GEMM_KERNELS[out[0]], "splits": out[1], "steps_per_split": out[2], "grid": (out[3], out[4], out[5]),
+            "threads": out[6], "lds_bytes": out[7]}
 
 
 def _fptr(a):
