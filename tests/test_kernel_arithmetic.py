@@ -81,10 +81,10 @@ def test_hi_lo_pair_keeps_sixteen_bits():
 
 
 def test_row_of_a_staged_chunk_without_a_division():
-    # t = int((cc + 0.5) * (1 / cpr)) in fp32 equals cc // cpr for every chunk count per row (a multiple of 16)
-    # and every chunk index a workgroup stages (at most 1280 + a round of 512 threads), also with the
-    # reciprocal one unit in the last place off either way
-    for cpr in range(16, 1281, 16):
+    # t = int((cc + 0.5) * (1 / cpr)) in fp32 equals cc // cpr for every chunk count per row (a multiple of 16
+    # with 4-bit weights; any count up to 1280 is covered here) and every chunk index a workgroup stages (at
+    # most 1280 + a round of 512 threads), also with the reciprocal one unit in the last place off either way
+    for cpr in range(1, 1281):
         cc = np.arange(0, 1280 + 512, dtype=np.int64)
         rcp = np.float32(1.0) / np.float32(cpr)
         for r in (rcp, np.nextafter(rcp, np.float32(0)), np.nextafter(rcp, np.float32(1))):
