@@ -906,6 +906,11 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny(PfGemm g) {
 //    sums and no cross-lane traffic, and the weights of the split's whole K range are requested before it (the
 //    host keeps a split within PF_SQ_GU groups).
 #define PF_SQ_GU 8                       // scale groups of a split: what a wave requests per tile, all at once
+// a constant the compiler has to treat as a register's value (S: scalar register, V: vector register)
+#ifndef PF_REG_CONST_S
+#define PF_REG_CONST_S(var, lit) asm volatile("s_mov_b32 %0, " #lit : "=s"(var))
+#define PF_REG_CONST_V(var, lit) asm volatile("v_mov_b32 %0, " #lit : "=v"(var))
+#endif
 typedef float pf_f32x4 __attribute__((ext_vector_type(4)));
 template <int RT, bool PACK, int NT, int WAVES>   // RT tiles of 16 activation rows (T <= 16 RT; PACK: T <= 8, RT = 1); NT weight tiles per wave
 __global__ __launch_bounds__(64 * WAVES) void k_pf_gemm_skinny_i4(PfGemm g) {
@@ -1010,9 +1015,9 @@ __global__ __launch_bounds__(64 * WAVES) void k_pf_gemm_skinny_i4(PfGemm g) {
     }
     // the unpacking constants live in registers: as literals each pair would cost an "and" and an "or"
     uint32_t nib_mask, nib_bias, m24;
-    asm volatile("s_mov_b32 %0, 0x00780078" : "=s"(nib_mask));
-    asm volatile("v_mov_b32 %0, 0x41804180" : "=v"(nib_bias));
-    asm volatile("v_mov_b32 %0, 0xc1c0c1c0" : "=v"(m24));              // two bf16 numbers -24
+    PF_REG_CONST_S(nib_mask, 0x00780078);
+    PF_REG_CONST_V(nib_bias, 0x41804180);
+    PF_REG_CONST_V(m24, 0xc1c0c1c0);                                   // two bf16 numbers -24
     const pf_bf16x8 BC = __builtin_bit_cast(pf_bf16x8, make_uint4(m24, m24, m24, m24));
     pf_f32x4 acc[RT][NT];
 #pragma unroll

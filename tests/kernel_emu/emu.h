@@ -1,0 +1,134 @@
+// A small host-side stand-in for the parts of the GPU programming model the few-row GEMM kernels use, so that
+// the kernels' own source text runs on the CPU (test infrastructure: one OS thread per GPU thread, a workgroup
+// at a time).  Cross-lane operations (wave shuffles, matrix instructions) meet at a per-wave barrier, which is
+// sound where the kernel calls them under wave-uniform control flow, as these kernels do.
+#pragma once
+#include <cmath>
+#include <condition_variable>
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <thread>
+#include <vector>
+
+struct uint4 { uint32_t x, y, z, w; };
+struct uint2 { uint32_t x, y; };
+struct dim3 { unsigned x, y, z; };
+static inline uint4 make_uint4(uint32_t x, uint32_t y, uint32_t z, uint32_t w) { return uint4{x, y, z, w}; }
+static inline uint2 make_uint2(uint32_t x, uint32_t y) { return uint2{x, y}; }
+struct pf_bf16x8 { uint16_t v[8]; };
+template <class T> static inline T min(T a, T b) { return b < a ? b : a; }
+template <class T> static inline T max(T a, T b) { return a < b ? b : a; }
+
+namespace emu {
+class Barrier {
+public:
+    explicit Barrier(int n) : n_(n) {}
+    void wait() {
+        std::unique_lock<std::mutex> lk(m_);
+        const unsigned gen = gen_;
+        if (++count_ == n_) { count_ = 0; ++gen_; cv_.notify_all(); }
+        else cv_.wait(lk, [&] { return gen_ != gen; });
+    }
+private:
+    std::mutex m_;
+    std::condition_variable cv_;
+    int n_, count_ = 0;
+    unsigned gen_ = 0;
+};
+struct Wave {
+    Barrier bar{64};
+    uint32_t a[64][4], b[64][4];
+    float f[64];
+};
+struct Block {
+    // the dynamic LDS is a heap block of exactly the size the launch asked for: under AddressSanitizer an access past
+    // it is reported like one past any other buffer
+    explicit Block(int threads, size_t lds_bytes) : bar(threads), waves((threads + 63) / 64), lds((unsigned char *)std::malloc(lds_bytes ? lds_bytes : 1)) {}
+    ~Block() { std::free(lds); }
+    Barrier bar;
+    std::vector<Wave> waves;
+    unsigned char *lds;
+};
+inline thread_local dim3 tl_thread, tl_block, tl_grid;
+inline thread_local Block *tl_blk = nullptr;
+inline Wave &wave() { return tl_blk->waves[tl_thread.x >> 6]; }
+inline int lane() { return (int)(tl_thread.x & 63); }
+inline uint16_t *lds() { return (uint16_t *)tl_blk->lds; }
+inline void sync_block() { tl_blk->bar.wait(); }
+inline float bf16_to_float(uint16_t h) { const uint32_t u = (uint32_t)h << 16; float f; std::memcpy(&f, &u, 4); return f; }
+inline float uint_as_float(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
+inline float shfl_xor(float v, int mask, int) {
+    Wave &w = wave();
+    w.f[lane()] = v;
+    w.bar.wait();
+    const float r = w.f[lane() ^ mask];
+    w.bar.wait();
+    return r;
+}
+// v_perm_b32: result byte i is byte sel[i] of the eight bytes {s0 (4..7), s1 (0..3)}
+inline uint32_t perm(uint32_t s0, uint32_t s1, uint32_t sel) {
+    const uint64_t both = ((uint64_t)s0 << 32) | s1;
+    uint32_t r = 0;
+    for (int i = 0; i < 4; ++i) {
+        const unsigned pick = (sel >> (8 * i)) & 0xff;
+        r |= (uint32_t)((both >> (8 * (pick & 7))) & 0xff) << (8 * i);     // (selectors above 7 are not used by these kernels)
+    }
+    return r;
+}
+// v_mfma_f32_16x16x32_bf16: D = A (16 x 32) . B (32 x 16) + C.  Lane l supplies row l % 16 of A and column
+// l % 16 of B, reduction elements 8 * (l / 16) .. + 7 of each; register r of lane l holds D[4 * (l / 16) + r][l % 16].
+template <class V4>
+inline V4 mfma_16x16x32_bf16(pf_bf16x8 a, pf_bf16x8 b, V4 c, int, int, int) {
+    Wave &w = wave();
+    const int l = lane();
+    std::memcpy(w.a[l], a.v, 16);
+    std::memcpy(w.b[l], b.v, 16);
+    w.bar.wait();
+    V4 d = c;
+    for (int r = 0; r < 4; ++r) {
+        const int i = 4 * (l / 16) + r, j = l % 16;
+        double s = 0.0;
+        for (int k = 0; k < 32; ++k) {
+            const uint16_t *ar = (const uint16_t *)w.a[(k / 8) * 16 + i], *br = (const uint16_t *)w.b[(k / 8) * 16 + j];
+            s += (double)bf16_to_float(ar[k % 8]) * (double)bf16_to_float(br[k % 8]);
+        }
+        d[r] = (float)((double)c[r] + s);
+    }
+    w.bar.wait();
+    return d;
+}
+// runs kernel(args) over the grid, one workgroup after the other
+template <class K, class A>
+inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, const A &args) {
+    for (unsigned bz = 0; bz < grid.z; ++bz)
+        for (unsigned by = 0; by < grid.y; ++by)
+            for (unsigned bx = 0; bx < grid.x; ++bx) {
+                Block blk((int)threads, lds_bytes);
+                std::vector<std::thread> ts;
+                ts.reserve(threads);
+                for (unsigned t = 0; t < threads; ++t)
+                    ts.emplace_back([&, t] {
+                        tl_thread = dim3{t, 0, 0}; tl_block = dim3{bx, by, bz}; tl_grid = grid; tl_blk = &blk;
+                        kernel(args);
+                    });
+                for (auto &th : ts) th.join();
+            }
+}
+}  // namespace emu
+
+#define __global__
+#define __device__
+#define __forceinline__ inline
+#define __launch_bounds__(...)
+#define threadIdx emu::tl_thread
+#define blockIdx emu::tl_block
+#define gridDim emu::tl_grid
+#define __syncthreads() emu::sync_block()
+#define __shfl_xor(v, m, w) emu::shfl_xor((v), (m), (w))
+#define __uint_as_float(u) emu::uint_as_float(u)
+#define __builtin_amdgcn_perm(a, b, s) emu::perm((a), (b), (s))
+#define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) emu::mfma_16x16x32_bf16((a), (b), (c), (x), (y), (z))
+#define PF_REG_CONST_S(var, lit) var = lit
+#define PF_REG_CONST_V(var, lit) var = lit

@@ -1,0 +1,78 @@
+"""The 4-bit few-row GEMM kernel's own source text, compiled for the host and run thread for thread on the CPU
+(tests/kernel_emu/emu.h stands in for workgroups, waves, LDS, shuffles and the matrix instruction) under the
+launch plans the library itself works out, with AddressSanitizer and UBSan: results against a plain fp64
+product, every result element written, and no access outside the operands, the planes or the LDS.  What this
+cannot show is the compiler's and the hardware's side (covered by the GPU tests); what it does show is the
+kernel's indexing, its arithmetic identities and the host/kernel contract for shapes and row counts at will."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+from rustane_amd import hipdec
+from rustane_amd.hipdec import WeightDtype
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EMU = os.path.join(ROOT, "tests", "kernel_emu")
+
+
+def host_clang():
+    for c in ("/opt/rocm/lib/llvm/bin/clang++", shutil.which("amdclang++"), shutil.which("clang++")):
+        if c and os.path.exists(c):
+            return c
+    return None
+
+
+@pytest.fixture(scope="module")
+def emulator(tmp_path_factory):
+    cxx = host_clang()
+    if cxx is None:
+        pytest.skip("no clang++ for the host (the kernel text uses clang's vector types)")
+    build = tmp_path_factory.mktemp("kernel_emu")
+    text = open(os.path.join(ROOT, "rustane_amd", "csrc", "hipdec_prefill.h")).read()
+    start, end = text.index("#define PF_SQ_GU"), text.index("// The same few-row GEMM for e4m3 weights.")
+    kernel = text[start:end]
+    assert "void k_pf_gemm_skinny_i4(PfGemm g)" in kernel
+    lds_decl = "extern __shared__ __align__(16) uint16_t s_act[];"
+    assert kernel.count(lds_decl) == 1
+    (build / "kernel_i4.inc").write_text(kernel.replace(lds_decl, "uint16_t *s_act = emu::lds();"))
+    (build / "pfgemm_struct.inc").write_text(re.search(r"struct PfGemm \{.*?\n\};\n", text, flags=re.S).group(0))
+    exe = build / "few_row_i4"
+    cmd = [cxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
+           "-pthread", "-I", str(build), "-I", EMU, os.path.join(EMU, "few_row_i4.cpp"), "-o", str(exe)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-4000:]
+    return str(exe)
+
+
+def run_case(exe, rows, n, k, num_cu, seed, lds_delta=0):
+    p = hipdec.gemm_plan(WeightDtype.INT4_G128, rows, n, k, num_cu)
+    assert p["kernel"] == "few_row_int4"
+    args = [rows, n, k, p["steps_per_split"], *p["grid"], p["threads"], p["lds_bytes"] + lds_delta, seed]
+    r = subprocess.run([exe] + [str(a) for a in args], capture_output=True, text=True, timeout=600)
+    return p, r
+
+
+# (rows, n, k, compute units the plan is made for): packed hi/lo tile up to 8 rows, one and two row tiles above;
+# reductions of 1, 3, 5, 9 and 16 scale groups; ragged n; splits of 1, 2, 3, 4 and 8 groups (the last through plans
+# for a small device, which keep the grid small enough to emulate)
+CASES = [
+    (8, 300, 384, 256), (5, 130, 1152, 256), (1, 16, 128, 256), (3, 257, 640, 256), (8, 128, 2048, 256),
+    (8, 512, 2048, 2), (7, 384, 1024, 1), (16, 200, 640, 256), (9, 129, 384, 256), (13, 256, 2048, 2),
+    (27, 70, 384, 256), (17, 130, 1152, 256), (32, 144, 640, 256), (32, 256, 1024, 1),
+]
+
+
+@pytest.mark.parametrize("rows,n,k,num_cu", CASES)
+def test_four_bit_few_row_kernel_source_on_the_cpu(emulator, rows, n, k, num_cu):
+    p, r = run_case(emulator, rows, n, k, num_cu, seed=rows * 1000 + n)
+    assert r.returncode == 0, (p, r.stdout, r.stderr[-3000:])
+    assert "not written 0" in r.stdout
+
+
+def test_the_sanitizer_sees_an_access_past_the_lds(emulator):
+    # the control for the test above: with less LDS than the staged rows take, the same launch is reported
+    p, r = run_case(emulator, 8, 300, 384, 256, 1, lds_delta=-640)
+    assert r.returncode != 0 and "heap-buffer-overflow" in r.stderr, (p, r.stdout, r.stderr[-2000:])
