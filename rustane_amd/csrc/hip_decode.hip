@@ -634,6 +634,8 @@ bool pf_use_skinny_i4() {
     return !off;
 }
 constexpr int kSkinnyI4WgsPerCu = 3;              // workgroups per CU its K splits aim at
+constexpr int kSkinnyF8Waves = 8;                 // waves per workgroup of k_pf_gemm_skinny_f8, 16 weight rows each
+constexpr int kSkinnyF8Bn = 16 * kSkinnyF8Waves;
 // the few-row GEMM of e4m3 models likewise (HIPDEC_NO_SKINNY_F8=1: the general few-row kernel)
 bool pf_use_skinny_f8(int K) {
     static const bool off = [] { const char *v = getenv("HIPDEC_NO_SKINNY_F8"); return v && v[0] == '1'; }();
@@ -678,14 +680,14 @@ PfSplit pf_split_k(int num_cu, int wt, int T, int N, int K, bool dl = false) {
         return PfSplit{(groups + gps - 1) / gps, 4 * gps};
     }
     if (T <= kSkinnyRows && wt == WT_FP8 && pf_use_skinny_f8(K)) {
-        // e4m3 weights: 64 weight rows per workgroup, every wave walks the whole K range of its split, a split is a
-        // whole number of 64-element blocks, a multiple of eight of them (one round of loads) where that fits
-        const int tiles = (N + 63) / 64, blocks = K / 64;
+        // e4m3 weights: kSkinnyF8Bn weight rows per workgroup, every wave walks the whole K range of its split, a
+        // split is a whole number of 64-element blocks, at most PF_S8_GU of them (what the kernel requests at once)
+        // and that many where the staged activation slice fits the LDS budget
+        const int tiles = (N + kSkinnyF8Bn - 1) / kSkinnyF8Bn, blocks = K / 64;
         const int s = std::max(1, (kSkinnyI4WgsPerCu * num_cu + tiles - 1) / tiles);
-        const int max_blocks = std::max(1, ((kSkinnyLdsBytes / (4 * T)) - PF_SK_PAD) / 64);
+        const int max_blocks = std::min(PF_S8_GU, std::max(1, ((kSkinnyLdsBytes / (4 * T)) - PF_SK_PAD) / 64));
         int bps = std::min(max_blocks, std::max(1, (blocks + s - 1) / s));
-        if (bps >= 8) bps &= ~7;
-        else if (max_blocks >= 8) bps = 8;
+        if (max_blocks >= PF_S8_GU) bps = PF_S8_GU;
         return PfSplit{(blocks + bps - 1) / bps, 2 * bps};
     }
     if (T <= kSkinnyRows) {
@@ -732,7 +734,8 @@ PfPlan pf_plan(int num_cu, int wt, int T, int N, int K, int act) {
         return PfPlan{PF_K_FEW_I4, sp.splits, sp.steps_per_split, (unsigned)((N + kSkinnyI4Bn - 1) / kSkinnyI4Bn),
                       (unsigned)sp.splits, 1, 64 * kSkinnyI4Waves, staged};
     if (T <= kSkinnyRows && wt == WT_FP8 && pf_use_skinny_f8(K))
-        return PfPlan{PF_K_FEW_F8, sp.splits, sp.steps_per_split, (unsigned)((N + 63) / 64), (unsigned)sp.splits, 1, 256, staged};
+        return PfPlan{PF_K_FEW_F8, sp.splits, sp.steps_per_split, (unsigned)((N + kSkinnyF8Bn - 1) / kSkinnyF8Bn), (unsigned)sp.splits, 1,
+                      64 * kSkinnyF8Waves, staged};
     if (T <= kSkinnyRows)
         return PfPlan{PF_K_FEW, sp.splits, sp.steps_per_split, (unsigned)((N + 31) / 32), (unsigned)sp.splits, 1, 256, staged};
     const int bn = PF_BN_OF(wt);
@@ -795,9 +798,9 @@ int pf_gemm(hipdec_model *m, int wt, const uint16_t *Ahi, const uint16_t *Alo, c
         else hipLaunchKernelGGL((k_pf_gemm_skinny_i4<2, false, kSkinnyI4Nt, kSkinnyI4Waves>), grid, block, lds, m->stream, g);
         break;
     case PF_K_FEW_F8:
-        if (T <= 8) hipLaunchKernelGGL((k_pf_gemm_skinny_f8<1, true>), grid, block, lds, m->stream, g);
-        else if (T <= 16) hipLaunchKernelGGL((k_pf_gemm_skinny_f8<1, false>), grid, block, lds, m->stream, g);
-        else hipLaunchKernelGGL((k_pf_gemm_skinny_f8<2, false>), grid, block, lds, m->stream, g);
+        if (T <= 8) hipLaunchKernelGGL((k_pf_gemm_skinny_f8<1, true, kSkinnyF8Waves>), grid, block, lds, m->stream, g);
+        else if (T <= 16) hipLaunchKernelGGL((k_pf_gemm_skinny_f8<1, false, kSkinnyF8Waves>), grid, block, lds, m->stream, g);
+        else hipLaunchKernelGGL((k_pf_gemm_skinny_f8<2, false, kSkinnyF8Waves>), grid, block, lds, m->stream, g);
         break;
     case PF_K_FEW:
         if (wt == WT_F32) hipLaunchKernelGGL(k_pf_gemm_skinny<WT_F32>, grid, block, lds, m->stream, g);

@@ -1094,46 +1094,52 @@ __global__ __launch_bounds__(64 * WAVES) void k_pf_gemm_skinny_i4(PfGemm g) {
 // elements 16 kg .. + 16 of a 64-element block, the four lanes of a row read 64 contiguous bytes, and dwords 2 j,
 // 2 j + 1 are the lane's 8 elements of matrix instruction j (j = 0, 1) of the block, widened to bf16 two at a time
 // by v_cvt_scalef32_pk_bf16_fp8 (exact).  The activations are staged as they are; the per-row scale is applied by
-// the kernel that sums the planes, as for k_pf_gemm_skinny.  A K split is a whole number of blocks.
-#define PF_S8_GU 8                       // 64-element blocks per wave whose loads are issued together
+// the kernel that sums the planes, as for k_pf_gemm_skinny.  A K split is a whole number of blocks, at most
+// PF_S8_GU of them, all requested before the rows are staged; the staging loop has no integer division.
+#define PF_S8_GU 8                       // 64-element blocks of a split: what a wave requests, all at once
 typedef __bf16 pf_bf16x2v __attribute__((ext_vector_type(2)));
-template <int RT, bool PACK>
-__global__ __launch_bounds__(256) void k_pf_gemm_skinny_f8(PfGemm g) {
+template <int RT, bool PACK, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void k_pf_gemm_skinny_f8(PfGemm g) {
+    constexpr int NTHR = 64 * WAVES;
     static_assert(!PACK || RT == 1, "packed planes are one row tile");
     extern __shared__ __align__(16) uint16_t s_act[];      // [2][T][astride] bf16
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kg = lane >> 4;
-    const int n0 = blockIdx.x * 64 + wave * 16, z = blockIdx.y;
+    const int n0 = blockIdx.x * (16 * WAVES) + wave * 16, z = blockIdx.y;
     const int nsteps = g.K / PF_BK;
     const int zb = z * g.steps_per_split, ze = min(nsteps, zb + g.steps_per_split);
     const int b_begin = zb / 2, b_end = ze / 2;            // 64-element blocks (the host makes every split a whole number of them)
     const int krange = (ze - zb) * PF_BK, astride = g.steps_per_split * PF_BK + PF_SK_PAD;
     const char *wrow = (const char *)g.W + (size_t)min(n0 + n, g.N - 1) * (size_t)g.K + 16 * kg;
+    // slot u holds the split's block u (the host keeps a split within PF_S8_GU blocks)
     uint4 w0[PF_S8_GU];
-    auto wload = [&](int bi) {
-#pragma unroll
-        for (int u = 0; u < PF_S8_GU; ++u) w0[u] = *(const uint4 *)(wrow + (size_t)min(bi + u, b_end - 1) * 64);
-    };
-    // the activation rows are requested first and the first round of weights behind them (staging waits for its own loads only)
+    // the activation rows are requested first and the weights behind them (staging waits for its own loads only)
     {
-        constexpr int MAXIT = 5;                               // 40 KB of staged rows: at most 1280 chunks of hi and lo
-        const int cpr = krange / 8, items = g.T * cpr;
+        constexpr int MAXIT = (1280 + NTHR - 1) / NTHR;        // 40 KB of staged rows: at most 1280 chunks of hi and lo
+        const int cpr = krange / 8, items = g.T * cpr;         // (cpr is a multiple of 8, items at most 1280)
+        const float rcp = 1.0f / (float)cpr;
         uint4 hh[MAXIT], ll[MAXIT];
+        int dst[MAXIT];
 #pragma unroll
         for (int it = 0; it < MAXIT; ++it) {
-            const int cc = min(it * 256 + tid, items - 1);
-            const int t = cc / cpr, kc = cc - t * cpr;
-            const size_t src = (size_t)t * g.K + (size_t)zb * PF_BK + kc * 8;
-            hh[it] = *(const uint4 *)(g.Ahi + src); ll[it] = *(const uint4 *)(g.Alo + src);
+            if (it * NTHR < items) {
+                const int cc = min(it * NTHR + tid, items - 1);
+                // cc / cpr without the division: the quotient's fraction is a multiple of 1 / cpr >= 1 / 1280, the
+                // half chunk added keeps it that far from the next integer, the rounding errors are below 1e-5
+                const int t = (int)(((float)cc + 0.5f) * rcp), kc = cc - t * cpr;
+                const size_t src = (size_t)t * g.K + (size_t)zb * PF_BK + kc * 8;
+                hh[it] = *(const uint4 *)(g.Ahi + src); ll[it] = *(const uint4 *)(g.Alo + src);
+                dst[it] = t * astride + kc * 8;
+            }
         }
-        wload(b_begin);
+#pragma unroll
+        for (int u = 0; u < PF_S8_GU; ++u)
+            if (b_begin + u < b_end) w0[u] = *(const uint4 *)(wrow + (size_t)(b_begin + u) * 64);
 #pragma unroll
         for (int it = 0; it < MAXIT; ++it) {
-            const int c = it * 256 + tid;
-            if (c < items) {
-                const int t = c / cpr, kc = c - t * cpr;
-                *(uint4 *)(s_act + t * astride + kc * 8) = hh[it];
-                *(uint4 *)(s_act + (g.T + t) * astride + kc * 8) = ll[it];
+            if (it * NTHR < items && it * NTHR + tid < items) {
+                *(uint4 *)(s_act + dst[it]) = hh[it];
+                *(uint4 *)(s_act + g.T * astride + dst[it]) = ll[it];
             }
         }
     }
@@ -1153,31 +1159,25 @@ __global__ __launch_bounds__(256) void k_pf_gemm_skinny_f8(PfGemm g) {
     pf_f32x4 acc[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt] = pf_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    for (int bi = b_begin; bi < b_end; bi += PF_S8_GU) {
-        uint4 wc[PF_S8_GU];
 #pragma unroll
-        for (int u = 0; u < PF_S8_GU; ++u) wc[u] = w0[u];
-        if (bi + PF_S8_GU < b_end) wload(bi + PF_S8_GU);      // the next round in flight while this one multiplies
+    for (int u = 0; u < PF_S8_GU; ++u) {
+        if (b_begin + u < b_end) {
+            const int kl = u * 64;
 #pragma unroll
-        for (int u = 0; u < PF_S8_GU; ++u) {
-            if (bi + u < b_end) {
-                const int kl = (bi + u - b_begin) * 64;
+            for (int j = 0; j < 2; ++j) {
+                const uint32_t q0 = j == 0 ? w0[u].x : w0[u].z, q1 = j == 0 ? w0[u].y : w0[u].w;
+                const uint4 b = make_uint4(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(q0, 1.0f, false)),
+                                           __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(q0, 1.0f, true)),
+                                           __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(q1, 1.0f, false)),
+                                           __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(q1, 1.0f, true)));
+                const pf_bf16x8 B = __builtin_bit_cast(pf_bf16x8, b);
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const uint32_t q0 = j == 0 ? wc[u].x : wc[u].z, q1 = j == 0 ? wc[u].y : wc[u].w;
-                    const uint4 b = make_uint4(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(q0, 1.0f, false)),
-                                               __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(q0, 1.0f, true)),
-                                               __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(q1, 1.0f, false)),
-                                               __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(q1, 1.0f, true)));
-                    const pf_bf16x8 B = __builtin_bit_cast(pf_bf16x8, b);
-#pragma unroll
-                    for (int rt = 0; rt < RT; ++rt) {
-                        const uint4 xh = *(const uint4 *)(ah[rt] + kl + 8 * j);
-                        acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, xh), B, acc[rt], 0, 0, 0);
-                        if (!PACK) {
-                            const uint4 xl = *(const uint4 *)(al[rt] + kl + 8 * j);
-                            acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, xl), B, acc[rt], 0, 0, 0);
-                        }
+                for (int rt = 0; rt < RT; ++rt) {
+                    const uint4 xh = *(const uint4 *)(ah[rt] + kl + 8 * j);
+                    acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, xh), B, acc[rt], 0, 0, 0);
+                    if (!PACK) {
+                        const uint4 xl = *(const uint4 *)(al[rt] + kl + 8 * j);
+                        acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, xl), B, acc[rt], 0, 0, 0);
                     }
                 }
             }

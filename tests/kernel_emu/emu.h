@@ -99,6 +99,27 @@ inline V4 mfma_16x16x32_bf16(pf_bf16x8 a, pf_bf16x8 b, V4 c, int, int, int) {
     w.bar.wait();
     return d;
 }
+// OCP e4m3fn -> float (exact): 1 sign, 4 exponent bits (bias 7), 3 mantissa bits; exponent 0 is subnormal
+inline float e4m3_to_float(uint8_t b) {
+    const int e = (b >> 3) & 15, m = b & 7;
+    float v;
+    if (e == 15 && m == 7) v = std::nanf("");
+    else if (e == 0) v = std::ldexp((float)m, -9);
+    else v = std::ldexp(1.0f + (float)m / 8.0f, e - 7);
+    return (b & 0x80) ? -v : v;
+}
+struct bf16x2 { uint16_t v[2]; };
+// v_cvt_scalef32_pk_bf16_fp8: bytes 0, 1 (hi = false) or 2, 3 (hi = true) of src as two bf16 numbers times scale
+inline bf16x2 cvt_scalef32_pk_bf16_fp8(uint32_t src, float scale, bool hi) {
+    bf16x2 r;
+    for (int i = 0; i < 2; ++i) {
+        const float f = e4m3_to_float((uint8_t)(src >> (8 * ((hi ? 2 : 0) + i)))) * scale;
+        uint32_t u;
+        std::memcpy(&u, &f, 4);
+        r.v[i] = (uint16_t)(u >> 16);                      // every e4m3 number is a bf16 number: nothing is rounded away
+    }
+    return r;
+}
 // runs kernel(args) over the grid, one workgroup after the other
 template <class K, class A>
 inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, const A &args) {
@@ -130,5 +151,6 @@ inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, cons
 #define __uint_as_float(u) emu::uint_as_float(u)
 #define __builtin_amdgcn_perm(a, b, s) emu::perm((a), (b), (s))
 #define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) emu::mfma_16x16x32_bf16((a), (b), (c), (x), (y), (z))
+#define __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(s, f, h) emu::cvt_scalef32_pk_bf16_fp8((s), (f), (h))
 #define PF_REG_CONST_S(var, lit) var = lit
 #define PF_REG_CONST_V(var, lit) var = lit

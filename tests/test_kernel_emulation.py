@@ -1,4 +1,4 @@
-"""The 4-bit few-row GEMM kernel's own source text, compiled for the host and run thread for thread on the CPU
+"""The 4-bit and e4m3 few-row GEMM kernels' own source text, compiled for the host and run thread for thread on the CPU
 (tests/kernel_emu/emu.h stands in for workgroups, waves, LDS, shuffles and the matrix instruction) under the
 launch plans the library itself works out, with AddressSanitizer and UBSan: results against a plain fp64
 product, every result element written, and no access outside the operands, the planes or the LDS.  What this
@@ -39,17 +39,25 @@ def emulator(tmp_path_factory):
     assert kernel.count(lds_decl) == 1
     (build / "kernel_i4.inc").write_text(kernel.replace(lds_decl, "uint16_t *s_act = emu::lds();"))
     (build / "pfgemm_struct.inc").write_text(re.search(r"struct PfGemm \{.*?\n\};\n", text, flags=re.S).group(0))
-    exe = build / "few_row_i4"
-    cmd = [cxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
-           "-pthread", "-I", str(build), "-I", EMU, os.path.join(EMU, "few_row_i4.cpp"), "-o", str(exe)]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    assert r.returncode == 0, r.stderr[-4000:]
-    return str(exe)
+    start, end = text.index("#define PF_S8_GU"), text.index("// ---------------------------------------------------------------- causal attention over the chunk")
+    kernel = text[start:end]
+    assert "void k_pf_gemm_skinny_f8(PfGemm g)" in kernel and kernel.count(lds_decl) == 1
+    (build / "kernel_f8.inc").write_text(kernel.replace(lds_decl, "uint16_t *s_act = emu::lds();"))
+    exes = {}
+    for name, extra in (("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"])):
+        exe = build / name
+        cmd = [cxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
+               "-pthread", *extra, "-I", str(build), "-I", EMU, os.path.join(EMU, name + ".cpp"), "-o", str(exe)]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-4000:]
+        exes[name] = str(exe)
+    return exes
 
 
-def run_case(exe, rows, n, k, num_cu, seed, lds_delta=0):
-    p = hipdec.gemm_plan(WeightDtype.INT4_G128, rows, n, k, num_cu)
-    assert p["kernel"] == "few_row_int4"
+def run_case(exes, wd, rows, n, k, num_cu, seed, lds_delta=0):
+    p = hipdec.gemm_plan(wd, rows, n, k, num_cu)
+    assert p["kernel"] == ("few_row_int4" if wd == WeightDtype.INT4_G128 else "few_row_e4m3")
+    exe = exes["few_row_i4" if wd == WeightDtype.INT4_G128 else "few_row_f8"]
     args = [rows, n, k, p["steps_per_split"], *p["grid"], p["threads"], p["lds_bytes"] + lds_delta, seed]
     r = subprocess.run([exe] + [str(a) for a in args], capture_output=True, text=True, timeout=600)
     return p, r
@@ -67,12 +75,27 @@ CASES = [
 
 @pytest.mark.parametrize("rows,n,k,num_cu", CASES)
 def test_four_bit_few_row_kernel_source_on_the_cpu(emulator, rows, n, k, num_cu):
-    p, r = run_case(emulator, rows, n, k, num_cu, seed=rows * 1000 + n)
+    p, r = run_case(emulator, WeightDtype.INT4_G128, rows, n, k, num_cu, seed=rows * 1000 + n)
     assert r.returncode == 0, (p, r.stdout, r.stderr[-3000:])
     assert "not written 0" in r.stdout
 
 
-def test_the_sanitizer_sees_an_access_past_the_lds(emulator):
-    # the control for the test above: with less LDS than the staged rows take, the same launch is reported
-    p, r = run_case(emulator, 8, 300, 384, 256, 1, lds_delta=-640)
+# e4m3: reductions of 1 to 32 blocks of 64 elements (k need not be a multiple of 128), splits of 1 to 8 blocks
+CASES_E4M3 = [
+    (8, 300, 384, 256), (5, 130, 1152, 256), (1, 16, 64, 256), (3, 257, 704, 256), (8, 256, 2048, 2), (7, 384, 1024, 1),
+    (16, 200, 640, 256), (9, 129, 448, 256), (19, 160, 1024, 256), (20, 160, 1024, 256), (27, 70, 384, 256), (32, 144, 640, 256),
+]
+
+
+@pytest.mark.parametrize("rows,n,k,num_cu", CASES_E4M3)
+def test_e4m3_few_row_kernel_source_on_the_cpu(emulator, rows, n, k, num_cu):
+    p, r = run_case(emulator, WeightDtype.FP8_E4M3, rows, n, k, num_cu, seed=rows * 1000 + n)
+    assert r.returncode == 0, (p, r.stdout, r.stderr[-3000:])
+    assert "not written 0" in r.stdout
+
+
+@pytest.mark.parametrize("wd", [WeightDtype.INT4_G128, WeightDtype.FP8_E4M3])
+def test_the_sanitizer_sees_an_access_past_the_lds(emulator, wd):
+    # the control for the tests above: with less LDS than the staged rows take, the same launch is reported
+    p, r = run_case(emulator, wd, 8, 300, 384, 256, 1, lds_delta=-640)
     assert r.returncode != 0 and "heap-buffer-overflow" in r.stderr, (p, r.stdout, r.stderr[-2000:])
