@@ -21,6 +21,16 @@ struct pf_bf16x8 { uint16_t v[8]; };
 template <class T> static inline T min(T a, T b) { return b < a ? b : a; }
 template <class T> static inline T max(T a, T b) { return a < b ? b : a; }
 
+// (the two conversions of hipdec_common.h that the kernels' helpers call)
+static inline float bf16_to_f32(uint16_t h) { const uint32_t u = (uint32_t)h << 16; float f; std::memcpy(&f, &u, 4); return f; }
+static inline uint16_t f32_to_bf16_rne(float f) {
+    uint32_t u; std::memcpy(&u, &f, 4);
+    if ((u & 0x7f800000u) == 0x7f800000u) return (uint16_t)(u >> 16);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+enum { WT_F32 = 0, WT_BF16 = 1, WT_FP8 = 2, WT_INT4 = 3 };
+
 namespace emu {
 class Barrier {
 public:
@@ -120,6 +130,37 @@ inline bf16x2 cvt_scalef32_pk_bf16_fp8(uint32_t src, float scale, bool hi) {
     }
     return r;
 }
+// v_mfma_f32_32x32x16_bf16: D = A (32 x 16) . B (16 x 32) + C.  Lane l supplies row l % 32 of A and column l % 32
+// of B, reduction elements 8 * (l / 32) .. + 7 of each; register i of lane l holds
+// D[8 * (i / 4) + 4 * (l / 32) + i % 4][l % 32].
+template <class V16>
+inline V16 mfma_32x32x16_bf16(pf_bf16x8 a, pf_bf16x8 b, V16 c, int, int, int) {
+    Wave &w = wave();
+    const int l = lane();
+    std::memcpy(w.a[l], a.v, 16);
+    std::memcpy(w.b[l], b.v, 16);
+    w.bar.wait();
+    V16 d = c;
+    for (int r = 0; r < 16; ++r) {
+        const int i = 8 * (r / 4) + 4 * (l / 32) + r % 4, j = l % 32;
+        double s = 0.0;
+        for (int k = 0; k < 16; ++k) {
+            const uint16_t *ar = (const uint16_t *)w.a[(k / 8) * 32 + i], *br = (const uint16_t *)w.b[(k / 8) * 32 + j];
+            s += (double)bf16_to_float(ar[k % 8]) * (double)bf16_to_float(br[k % 8]);
+        }
+        d[r] = (float)((double)c[r] + s);
+    }
+    w.bar.wait();
+    return d;
+}
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+// v_cvt_pk_f32_fp8: bytes 0, 1 (hi = false) or 2, 3 (hi = true) of src as two floats
+inline f32x2 cvt_pk_f32_fp8(uint32_t src, bool hi) {
+    f32x2 r;
+    for (int i = 0; i < 2; ++i) r[i] = e4m3_to_float((uint8_t)(src >> (8 * ((hi ? 2 : 0) + i))));
+    return r;
+}
+inline uint32_t float_as_uint(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
 // runs kernel(args) over the grid, one workgroup after the other
 template <class K, class A>
 inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, const A &args) {
@@ -151,6 +192,10 @@ inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, cons
 #define __uint_as_float(u) emu::uint_as_float(u)
 #define __builtin_amdgcn_perm(a, b, s) emu::perm((a), (b), (s))
 #define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) emu::mfma_16x16x32_bf16((a), (b), (c), (x), (y), (z))
+#define __shared__ static
+#define __float_as_uint(f) emu::float_as_uint(f)
+#define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) emu::mfma_32x32x16_bf16((a), (b), (c), (x), (y), (z))
+#define __builtin_amdgcn_cvt_pk_f32_fp8(s, h) emu::cvt_pk_f32_fp8((s), (h))
 #define __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(s, f, h) emu::cvt_scalef32_pk_bf16_fp8((s), (f), (h))
 #define PF_REG_CONST_S(var, lit) var = lit
 #define PF_REG_CONST_V(var, lit) var = lit

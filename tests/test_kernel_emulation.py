@@ -1,13 +1,15 @@
-"""The 4-bit and e4m3 few-row GEMM kernels' own source text, compiled for the host and run thread for thread on the CPU
+"""The few-row GEMM kernels' own source text (the 4-bit one, the e4m3 one and the general one), compiled for the host and run thread for thread on the CPU
 (tests/kernel_emu/emu.h stands in for workgroups, waves, LDS, shuffles and the matrix instruction) under the
 launch plans the library itself works out, with AddressSanitizer and UBSan: results against a plain fp64
 product, every result element written, and no access outside the operands, the planes or the LDS.  What this
 cannot show is the compiler's and the hardware's side (covered by the GPU tests); what it does show is the
 kernel's indexing, its arithmetic identities and the host/kernel contract for shapes and row counts at will."""
+import json
 import os
 import re
 import shutil
 import subprocess
+import sys
 
 import pytest
 
@@ -43,8 +45,14 @@ def emulator(tmp_path_factory):
     kernel = text[start:end]
     assert "void k_pf_gemm_skinny_f8(PfGemm g)" in kernel and kernel.count(lds_decl) == 1
     (build / "kernel_f8.inc").write_text(kernel.replace(lds_decl, "uint16_t *s_act = emu::lds();"))
+    # the general kernel with the two helpers it calls (the pair split of fp32 weights)
+    helpers = text[text.index("typedef __bf16 pf_bf16x2 __attribute__((ext_vector_type(2)));"):text.index("__device__ __forceinline__ float pf_block_sum(")]
+    kernel = text[text.index("#define PF_SK_UNROLL 4"):text.index("// The few-row GEMM for 4-bit weights.  In k_pf_gemm_skinny")]
+    assert "void k_pf_gemm_skinny(PfGemm g)" in kernel and kernel.count(lds_decl) == 1 and "pf_split2" in helpers
+    (build / "kernel_few.inc").write_text(helpers + kernel.replace(lds_decl, "uint16_t *s_act = emu::lds();"))
     exes = {}
-    for name, extra in (("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"])):
+    for name, extra in (("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
+                        ("few_row_general", ["-Wno-psabi"])):
         exe = build / name
         cmd = [cxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
                "-pthread", *extra, "-I", str(build), "-I", EMU, os.path.join(EMU, name + ".cpp"), "-o", str(exe)]
@@ -99,3 +107,28 @@ def test_the_sanitizer_sees_an_access_past_the_lds(emulator, wd):
     # the control for the tests above: with less LDS than the staged rows take, the same launch is reported
     p, r = run_case(emulator, wd, 8, 300, 384, 256, 1, lds_delta=-640)
     assert r.returncode != 0 and "heap-buffer-overflow" in r.stderr, (p, r.stdout, r.stderr[-2000:])
+
+
+# the general few-row kernel: all four weight formats (fp32 weights as bf16 pairs, bf16, e4m3 widened in registers,
+# 4-bit through the integer trick); the library plans it for e4m3 and 4-bit weights only with the kernels of their
+# own switched off, which the environment decides once per process -- so these plans come from a child process
+CASES_GENERAL = [(8, 100, 384, 256), (5, 130, 1152, 256), (16, 65, 640, 256), (27, 70, 384, 256), (32, 64, 1024, 2), (1, 33, 128, 256)]
+
+
+@pytest.fixture(scope="module")
+def general_plans():
+    code = ("import json; from rustane_amd import hipdec; "
+            "print(json.dumps([[wd, c, hipdec.gemm_plan(wd, *c)] for wd in range(4) for c in %r if not (wd == 3 and c[2] %% 128)]))" % (CASES_GENERAL,))
+    env = dict(os.environ, HIPDEC_NO_SKINNY_I4="1", HIPDEC_NO_SKINNY_F8="1")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=ROOT, env=env, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    return json.loads(r.stdout)
+
+
+def test_general_few_row_kernel_source_on_the_cpu(emulator, general_plans):
+    assert len(general_plans) == 4 * len(CASES_GENERAL)
+    for wd, (rows, n, k, num_cu), p in general_plans:
+        assert p["kernel"] == "few_row", (wd, p)
+        args = [wd, rows, n, k, p["steps_per_split"], *p["grid"], p["threads"], p["lds_bytes"], rows * 1000 + n]
+        r = subprocess.run([emulator["few_row_general"]] + [str(a) for a in args], capture_output=True, text=True, timeout=600)
+        assert r.returncode == 0 and "not written 0" in r.stdout, (wd, p, r.stdout, r.stderr[-3000:])
