@@ -17,6 +17,10 @@ struct uint2 { uint32_t x, y; };
 struct dim3 { unsigned x, y, z; };
 static inline uint4 make_uint4(uint32_t x, uint32_t y, uint32_t z, uint32_t w) { return uint4{x, y, z, w}; }
 static inline uint2 make_uint2(uint32_t x, uint32_t y) { return uint2{x, y}; }
+struct float4 { float x, y, z, w; };
+struct float2 { float x, y; };
+static inline float4 make_float4(float x, float y, float z, float w) { return float4{x, y, z, w}; }
+static inline float2 make_float2(float x, float y) { return float2{x, y}; }
 struct pf_bf16x8 { uint16_t v[8]; };
 template <class T> static inline T min(T a, T b) { return b < a ? b : a; }
 template <class T> static inline T max(T a, T b) { return a < b ? b : a; }
@@ -61,7 +65,7 @@ struct Block {
     std::vector<Wave> waves;
     unsigned char *lds;
 };
-inline thread_local dim3 tl_thread, tl_block, tl_grid;
+inline thread_local dim3 tl_thread, tl_block, tl_grid, tl_blockdim;
 inline thread_local Block *tl_blk = nullptr;
 inline Wave &wave() { return tl_blk->waves[tl_thread.x >> 6]; }
 inline int lane() { return (int)(tl_thread.x & 63); }
@@ -161,9 +165,9 @@ inline f32x2 cvt_pk_f32_fp8(uint32_t src, bool hi) {
     return r;
 }
 inline uint32_t float_as_uint(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
-// runs kernel(args) over the grid, one workgroup after the other
-template <class K, class A>
-inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, const A &args) {
+// runs body() as every thread of every workgroup of the grid, one workgroup after the other
+template <class F>
+inline void launch_fn(F body, dim3 grid, unsigned threads, size_t lds_bytes) {
     for (unsigned bz = 0; bz < grid.z; ++bz)
         for (unsigned by = 0; by < grid.y; ++by)
             for (unsigned bx = 0; bx < grid.x; ++bx) {
@@ -172,11 +176,15 @@ inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, cons
                 ts.reserve(threads);
                 for (unsigned t = 0; t < threads; ++t)
                     ts.emplace_back([&, t] {
-                        tl_thread = dim3{t, 0, 0}; tl_block = dim3{bx, by, bz}; tl_grid = grid; tl_blk = &blk;
-                        kernel(args);
+                        tl_thread = dim3{t, 0, 0}; tl_block = dim3{bx, by, bz}; tl_grid = grid; tl_blockdim = dim3{threads, 1, 1}; tl_blk = &blk;
+                        body();
                     });
                 for (auto &th : ts) th.join();
             }
+}
+template <class K, class A>
+inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, const A &args) {
+    launch_fn([&] { kernel(args); }, grid, threads, lds_bytes);
 }
 }  // namespace emu
 
@@ -187,6 +195,8 @@ inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, cons
 #define threadIdx emu::tl_thread
 #define blockIdx emu::tl_block
 #define gridDim emu::tl_grid
+#define blockDim emu::tl_blockdim
+#define WAVE 64
 #define __syncthreads() emu::sync_block()
 #define __shfl_xor(v, m, w) emu::shfl_xor((v), (m), (w))
 #define __uint_as_float(u) emu::uint_as_float(u)
@@ -199,3 +209,8 @@ inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, cons
 #define __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(s, f, h) emu::cvt_scalef32_pk_bf16_fp8((s), (f), (h))
 #define PF_REG_CONST_S(var, lit) var = lit
 #define PF_REG_CONST_V(var, lit) var = lit
+// (the wave reduction of hipdec_common.h: xor shuffles over 32 .. 1)
+static inline float wave_sum(float v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}

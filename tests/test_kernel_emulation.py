@@ -50,8 +50,16 @@ def emulator(tmp_path_factory):
     kernel = text[text.index("#define PF_SK_UNROLL 4"):text.index("// The few-row GEMM for 4-bit weights.  In k_pf_gemm_skinny")]
     assert "void k_pf_gemm_skinny(PfGemm g)" in kernel and kernel.count(lds_decl) == 1 and "pf_split2" in helpers
     (build / "kernel_few.inc").write_text(helpers + kernel.replace(lds_decl, "uint16_t *s_act = emu::lds();"))
+    # the element-wise kernels between the products (with the helpers in front of them) and the multi-row step's two
+    batch = open(os.path.join(ROOT, "rustane_amd", "csrc", "hipdec_batch.h")).read()
+    epi = (text[text.index("// f16 != 0: the activation as ONE fp16 number in hi"):text.index("// ---------------------------------------------------------------- GEMM on the bf16 matrix cores")]
+           + batch[batch.index("struct BatchParams {"):batch.index("// One workgroup per (head, row): online softmax over the shared prefix rows")]
+           + batch[batch.index("// logits[r][v] = inv_rms[r] * sum_z P[z][r][v]"):batch.index("// ---- head kernels, one grid row per sequence")])
+    for k in ("void k_pf_resid(", "void k_pf_gate_epi(", "void k_bd_qkv_epi(", "void k_bd_sum_planes(", "void pf_sum_planes("):
+        assert k in epi, k
+    (build / "kernels_epi.inc").write_text(epi)
     exes = {}
-    for name, extra in (("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
+    for name, extra in (("epilogues", ["-Wno-psabi"]), ("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
                         ("few_row_general", ["-Wno-psabi"])):
         exe = build / name
         cmd = [cxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
@@ -132,3 +140,11 @@ def test_general_few_row_kernel_source_on_the_cpu(emulator, general_plans):
         args = [wd, rows, n, k, p["steps_per_split"], *p["grid"], p["threads"], p["lds_bytes"], rows * 1000 + n]
         r = subprocess.run([emulator["few_row_general"]] + [str(a) for a in args], capture_output=True, text=True, timeout=600)
         assert r.returncode == 0 and "not written 0" in r.stdout, (wd, p, r.stdout, r.stderr[-3000:])
+
+
+def test_element_wise_kernels_source_on_the_cpu(emulator):
+    # k_pf_resid, k_pf_gate_epi, k_bd_qkv_epi (both cache formats) and k_bd_sum_planes against fp64 restatements, with
+    # split counts on both sides of the plane sums' request rounds of four and eight
+    r = subprocess.run([emulator["epilogues"]], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
+    assert r.stdout.count("k_pf_resid") >= 11 and r.stdout.count("k_bd_qkv_epi") >= 6
