@@ -4,6 +4,7 @@
 // sound where the kernel calls them under wave-uniform control flow, as these kernels do.
 #pragma once
 #include <cmath>
+#include <atomic>
 #include <condition_variable>
 #include <cstdint>
 #include <cstdlib>
@@ -51,10 +52,17 @@ private:
     int n_, count_ = 0;
     unsigned gen_ = 0;
 };
+// one lane's side of the shuffles: value n of the lane (two slots, by the parity of n), how many it has published
+// and how many of them its partners have read
+struct ShuffleBox {
+    float val[2] = {0.0f, 0.0f};
+    std::atomic<uint64_t> published{0}, consumed[2] = {{0}, {0}};   // consumed: reads of the values a slot has held
+    uint64_t count = 0;                                  // (touched by the owning lane only)
+};
 struct Wave {
     Barrier bar{64};
     uint32_t a[64][4], b[64][4];
-    float f[64];
+    ShuffleBox box[64];
 };
 struct Block {
     // the dynamic LDS is a heap block of exactly the size the launch asked for: under AddressSanitizer an access past
@@ -73,12 +81,21 @@ inline uint16_t *lds() { return (uint16_t *)tl_blk->lds; }
 inline void sync_block() { tl_blk->bar.wait(); }
 inline float bf16_to_float(uint16_t h) { const uint32_t u = (uint32_t)h << 16; float f; std::memcpy(&f, &u, 4); return f; }
 inline float uint_as_float(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
+// A shuffle is a rendezvous of the two lanes that exchange, not of the wave: the kernels also shuffle inside
+// branches that only some lane groups of a wave take (every lane's partner takes the same branch, so the two run
+// the same sequence of shuffles).  Lane l publishes its n-th value, waits for its partner's n-th, reads it and
+// says so; it reuses a slot only after every value the slot has held has been read (reads of different values can
+// finish out of order: their readers are different lanes).
 inline float shfl_xor(float v, int mask, int) {
     Wave &w = wave();
-    w.f[lane()] = v;
-    w.bar.wait();
-    const float r = w.f[lane() ^ mask];
-    w.bar.wait();
+    ShuffleBox &mine = w.box[lane()], &theirs = w.box[lane() ^ mask];
+    const uint64_t n = ++mine.count;
+    while (mine.consumed[n & 1].load(std::memory_order_acquire) < (n - 1) / 2) std::this_thread::yield();   // the slot's earlier values
+    mine.val[n & 1] = v;
+    mine.published.store(n, std::memory_order_release);
+    while (theirs.published.load(std::memory_order_acquire) < n) std::this_thread::yield();
+    const float r = theirs.val[n & 1];
+    theirs.consumed[n & 1].fetch_add(1, std::memory_order_release);
     return r;
 }
 // v_perm_b32: result byte i is byte sel[i] of the eight bytes {s0 (4..7), s1 (0..3)}
@@ -200,6 +217,7 @@ inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, cons
 #define __syncthreads() emu::sync_block()
 #define __shfl_xor(v, m, w) emu::shfl_xor((v), (m), (w))
 #define __uint_as_float(u) emu::uint_as_float(u)
+#define __expf(x) expf(x)
 #define __builtin_amdgcn_perm(a, b, s) emu::perm((a), (b), (s))
 #define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) emu::mfma_16x16x32_bf16((a), (b), (c), (x), (y), (z))
 #define __shared__ static

@@ -58,8 +58,16 @@ def emulator(tmp_path_factory):
     for k in ("void k_pf_resid(", "void k_pf_gate_epi(", "void k_bd_qkv_epi(", "void k_bd_sum_planes(", "void pf_sum_planes("):
         assert k in epi, k
     (build / "kernels_epi.inc").write_text(epi)
+    # the multi-row step's attention kernel with the cache-row decoders and the pair split it calls
+    common = open(os.path.join(ROOT, "rustane_amd", "csrc", "hipdec_common.h")).read()
+    att = (common[common.index("template <int WT> struct WS;"):common.index("template <> struct WS<WT_FP8> {")]
+           + text[text.index("// f16 != 0: the activation as ONE fp16 number in hi"):text.index("typedef __bf16 pf_bf16x2 __attribute__((ext_vector_type(2)));")]
+           + batch[batch.index("struct BatchParams {"):batch.index("// q/k/v rows of the step: sum the split planes")]
+           + batch[batch.index("// One workgroup per (head, row): online softmax over the shared prefix rows"):batch.index("// logits[r][v] = inv_rms[r] * sum_z P[z][r][v]")])
+    assert "void k_bd_attn(" in att and "struct WS<WT_BF16>" in att and "void pf_split(" in att
+    (build / "kernel_bd_attn.inc").write_text(att)
     exes = {}
-    for name, extra in (("epilogues", ["-Wno-psabi"]), ("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
+    for name, extra in (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
                         ("few_row_general", ["-Wno-psabi"])):
         exe = build / name
         cmd = [cxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
@@ -148,3 +156,11 @@ def test_element_wise_kernels_source_on_the_cpu(emulator):
     r = subprocess.run([emulator["epilogues"]], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
     assert r.stdout.count("k_pf_resid") >= 11 and r.stdout.count("k_bd_qkv_epi") >= 6
+
+
+def test_multi_row_attention_kernel_source_on_the_cpu(emulator):
+    # k_bd_attn (1024 threads per (head, row)) against an fp64 softmax attention over prefix + suffix rows: both cache
+    # formats, head dimensions 64 and 128, grouped heads, row counts below one pass, inside a pass and over several
+    r = subprocess.run([emulator["batch_attention"]], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
+    assert r.stdout.count("k_bd_attn<") == 6
