@@ -98,6 +98,12 @@ inline float shfl_xor(float v, int mask, int) {
     theirs.consumed[n & 1].fetch_add(1, std::memory_order_release);
     return r;
 }
+inline int shfl_xor(int v, int mask, int width) {
+    float f; std::memcpy(&f, &v, 4);
+    f = shfl_xor(f, mask, width);                        // (bits only: nothing is computed on the way)
+    std::memcpy(&v, &f, 4);
+    return v;
+}
 // v_perm_b32: result byte i is byte sel[i] of the eight bytes {s0 (4..7), s1 (0..3)}
 inline uint32_t perm(uint32_t s0, uint32_t s1, uint32_t sel) {
     const uint64_t both = ((uint64_t)s0 << 32) | s1;

@@ -66,8 +66,14 @@ def emulator(tmp_path_factory):
            + batch[batch.index("// One workgroup per (head, row): online softmax over the shared prefix rows"):batch.index("// logits[r][v] = inv_rms[r] * sum_z P[z][r][v]")])
     assert "void k_bd_attn(" in att and "struct WS<WT_BF16>" in att and "void pf_split(" in att
     (build / "kernel_bd_attn.inc").write_text(att)
+    # the multi-row step's greedy and top-k head kernels with the ordering they share
+    sel = (common[common.index("// (value desc, index asc) ordering used by every head kernel of the reference"):common.index("// 16-byte load of data that is used once per step")]
+           + batch[batch.index("struct BatchParams {"):batch.index("// q/k/v rows of the step: sum the split planes")]
+           + batch[batch.index("// ---- head kernels, one grid row per sequence"):batch.index("__global__ __launch_bounds__(256) void k_bd_block_stats(")])
+    assert "void k_bd_argmax(" in sel and "void k_bd_topk(" in sel and "bool better(" in sel
+    (build / "kernels_sel.inc").write_text(sel)
     exes = {}
-    for name, extra in (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
+    for name, extra in (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("selection", []), ("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
                         ("few_row_general", ["-Wno-psabi"])):
         exe = build / name
         cmd = [cxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
@@ -164,3 +170,11 @@ def test_multi_row_attention_kernel_source_on_the_cpu(emulator):
     r = subprocess.run([emulator["batch_attention"]], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
     assert r.stdout.count("k_bd_attn<") == 6
+
+
+def test_greedy_and_top_k_head_kernels_source_on_the_cpu(emulator):
+    # k_bd_argmax and k_bd_topk against a sort by (value descending, index ascending): ties, -inf entries, a block of
+    # nothing but -inf, vocabularies that end inside a block, k above the number of rows (padded lists)
+    r = subprocess.run([emulator["selection"]], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
+    assert r.stdout.count("0 mismatches") == 5
