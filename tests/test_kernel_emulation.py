@@ -72,8 +72,20 @@ def emulator(tmp_path_factory):
            + batch[batch.index("// ---- head kernels, one grid row per sequence"):batch.index("__global__ __launch_bounds__(256) void k_bd_block_stats(")])
     assert "void k_bd_argmax(" in sel and "void k_bd_topk(" in sel and "bool better(" in sel
     (build / "kernels_sel.inc").write_text(sel)
+    # the weight conversion kernel with the e4m3 encoder; the oracle's C file is linked in as its checker
+    kern = open(os.path.join(ROOT, "rustane_amd", "csrc", "hipdec_kernels.h")).read()
+    enc = common[common.index("// software OCP e4m3fn encoder, round to nearest even, saturating"):]
+    conv = (enc[:enc.index("\n}\n") + 3]
+            + common[common.index("__device__ __forceinline__ float wave_max(float v) {"):common.index("// (value desc, index asc) ordering used by every head kernel of the reference")]
+            + kern[kern.index("// one workgroup per source row of an out-major fp32 matrix [rows][K]; destination row ="):kern.index("// inverse of k_convert_rows for verification: stored row -> fp32")])
+    assert "void k_convert_rows(" in conv and "uint8_t f32_to_e4m3(" in conv
+    (build / "kernel_convert.inc").write_text(conv)
+    oracle_o = build / "oracle.o"
+    r = subprocess.run([cxx.replace("clang++", "clang"), "-O1", "-w", "-c", os.path.join(ROOT, "oracle", "rustane_oracle.c"), "-o", str(oracle_o)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
     exes = {}
-    for name, extra in (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("selection", []), ("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
+    for name, extra in (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("selection", []), ("convert_rows", [str(oracle_o), "-lm"]), ("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
                         ("few_row_general", ["-Wno-psabi"])):
         exe = build / name
         cmd = [cxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
@@ -178,3 +190,11 @@ def test_greedy_and_top_k_head_kernels_source_on_the_cpu(emulator):
     r = subprocess.run([emulator["selection"]], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
     assert r.stdout.count("0 mismatches") == 5
+
+
+def test_weight_conversion_kernel_source_on_the_cpu(emulator):
+    # k_convert_rows: stored e4m3 rows + row scales and stored 4-bit rows + bf16 group scales bit for bit against the
+    # oracle's quantisers, bf16 rows to the nearest, with the interleaving row map
+    r = subprocess.run([emulator["convert_rows"]], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
+    assert r.stdout.count("0 mismatches") == 4
