@@ -224,6 +224,9 @@ inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, cons
 #define __shfl_xor(v, m, w) emu::shfl_xor((v), (m), (w))
 #define __uint_as_float(u) emu::uint_as_float(u)
 #define __expf(x) expf(x)
+#define __threadfence() std::atomic_thread_fence(std::memory_order_seq_cst)
+// (workgroups run one after the other here, so "the last workgroup to arrive" is the last of the grid)
+static inline unsigned atomicAdd(unsigned *p, unsigned v) { return __atomic_fetch_add(p, v, __ATOMIC_SEQ_CST); }
 #define __builtin_amdgcn_perm(a, b, s) emu::perm((a), (b), (s))
 #define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) emu::mfma_16x16x32_bf16((a), (b), (c), (x), (y), (z))
 #define __shared__ static

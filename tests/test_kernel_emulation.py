@@ -80,12 +80,18 @@ def emulator(tmp_path_factory):
             + kern[kern.index("// one workgroup per source row of an out-major fp32 matrix [rows][K]; destination row ="):kern.index("// inverse of k_convert_rows for verification: stored row -> fp32")])
     assert "void k_convert_rows(" in conv and "uint8_t f32_to_e4m3(" in conv
     (build / "kernel_convert.inc").write_text(conv)
+    # the single-row attention kernel of the one-kernel-per-product path
+    ad = (common[common.index("struct StepParams {"):common.index("enum { WT_F32 = 0")]
+          + common[common.index("template <int WT> struct WS;"):common.index("template <> struct WS<WT_FP8> {")]
+          + kern[kern.index("// ---------------------------------------------------------------- attention (one query row)"):kern.index("// ---------------------------------------------------------------- heads (on the raw logits)")])
+    assert "void k_attn_decode(" in ad
+    (build / "kernel_attn_decode.inc").write_text(ad)
     oracle_o = build / "oracle.o"
     r = subprocess.run([cxx.replace("clang++", "clang"), "-O1", "-w", "-c", os.path.join(ROOT, "oracle", "rustane_oracle.c"), "-o", str(oracle_o)],
                        capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
     exes = {}
-    for name, extra in (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("selection", []), ("convert_rows", [str(oracle_o), "-lm"]), ("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
+    for name, extra in (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("selection", []), ("single_row_attention", ["-Wno-psabi"]), ("convert_rows", [str(oracle_o), "-lm"]), ("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
                         ("few_row_general", ["-Wno-psabi"])):
         exe = build / name
         cmd = [cxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
@@ -198,3 +204,11 @@ def test_weight_conversion_kernel_source_on_the_cpu(emulator):
     r = subprocess.run([emulator["convert_rows"]], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
     assert r.stdout.count("0 mismatches") == 4
+
+
+def test_single_row_attention_kernel_source_on_the_cpu(emulator):
+    # k_attn_decode ((head, split) workgroups, the last of a head folds the partial records) against an fp64 softmax
+    # attention: both cache formats, head dimensions 64 and 128, grouped heads, splits with few or no rows
+    r = subprocess.run([emulator["single_row_attention"]], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
+    assert r.stdout.count("k_attn_decode<") == 5
