@@ -187,6 +187,8 @@ inline f32x2 cvt_pk_f32_fp8(uint32_t src, bool hi) {
     for (int i = 0; i < 2; ++i) r[i] = e4m3_to_float((uint8_t)(src >> (8 * ((hi ? 2 : 0) + i))));
     return r;
 }
+// v_cvt_off_f32_i4: the low four bits as a two's complement number, over 16
+inline float cvt_off_f32_i4(int x) { int n = x & 15; if (n >= 8) n -= 16; return (float)n / 16.0f; }
 inline uint32_t float_as_uint(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
 // runs body() as every thread of every workgroup of the grid, one workgroup after the other
 template <class F>
@@ -233,6 +235,7 @@ static inline unsigned atomicAdd(unsigned *p, unsigned v) { return __atomic_fetc
 #define __float_as_uint(f) emu::float_as_uint(f)
 #define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) emu::mfma_32x32x16_bf16((a), (b), (c), (x), (y), (z))
 #define __builtin_amdgcn_cvt_pk_f32_fp8(s, h) emu::cvt_pk_f32_fp8((s), (h))
+#define __builtin_amdgcn_cvt_off_f32_i4(x) emu::cvt_off_f32_i4(x)
 #define __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(s, f, h) emu::cvt_scalef32_pk_bf16_fp8((s), (f), (h))
 #define PF_REG_CONST_S(var, lit) var = lit
 #define PF_REG_CONST_V(var, lit) var = lit

@@ -86,12 +86,21 @@ def emulator(tmp_path_factory):
           + kern[kern.index("// ---------------------------------------------------------------- attention (one query row)"):kern.index("// ---------------------------------------------------------------- heads (on the raw logits)")])
     assert "void k_attn_decode(" in ad
     (build / "kernel_attn_decode.inc").write_text(ad)
+    # the matrix-vector kernel of the same path with the four weight decoders (shared with the persistent kernels); its
+    # empty asm that pins a register names a GPU register class, and its LDS declaration becomes the stand-in's block
+    gv = (common[common.index("struct StepParams {"):common.index("enum { WT_F32 = 0")]
+          + common[common.index("template <int WT> struct WS;"):common.index("// software OCP e4m3fn encoder, round to nearest even, saturating")]
+          + kern[kern.index("enum { EPI_QKV = 0"):kern.index("// ---------------------------------------------------------------- embedding / input")]
+          + kern[kern.index("// ---------------------------------------------------------------- GEMV"):kern.index("// ---------------------------------------------------------------- attention (one query row)")])
+    pin, xs_decl = 'asm volatile("" : "+v"(hi));', "extern __shared__ __align__(16) float xs[];"
+    assert gv.count(pin) == 1 and gv.count(xs_decl) == 1 and "void k_gemv(GemvArgs a)" in gv
+    (build / "kernel_gemv.inc").write_text(gv.replace(pin, 'asm volatile("" : "+r"(hi));').replace(xs_decl, "float *xs = (float *)emu::lds();"))
     oracle_o = build / "oracle.o"
     r = subprocess.run([cxx.replace("clang++", "clang"), "-O1", "-w", "-c", os.path.join(ROOT, "oracle", "rustane_oracle.c"), "-o", str(oracle_o)],
                        capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
     exes = {}
-    for name, extra in (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("selection", []), ("single_row_attention", ["-Wno-psabi"]), ("convert_rows", [str(oracle_o), "-lm"]), ("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
+    for name, extra in (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("selection", []), ("single_row_attention", ["-Wno-psabi"]), ("gemv", ["-Wno-psabi"]), ("convert_rows", [str(oracle_o), "-lm"]), ("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
                         ("few_row_general", ["-Wno-psabi"])):
         exe = build / name
         cmd = [cxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
@@ -212,3 +221,11 @@ def test_single_row_attention_kernel_source_on_the_cpu(emulator):
     r = subprocess.run([emulator["single_row_attention"]], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
     assert r.stdout.count("k_attn_decode<") == 5
+
+
+def test_matrix_vector_kernel_source_on_the_cpu(emulator):
+    # k_gemv for fp32, bf16, e4m3 and 4-bit weights with every fused prologue / epilogue (RMSNorm in; RoPE + cache
+    # append with both cache formats, residual, both activations, logits out) against fp64 restatements
+    r = subprocess.run([emulator["gemv"]], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
+    assert r.stdout.count("k_gemv<format") == 28
