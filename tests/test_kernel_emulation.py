@@ -4,6 +4,7 @@ launch plans the library itself works out, with AddressSanitizer and UBSan: resu
 product, every result element written, and no access outside the operands, the planes or the LDS.  What this
 cannot show is the compiler's and the hardware's side (covered by the GPU tests); what it does show is the
 kernel's indexing, its arithmetic identities and the host/kernel contract for shapes and row counts at will."""
+import concurrent.futures
 import json
 import os
 import re
@@ -100,14 +101,20 @@ def emulator(tmp_path_factory):
                        capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
     exes = {}
-    for name, extra in (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("selection", []), ("single_row_attention", ["-Wno-psabi"]), ("gemv", ["-Wno-psabi"]), ("convert_rows", [str(oracle_o), "-lm"]), ("few_row_i4", []), ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]),
-                        ("few_row_general", ["-Wno-psabi"])):
-        exe = build / name
+    programs = (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("selection", []), ("single_row_attention", ["-Wno-psabi"]),
+                ("gemv", ["-Wno-psabi"]), ("convert_rows", [str(oracle_o), "-lm"]), ("few_row_i4", []),
+                ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]), ("few_row_general", ["-Wno-psabi"]))
+
+    def compile_one(item):
+        name, extra = item
         cmd = [cxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
-               "-pthread", *extra, "-I", str(build), "-I", EMU, os.path.join(EMU, name + ".cpp"), "-o", str(exe)]
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        assert r.returncode == 0, r.stderr[-4000:]
-        exes[name] = str(exe)
+               "-pthread", *extra, "-I", str(build), "-I", EMU, os.path.join(EMU, name + ".cpp"), "-o", str(build / name)]
+        return name, subprocess.run(cmd, capture_output=True, text=True)
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=4) as pool:
+        for name, r in pool.map(compile_one, programs):
+            assert r.returncode == 0, (name, r.stderr[-4000:])
+            exes[name] = str(build / name)
     return exes
 
 
