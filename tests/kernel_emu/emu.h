@@ -227,6 +227,13 @@ inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, cons
 #define __uint_as_float(u) emu::uint_as_float(u)
 #define __expf(x) expf(x)
 #define __threadfence() std::atomic_thread_fence(std::memory_order_seq_cst)
+#define __host__
+// single-rounding float operations (the programs that use them are built with floating-point contraction off)
+#define __fadd_rn(a, b) ((float)(a) + (float)(b))
+#define __fsub_rn(a, b) ((float)(a) - (float)(b))
+#define __fmul_rn(a, b) ((float)(a) * (float)(b))
+#define __fdiv_rn(a, b) ((float)(a) / (float)(b))
+#define __float_as_int(f) ((int)emu::float_as_uint(f))
 // (workgroups run one after the other here, so "the last workgroup to arrive" is the last of the grid)
 static inline unsigned atomicAdd(unsigned *p, unsigned v) { return __atomic_fetch_add(p, v, __ATOMIC_SEQ_CST); }
 #define __builtin_amdgcn_perm(a, b, s) emu::perm((a), (b), (s))

@@ -96,13 +96,22 @@ def emulator(tmp_path_factory):
     pin, xs_decl = 'asm volatile("" : "+v"(hi));', "extern __shared__ __align__(16) float xs[];"
     assert gv.count(pin) == 1 and gv.count(xs_decl) == 1 and "void k_gemv(GemvArgs a)" in gv
     (build / "kernel_gemv.inc").write_text(gv.replace(pin, 'asm volatile("" : "+r"(hi));').replace(xs_decl, "float *xs = (float *)emu::lds();"))
+    # the top-k draw on the device with the restated host expf / tanhf and the run state
+    smp = open(os.path.join(ROOT, "rustane_amd", "csrc", "hipdec_sample.h")).read()
+    draw = (common[common.index("// (value desc, index asc) ordering used by every head kernel of the reference"):common.index("// 16-byte load of data that is used once per step")]
+            + batch[batch.index("struct BatchParams {"):batch.index("// q/k/v rows of the step: sum the split planes")]
+            + smp[smp.index("__host__ __device__ __forceinline__ uint64_t sample_exp2_tab(unsigned i) {"):smp.index("// order-independent checksum of a restated function")]
+            + smp[smp.index("// ---------------------------------------------------------------- run state"):smp.index("// One workgroup per row: the block from the statistics, then the token inside the block.")])
+    assert "void k_sample_topk(" in draw and "float expf_as_host(" in draw and "float tanhf_as_host(" in draw
+    (build / "kernel_sample.inc").write_text(draw)
     oracle_o = build / "oracle.o"
     r = subprocess.run([cxx.replace("clang++", "clang"), "-O1", "-w", "-c", os.path.join(ROOT, "oracle", "rustane_oracle.c"), "-o", str(oracle_o)],
                        capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
     exes = {}
     programs = (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("selection", []), ("single_row_attention", ["-Wno-psabi"]),
-                ("gemv", ["-Wno-psabi"]), ("convert_rows", [str(oracle_o), "-lm"]), ("few_row_i4", []),
+                ("gemv", ["-Wno-psabi"]), ("convert_rows", [str(oracle_o), "-lm"]),
+                ("sample_topk", ["-ffp-contract=off", "-Wno-psabi", str(oracle_o), "-lm"]), ("few_row_i4", []),
                 ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]), ("few_row_general", ["-Wno-psabi"]))
 
     def compile_one(item):
@@ -236,3 +245,11 @@ def test_matrix_vector_kernel_source_on_the_cpu(emulator):
     r = subprocess.run([emulator["gemv"]], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
     assert r.stdout.count("k_gemv<format") == 28
+
+
+def test_top_k_draw_kernel_source_on_the_cpu(emulator):
+    # k_sample_topk (candidate merge, softcap, softmax draw, LCG, run state) against the oracle's restatement of the
+    # reference's host code, token for token and RNG state for RNG state over consecutive steps of several rows
+    r = subprocess.run([emulator["sample_topk"]], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
+    assert r.stdout.count("0 mismatches") == 5
