@@ -104,6 +104,17 @@ def emulator(tmp_path_factory):
             + smp[smp.index("// ---------------------------------------------------------------- run state"):smp.index("// One workgroup per row: the block from the statistics, then the token inside the block.")])
     assert "void k_sample_topk(" in draw and "float expf_as_host(" in draw and "float tanhf_as_host(" in draw
     (build / "kernel_sample.inc").write_text(draw)
+    # the full-vocabulary draw: block from the statistics, token inside the block
+    softcap_line = "__device__ __forceinline__ float softcap_dev(float x, float cap) { return cap > 0.0f ? cap * tanhf(x / cap) : x; }\n"
+    assert softcap_line in kern
+    fv = smp[smp.index("// One workgroup per row: the block from the statistics, then the token inside the block."):]
+    fv = (common[common.index("__device__ __forceinline__ float wave_max(float v) {"):common.index("// (value desc, index asc) ordering used by every head kernel of the reference")]
+          + batch[batch.index("struct BatchParams {"):batch.index("// q/k/v rows of the step: sum the split planes")] + softcap_line
+          + smp[smp.index("__host__ __device__ __forceinline__ uint64_t sample_exp2_tab(unsigned i) {"):smp.index("// order-independent checksum of a restated function")]
+          + smp[smp.index("// ---------------------------------------------------------------- run state"):smp.index("// One workgroup per row.  vals/idxs: [rows][blocks * top_k]")]
+          + "#define SAMPLE_MAX_BLOCKS 1024\n" + fv[:fv.index("\n}\n") + 3])
+    assert "void k_sample_fullvocab(" in fv and "#define SAMPLE_MAX_BLOCKS 1024" in smp
+    (build / "kernel_sample_fv.inc").write_text(fv)
     oracle_o = build / "oracle.o"
     r = subprocess.run([cxx.replace("clang++", "clang"), "-O1", "-w", "-c", os.path.join(ROOT, "oracle", "rustane_oracle.c"), "-o", str(oracle_o)],
                        capture_output=True, text=True)
@@ -111,7 +122,8 @@ def emulator(tmp_path_factory):
     exes = {}
     programs = (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("selection", []), ("single_row_attention", ["-Wno-psabi"]),
                 ("gemv", ["-Wno-psabi"]), ("convert_rows", [str(oracle_o), "-lm"]),
-                ("sample_topk", ["-ffp-contract=off", "-Wno-psabi", str(oracle_o), "-lm"]), ("few_row_i4", []),
+                ("sample_topk", ["-ffp-contract=off", "-Wno-psabi", str(oracle_o), "-lm"]),
+                ("sample_fullvocab", ["-ffp-contract=off", "-Wno-psabi", str(oracle_o), "-lm"]), ("few_row_i4", []),
                 ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]), ("few_row_general", ["-Wno-psabi"]))
 
     def compile_one(item):
@@ -253,3 +265,12 @@ def test_top_k_draw_kernel_source_on_the_cpu(emulator):
     r = subprocess.run([emulator["sample_topk"]], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
     assert r.stdout.count("0 mismatches") == 5
+
+
+def test_full_vocabulary_draw_kernel_source_on_the_cpu(emulator):
+    # k_sample_fullvocab (block from the statistics, then the token inside the block; two draws per token) against the
+    # oracle's restatement of the reference's host code, token for token and RNG state for RNG state, with blocks of
+    # nothing but -inf, softcap, a last block that is not full and more blocks than threads
+    r = subprocess.run([emulator["sample_fullvocab"]], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
+    assert r.stdout.count("0 mismatches") == 4
