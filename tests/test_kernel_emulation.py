@@ -115,6 +115,15 @@ def emulator(tmp_path_factory):
           + "#define SAMPLE_MAX_BLOCKS 1024\n" + fv[:fv.index("\n}\n") + 3])
     assert "void k_sample_fullvocab(" in fv and "#define SAMPLE_MAX_BLOCKS 1024" in smp
     (build / "kernel_sample_fv.inc").write_text(fv)
+    # the single-row head kernels and the multi-row block statistics
+    bst = batch[batch.index("__global__ __launch_bounds__(256) void k_bd_block_stats("):]
+    heads = (common[common.index("struct StepParams {"):common.index("enum { WT_F32 = 0")]
+             + common[common.index("__device__ __forceinline__ float wave_max(float v) {"):common.index("// 16-byte load of data that is used once per step")]
+             + kern[kern.index("// ---------------------------------------------------------------- heads (on the raw logits)"):kern.index("__global__ void k_advance(StepParams *sp)")]
+             + batch[batch.index("struct BatchParams {"):batch.index("// q/k/v rows of the step: sum the split planes")] + bst[:bst.index("\n}\n") + 3])
+    for k in ("void k_head_argmax(", "void k_head_topk(", "void k_head_block_stats(", "void k_softcap_copy(", "void k_bd_block_stats("):
+        assert k in heads, k
+    (build / "kernels_heads.inc").write_text(heads)
     oracle_o = build / "oracle.o"
     r = subprocess.run([cxx.replace("clang++", "clang"), "-O1", "-w", "-c", os.path.join(ROOT, "oracle", "rustane_oracle.c"), "-o", str(oracle_o)],
                        capture_output=True, text=True)
@@ -123,7 +132,8 @@ def emulator(tmp_path_factory):
     programs = (("epilogues", ["-Wno-psabi"]), ("batch_attention", ["-Wno-psabi"]), ("selection", []), ("single_row_attention", ["-Wno-psabi"]),
                 ("gemv", ["-Wno-psabi"]), ("convert_rows", [str(oracle_o), "-lm"]),
                 ("sample_topk", ["-ffp-contract=off", "-Wno-psabi", str(oracle_o), "-lm"]),
-                ("sample_fullvocab", ["-ffp-contract=off", "-Wno-psabi", str(oracle_o), "-lm"]), ("few_row_i4", []),
+                ("sample_fullvocab", ["-ffp-contract=off", "-Wno-psabi", str(oracle_o), "-lm"]),
+                ("single_row_heads", ["-ffp-contract=off", "-Wno-psabi", str(oracle_o), "-lm"]), ("few_row_i4", []),
                 ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]), ("few_row_general", ["-Wno-psabi"]))
 
     def compile_one(item):
@@ -272,5 +282,13 @@ def test_full_vocabulary_draw_kernel_source_on_the_cpu(emulator):
     # oracle's restatement of the reference's host code, token for token and RNG state for RNG state, with blocks of
     # nothing but -inf, softcap, a last block that is not full and more blocks than threads
     r = subprocess.run([emulator["sample_fullvocab"]], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
+    assert r.stdout.count("0 mismatches") == 4
+
+
+def test_single_row_head_kernels_source_on_the_cpu(emulator):
+    # k_head_argmax (with the step state it advances), k_head_topk (exact lists), k_head_block_stats / k_bd_block_stats
+    # (exact maxima, sums at 1e-5) and k_softcap_copy against the oracle's restatements
+    r = subprocess.run([emulator["single_row_heads"]], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
     assert r.stdout.count("0 mismatches") == 4
