@@ -180,6 +180,39 @@ inline V16 mfma_32x32x16_bf16(pf_bf16x8 a, pf_bf16x8 b, V16 c, int, int, int) {
     w.bar.wait();
     return d;
 }
+// v_mfma_f32_32x32x16_f16: the same tile shape and lane layout with fp16 operands
+template <class H8, class V16>
+inline V16 mfma_32x32x16_f16(H8 a, H8 b, V16 c, int, int, int) {
+    Wave &w = wave();
+    const int l = lane();
+    std::memcpy(w.a[l], &a, 16);
+    std::memcpy(w.b[l], &b, 16);
+    w.bar.wait();
+    V16 d = c;
+    for (int r = 0; r < 16; ++r) {
+        const int i = 8 * (r / 4) + 4 * (l / 32) + r % 4, j = l % 32;
+        double s = 0.0;
+        for (int k = 0; k < 16; ++k) {
+            _Float16 x, y;
+            std::memcpy(&x, (const uint16_t *)w.a[(k / 8) * 32 + i] + k % 8, 2);
+            std::memcpy(&y, (const uint16_t *)w.b[(k / 8) * 32 + j] + k % 8, 2);
+            s += (double)(float)x * (double)(float)y;
+        }
+        d[r] = (float)((double)c[r] + s);
+    }
+    w.bar.wait();
+    return d;
+}
+typedef __fp16 f16x2 __attribute__((ext_vector_type(2)));
+// v_cvt_pkrtz_f16_f32: two floats as packed fp16, rounded toward zero (the kernels only pass values fp16 holds exactly)
+inline f16x2 cvt_pkrtz(float a, float b) {
+    auto rtz = [](float f) { _Float16 h = (_Float16)f; if (std::fabs((float)h) > std::fabs(f)) { uint16_t u; std::memcpy(&u, &h, 2); --u; std::memcpy(&h, &u, 2); } return h; };
+    const _Float16 x = rtz(a), y = rtz(b);
+    f16x2 r;
+    std::memcpy(&r, &x, 2);
+    std::memcpy((char *)&r + 2, &y, 2);
+    return r;
+}
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 // v_cvt_pk_f32_fp8: bytes 0, 1 (hi = false) or 2, 3 (hi = true) of src as two floats
 inline f32x2 cvt_pk_f32_fp8(uint32_t src, bool hi) {
@@ -217,6 +250,7 @@ inline void launch(K kernel, dim3 grid, unsigned threads, size_t lds_bytes, cons
 #define __device__
 #define __forceinline__ inline
 #define __launch_bounds__(...)
+#define __align__(n) __attribute__((aligned(n)))
 #define threadIdx emu::tl_thread
 #define blockIdx emu::tl_block
 #define gridDim emu::tl_grid
@@ -242,6 +276,8 @@ static inline unsigned atomicAdd(unsigned *p, unsigned v) { return __atomic_fetc
 #define __float_as_uint(f) emu::float_as_uint(f)
 #define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) emu::mfma_32x32x16_bf16((a), (b), (c), (x), (y), (z))
 #define __builtin_amdgcn_cvt_pk_f32_fp8(s, h) emu::cvt_pk_f32_fp8((s), (h))
+#define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) emu::mfma_32x32x16_f16((a), (b), (c), (x), (y), (z))
+#define __builtin_amdgcn_cvt_pkrtz(a, b) emu::cvt_pkrtz((a), (b))
 #define __builtin_amdgcn_cvt_off_f32_i4(x) emu::cvt_off_f32_i4(x)
 #define __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(s, f, h) emu::cvt_scalef32_pk_bf16_fp8((s), (f), (h))
 #define PF_REG_CONST_S(var, lit) var = lit

@@ -124,6 +124,10 @@ def emulator(tmp_path_factory):
     for k in ("void k_head_argmax(", "void k_head_topk(", "void k_head_block_stats(", "void k_softcap_copy(", "void k_bd_block_stats("):
         assert k in heads, k
     (build / "kernels_heads.inc").write_text(heads)
+    # the tiled prefill GEMM with its helpers
+    tiled = text[text.index("struct PfGemm {"):text.index("#define PF_DL_BM 128")]
+    assert "void k_pf_gemm(PfGemm g)" in tiled
+    (build / "kernel_tiled.inc").write_text(tiled)
     oracle_o = build / "oracle.o"
     r = subprocess.run([cxx.replace("clang++", "clang"), "-O1", "-w", "-c", os.path.join(ROOT, "oracle", "rustane_oracle.c"), "-o", str(oracle_o)],
                        capture_output=True, text=True)
@@ -133,7 +137,7 @@ def emulator(tmp_path_factory):
                 ("gemv", ["-Wno-psabi"]), ("convert_rows", [str(oracle_o), "-lm"]),
                 ("sample_topk", ["-ffp-contract=off", "-Wno-psabi", str(oracle_o), "-lm"]),
                 ("sample_fullvocab", ["-ffp-contract=off", "-Wno-psabi", str(oracle_o), "-lm"]),
-                ("single_row_heads", ["-ffp-contract=off", "-Wno-psabi", str(oracle_o), "-lm"]), ("few_row_i4", []),
+                ("single_row_heads", ["-ffp-contract=off", "-Wno-psabi", str(oracle_o), "-lm"]), ("tiled_gemm", ["-Wno-psabi"]), ("few_row_i4", []),
                 ("few_row_f8", ["-DEMU_F8_WAVES=8", "-DEMU_F8_KERNEL(RT,PACK)=k_pf_gemm_skinny_f8<RT,PACK,8>"]), ("few_row_general", ["-Wno-psabi"]))
 
     def compile_one(item):
@@ -292,3 +296,28 @@ def test_single_row_head_kernels_source_on_the_cpu(emulator):
     r = subprocess.run([emulator["single_row_heads"]], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
     assert r.stdout.count("0 mismatches") == 4
+
+
+# the tiled prefill GEMM: 33 rows up, two row tiles, ragged n, a reduction that ends inside a 64-element step
+CASES_TILED = [(100, 200, 512, 256), (40, 130, 384, 4), (150, 257, 640, 256), (33, 64, 416, 256), (130, 140, 288, 256)]
+
+
+@pytest.mark.parametrize("wd", [WeightDtype.BF16, WeightDtype.FP8_E4M3, WeightDtype.INT4_G128])
+def test_tiled_prefill_gemm_kernel_source_on_the_cpu(emulator, wd):
+    # k_pf_gemm for bf16, e4m3 and 4-bit weights with the three activation formats (bf16 pair, bf16 hi part, fp16)
+    # under the library's plans against an fp64 product of the stored operands
+    ran = 0
+    for rows, n, k, num_cu in CASES_TILED:
+        if wd == WeightDtype.INT4_G128 and k % 128:
+            continue
+        p = hipdec.gemm_plan(wd, rows, n, k, num_cu)
+        if wd == WeightDtype.BF16 and rows >= 129 and k % 64 == 0:
+            assert p["kernel"] == "tiled_direct_lds"       # (that kernel's loads write LDS directly: not emulated)
+            continue
+        assert p["kernel"] == "tiled" and p["threads"] == 256 and p["lds_bytes"] == 0, p
+        for act in (0, 1, 2):
+            args = [int(wd), act, rows, n, k, p["steps_per_split"], *p["grid"], rows + act]
+            r = subprocess.run([emulator["tiled_gemm"]] + [str(a) for a in args], capture_output=True, text=True, timeout=600)
+            assert r.returncode == 0 and "not written 0" in r.stdout, (wd, act, p, r.stdout, r.stderr[-3000:])
+            ran += 1
+    assert ran >= 6
