@@ -226,11 +226,12 @@ def test_general_few_row_kernel_source_on_the_cpu(emulator, general_plans):
 
 
 def test_element_wise_kernels_source_on_the_cpu(emulator):
-    # k_pf_resid, k_pf_gate_epi, k_bd_qkv_epi (both cache formats) and k_bd_sum_planes against fp64 restatements, with
+    # k_pf_embed, k_pf_qkv_epi, k_pf_resid, k_pf_gate_epi, k_bd_qkv_epi (both cache formats) and k_bd_sum_planes against fp64 restatements, with
     # split counts on both sides of the plane sums' request rounds of four and eight
     r = subprocess.run([emulator["epilogues"]], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0 and "0 checks failed" in r.stdout, (r.stdout[-4000:], r.stderr[-3000:])
     assert r.stdout.count("k_pf_resid") >= 11 and r.stdout.count("k_bd_qkv_epi") >= 6
+    assert r.stdout.count("k_pf_embed<") == 2 and r.stdout.count("k_pf_qkv_epi<") == 6
 
 
 def test_multi_row_attention_kernel_source_on_the_cpu(emulator):
